@@ -1,0 +1,230 @@
+"""ctypes/numpy front end of the CPU oracle (``bsi_oracle.c``).
+
+TEST INFRASTRUCTURE ONLY: imported by ``tests/``, by the smoke check and by the CPU-baseline
+leg of the benchmark, never by the library.  Each function forwards to the C restatement of
+the reference block named in its docstring (paths relative to the reference's
+``bsi_ops/csrc/cuda/``).
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "libbsi_oracle.so")
+
+_i64p = np.ctypeslib.ndpointer(np.int64, flags="C_CONTIGUOUS")
+_u64p = np.ctypeslib.ndpointer(np.uint64, flags="C_CONTIGUOUS")
+_i32p = np.ctypeslib.ndpointer(np.int32, flags="C_CONTIGUOUS")
+_f32p = np.ctypeslib.ndpointer(np.float32, flags="C_CONTIGUOUS")
+
+
+def build(force: bool = False) -> str:
+    """Compile the oracle with gcc (``make -C oracle``)."""
+    if force and os.path.exists(_SO):
+        os.remove(_SO)
+    subprocess.run(["make", "-C", _HERE], check=True, stdout=subprocess.DEVNULL)
+    return _SO
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_SO):
+        build()
+    L = ctypes.CDLL(_SO)
+    L.bsi_oracle_round_half_away.restype = ctypes.c_int64
+    L.bsi_oracle_round_half_away.argtypes = [ctypes.c_double]
+    L.bsi_oracle_round_to_int64.restype = None
+    L.bsi_oracle_round_to_int64.argtypes = [_f32p, ctypes.c_int64, ctypes.c_int, _i64p]
+    L.bsi_oracle_compute_shift.restype = ctypes.c_int
+    L.bsi_oracle_compute_shift.argtypes = [ctypes.c_uint64, ctypes.c_double, ctypes.c_int, ctypes.c_int, ctypes.c_float]
+    L.bsi_oracle_shift_clamp.restype = ctypes.c_int64
+    L.bsi_oracle_shift_clamp.argtypes = [ctypes.c_int64, ctypes.c_int, ctypes.c_int]
+    L.bsi_oracle_quantize_fixed.restype = None
+    L.bsi_oracle_quantize_fixed.argtypes = [_f32p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+                                            ctypes.c_int, ctypes.c_float, _i64p, _i32p, _f32p]
+    L.bsi_oracle_pack.restype = None
+    L.bsi_oracle_pack.argtypes = [_i64p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_int64, _u64p]
+    L.bsi_oracle_slice_weights.restype = None
+    L.bsi_oracle_slice_weights.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, _f32p]
+    L.bsi_oracle_compress_flags.restype = None
+    L.bsi_oracle_compress_flags.argtypes = [_u64p, ctypes.c_int, ctypes.c_int, ctypes.c_double, _i32p]
+    L.bsi_oracle_ewah_size.restype = None
+    L.bsi_oracle_ewah_size.argtypes = [_u64p, ctypes.c_int, ctypes.c_int, _i32p, _u64p]
+    L.bsi_oracle_ewah_emit.restype = None
+    L.bsi_oracle_ewah_emit.argtypes = [_u64p, ctypes.c_int, ctypes.c_int, _i32p, _u64p, _u64p, _i32p]
+    L.bsi_oracle_ewah_decompress.restype = None
+    L.bsi_oracle_ewah_decompress.argtypes = [_u64p, ctypes.c_int, ctypes.c_int, _u64p]
+    L.bsi_oracle_dot_fixed.restype = None
+    L.bsi_oracle_dot_fixed.argtypes = [_u64p, _f32p, ctypes.c_int64, ctypes.c_int, ctypes.c_int, _u64p, _f32p,
+                                       ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.c_float, ctypes.c_int64,
+                                       ctypes.c_void_p, ctypes.c_void_p]
+    L.bsi_oracle_num_threads.restype = ctypes.c_int
+    L.bsi_oracle_num_threads.argtypes = []
+    _lib = L
+    return L
+
+
+def num_threads() -> int:
+    return int(lib().bsi_oracle_num_threads())
+
+
+def round_half_away(x: float) -> int:
+    """bsi_cuda_kernels_quant.cuh:24-29."""
+    return int(lib().bsi_oracle_round_half_away(float(x)))
+
+
+def round_to_int64(x: np.ndarray, decimal_places: int) -> np.ndarray:
+    """bsi_cuda_kernels_quant.cuh:110-121."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty(x.shape, dtype=np.int64)
+    lib().bsi_oracle_round_to_int64(x.reshape(-1), x.size, int(decimal_places), out.reshape(-1))
+    return out
+
+
+def compute_shift(max_abs: int, sum_abs: float, count: int, fixed_bits: int, clip_k: float = 0.0) -> int:
+    """bsi_cuda_kernels_quant.cuh:82-108."""
+    return int(lib().bsi_oracle_compute_shift(int(max_abs), float(sum_abs), int(count), int(fixed_bits), float(clip_k)))
+
+
+def shift_clamp(v: int, shift: int, fixed_bits: int) -> int:
+    """bsi_cuda_kernels_quant.cuh:205-226."""
+    return int(lib().bsi_oracle_shift_clamp(int(v), int(shift), int(fixed_bits)))
+
+
+def quantize_fixed(x: np.ndarray, decimal_places: int, fixed_bits: int, chunk_scale: bool, clip_k: float = 0.0):
+    """Fixed-bit quantiser, bsi_cuda_kernels_quant.cuh:255-488.
+
+    Returns ``(ints[Q,d] int64, shifts int32, scales float32)``; shifts/scales are
+    ``[Q, ceil(d/256)]`` with ``chunk_scale`` and ``[Q]`` without.
+    """
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    Q, d = x.shape
+    chunks = (d + 255) // 256 if chunk_scale else 1
+    ints = np.zeros((Q, d), dtype=np.int64)
+    shifts = np.zeros((Q, chunks), dtype=np.int32)
+    scales = np.ones((Q, chunks), dtype=np.float32)
+    if Q and d:
+        lib().bsi_oracle_quantize_fixed(x.reshape(-1), Q, d, int(decimal_places), int(fixed_bits), int(bool(chunk_scale)),
+                                        float(clip_k), ints.reshape(-1), shifts.reshape(-1), scales.reshape(-1))
+    if not chunk_scale:
+        shifts, scales = shifts[:, 0].copy(), scales[:, 0].copy()
+    return ints, shifts, scales
+
+
+def pack(ints: np.ndarray, slices: int) -> np.ndarray:
+    """bsi_cuda_kernels_pack.cuh:129-174 -> words ``[Q, slices, W64]`` uint64."""
+    ints = np.ascontiguousarray(ints, dtype=np.int64)
+    Q, d = ints.shape
+    W = (d + 63) // 64 if d > 0 else 1
+    words = np.zeros((Q, slices, W), dtype=np.uint64)
+    if Q and d:
+        lib().bsi_oracle_pack(ints.reshape(-1), Q, d, int(slices), W, words.reshape(-1))
+    return words
+
+
+def slice_weights(S: int, offset: int = 0, twos: bool = True) -> np.ndarray:
+    """bsi_cuda.cpp:217-236."""
+    out = np.zeros(S, dtype=np.float32)
+    lib().bsi_oracle_slice_weights(int(S), int(offset), int(bool(twos)), out)
+    return out
+
+
+def compress_flags(words: np.ndarray, threshold: float) -> np.ndarray:
+    """bsi_cuda_kernels_ewah.cuh:47-69,84-102; ``words`` is ``[S, W]``."""
+    words = np.ascontiguousarray(words, dtype=np.uint64)
+    S, W = words.shape
+    flags = np.zeros(S, dtype=np.int32)
+    lib().bsi_oracle_compress_flags(words.reshape(-1), S, W, float(threshold), flags)
+    return flags
+
+
+def ewah_encode(words: np.ndarray, flags: np.ndarray):
+    """bsi_cuda_kernels_ewah.cuh:118-232 -> ``(stream uint64[total], off int64[S], len int32[S])``."""
+    words = np.ascontiguousarray(words, dtype=np.uint64)
+    flags = np.ascontiguousarray(flags, dtype=np.int32)
+    S, W = words.shape
+    sizes = np.zeros(S, dtype=np.uint64)
+    lib().bsi_oracle_ewah_size(words.reshape(-1), S, W, flags, sizes)
+    off = np.zeros(S, dtype=np.uint64)
+    off[1:] = np.cumsum(sizes)[:-1]
+    total = int(sizes.sum())
+    out = np.zeros(max(total, 1), dtype=np.uint64)
+    lens = np.zeros(S, dtype=np.int32)
+    lib().bsi_oracle_ewah_emit(words.reshape(-1), S, W, flags, off, out, lens)
+    assert (lens.astype(np.uint64) == sizes).all(), "size pass and emit pass disagree"
+    return out[:total], off.astype(np.int64), lens
+
+
+def ewah_decompress(stream: np.ndarray, W: int) -> np.ndarray:
+    """bsi_cuda_kernels_ewah.cuh:5-33."""
+    stream = np.ascontiguousarray(stream, dtype=np.uint64)
+    out = np.zeros(W, dtype=np.uint64)
+    buf = stream if stream.size else np.zeros(1, dtype=np.uint64)
+    lib().bsi_oracle_ewah_decompress(buf, int(stream.size), int(W), out)
+    return out
+
+
+def dot_fixed(A: np.ndarray, qscale: np.ndarray, B: np.ndarray, bscale: np.ndarray, scale_inv: float,
+              want_ints: bool = True, want_out: bool = True):
+    """bsi_cuda_kernels_dot.cuh:1384-1542.
+
+    ``A`` ``[Q,Sa,W]`` uint64, ``qscale`` ``[Q,chunks]`` or ``[Q]`` (row scale, broadcast over chunks),
+    ``B`` ``[R,Sb,W]``, ``bscale`` ``[R]``.  Returns ``(chunk_ints int32 [Q,R,chunks] | None, out f32 [Q,R] | None)``.
+    """
+    A = np.ascontiguousarray(A, dtype=np.uint64)
+    B = np.ascontiguousarray(B, dtype=np.uint64)
+    Q, Sa, W = A.shape
+    R, Sb, Wb = B.shape
+    assert W == Wb
+    chunks = (W + 3) // 4
+    qscale = np.asarray(qscale, dtype=np.float32)
+    if qscale.ndim == 1:
+        qscale = np.repeat(qscale[:, None], chunks, axis=1)
+    qscale = np.ascontiguousarray(qscale)
+    assert qscale.shape == (Q, chunks), (qscale.shape, (Q, chunks))
+    bscale = np.ascontiguousarray(bscale, dtype=np.float32)
+    assert bscale.shape == (R,)
+    ints = np.zeros((Q, R, chunks), dtype=np.int32) if want_ints else None
+    out = np.zeros((Q, R), dtype=np.float32) if want_out else None
+    lib().bsi_oracle_dot_fixed(A.reshape(-1), qscale.reshape(-1), chunks, Sa, W, B.reshape(-1), bscale, Sb, R, Q,
+                               ctypes.c_float(scale_inv), R,
+                               ints.ctypes.data if ints is not None else None,
+                               out.ctypes.data if out is not None else None)
+    return ints, out
+
+
+def scale_inv(dec_q: int, dec_k: int) -> np.float32:
+    """bsi_cuda.cpp:709-711: ``(float)(1 / 10^(dec_q + dec_k))``."""
+    total = int(dec_q) + int(dec_k)
+    return np.float32(1.0 / (10.0 ** total)) if total > 0 else np.float32(1.0)
+
+
+def build_queries(x: np.ndarray, decimal_places: int = 2, fixed_bits: int = 7, clip_k: float = 0.0):
+    """Query side of bsi_vector_cuda.cpp:971-1064: chunk scales iff ``W64 % 4 == 0``.
+
+    Returns dict(words, ints, shifts, scales, chunk_scale, slice_weights).
+    """
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    d = x.shape[1]
+    W = (d + 63) // 64 if d > 0 else 1
+    chunk = (W % 4) == 0
+    ints, shifts, scales = quantize_fixed(x, decimal_places, fixed_bits, chunk, clip_k)
+    return dict(words=pack(ints, fixed_bits), ints=ints, shifts=shifts, scales=scales, chunk_scale=chunk,
+                slice_weights=slice_weights(fixed_bits))
+
+
+def build_keys(k: np.ndarray, decimal_places: int = 2, fixed_bits: int = 6, clip_k: float = 0.0):
+    """Key side of bsi_vector_cuda.cpp:971-1197 (``for_keys``): per-row scale, ``Bw[r,j] = w_j * 2^shift_r``."""
+    k = np.ascontiguousarray(k, dtype=np.float32)
+    ints, shifts, scales = quantize_fixed(k, decimal_places, fixed_bits, False, clip_k)
+    bw = slice_weights(fixed_bits)[None, :] * scales[:, None]
+    return dict(words=pack(ints, fixed_bits), ints=ints, shifts=shifts, scales=scales, slice_weights=bw.astype(np.float32))
