@@ -1,0 +1,625 @@
+"""Python mirror of the reference ``bsi_ops`` extension module for the GPU tensor-dot path.
+
+Same function names, argument meaning, return tuples and error behaviour as the pybind module the
+reference registers in ``bsi_ops/csrc/cuda/bsi_cuda.cpp:1010-1078`` (and the module shell in
+``bsi_ops/bsiFunctions.cpp:810-847``), so the reference's microbenchmarks and its
+``BSIQuantizedLinear`` call it unchanged (``import bsipytorch_amd.bsi_ops as bsi_ops`` or the
+top-level ``bsi_ops`` shim).  Handles are opaque objects with the reference's capsule names; they
+own torch tensors, so device memory is released when the handle is garbage collected.
+
+Every function forwards to ``libbsi_hip.so`` through its C ABI; torch is used for device memory
+and the current stream only.  Fixed-bit mode (queries 7 bits with per-256-element chunk scales,
+keys 6 bits with a per-row scale) is the default; the reference's environment names override it:
+``BSI_FIXED_BITS``, ``BSI_FIXED_BITS_QUERIES``, ``BSI_FIXED_BITS_KEYS``, ``BSI_FIXED_CHUNK_SCALE``,
+``BSI_FIXED_CLIP_K``, ``BSI_PROFILE``, ``BSI_DEBUG``, ``BSI_DOT_DEBUG``.  Flags that select NVIDIA
+code paths (``BSI_TC_DOT``, ``BSI_TC_TMA``, ``BSI_TC_CPASYNC``, ``BSI_TC_R_SWEEP``,
+``BSI_TC_FIXED_INT``, ``BSI_CUSTOM_QUANT``, ``BSI_FUSED_QPACK``, ``BSI_PACK_ONESHOT``, ``BSI_Q_TILE``,
+``BSI_R_TILE``) are accepted and ignored.  Two flags are new: ``BSI_DOT_CORE`` = ``auto`` | ``mfma`` |
+``valu`` and ``BSI_KEY_LAYOUT`` = ``tiled`` | ``canonical``.
+"""
+from __future__ import annotations
+
+import os
+import sys
+from typing import List, Optional
+
+import torch
+
+from . import _lib
+from ._lib import check, lib
+
+# --------------------------------------------------------------------------- flags
+
+
+def _env_int(name: str, default: Optional[int]) -> Optional[int]:
+    s = os.environ.get(name)
+    if s is None:
+        return default
+    try:
+        return int(s)
+    except ValueError:
+        return 0  # atoi semantics
+
+
+def _clamp_bits(v: int) -> int:
+    # bsi_vector_cuda.cpp:254-276: <= 0 disables, otherwise clamp to [2, 63]
+    if v <= 0:
+        return 0
+    return min(63, max(2, v))
+
+
+_flag_cache: dict = {}
+
+
+def _flags() -> dict:
+    """Environment flags, read once per process like the reference's function-local statics."""
+    if _flag_cache:
+        return _flag_cache
+    base = _env_int("BSI_FIXED_BITS", None)
+    q = _env_int("BSI_FIXED_BITS_QUERIES", None)
+    k = _env_int("BSI_FIXED_BITS_KEYS", None)
+    # default (nothing set): fixed76 chunk-scale
+    bits_q = _clamp_bits(q if q is not None else (base if base is not None else 7))
+    bits_k = _clamp_bits(k if k is not None else (base if base is not None else 6))
+    clip = 0.0
+    try:
+        clip = float(os.environ.get("BSI_FIXED_CLIP_K", "0") or 0)
+    except ValueError:
+        clip = 0.0
+    core = os.environ.get("BSI_DOT_CORE", "auto").strip().lower()
+    layout = os.environ.get("BSI_KEY_LAYOUT", "tiled").strip().lower()
+    _flag_cache.update(
+        bits_q=bits_q,
+        bits_k=bits_k,
+        chunk_scale=(_env_int("BSI_FIXED_CHUNK_SCALE", 1) or 0) != 0,
+        clip_k=clip if clip > 0.0 else 0.0,
+        profile=(_env_int("BSI_PROFILE", 0) or 0) != 0,
+        debug=os.environ.get("BSI_DEBUG") is not None,
+        dot_debug=(_env_int("BSI_DOT_DEBUG", 0) or 0) != 0,
+        core={"auto": _lib.CORE_AUTO, "valu": _lib.CORE_VALU, "mfma": _lib.CORE_MFMA}.get(core, _lib.CORE_AUTO),
+        tiled=(layout != "canonical"),
+    )
+    return _flag_cache
+
+
+def _reset_flag_cache() -> None:
+    """Test hook: re-read the environment on the next call."""
+    _flag_cache.clear()
+    _DOT_DEBUG_PRINTED[0] = False
+
+
+def _check(cond: bool, msg: str) -> None:
+    # TORCH_CHECK surfaces as RuntimeError in Python
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _device() -> torch.device:
+    _check(torch.cuda.is_available(), "bsi_ops: no GPU visible; the HIP path is the only path")
+    return torch.device("cuda", torch.cuda.current_device())
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    return {torch.float32: _lib.DTYPE_F32, torch.float16: _lib.DTYPE_F16, torch.bfloat16: _lib.DTYPE_BF16}[t.dtype]
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+# --------------------------------------------------------------------------- handles
+
+
+class _Capsule:
+    """Opaque handle; ``name`` is the reference's PyCapsule name."""
+
+    name = ""
+
+    def __repr__(self) -> str:  # pragma: no cover - cosmetic
+        return f'<capsule object "{self.name}" at {hex(id(self))}>'
+
+
+class PrebuiltBSIKeysCUDA(_Capsule):
+    """bsi_cuda.cpp:153-177 (single Sb group, identity key order)."""
+
+    name = "PrebuiltBSIKeysCUDA"
+
+    def __init__(self):
+        self.words: torch.Tensor = None          # canonical [R, Sb, W] or tiled [ceil(R/16), chunks, Sb, 64]
+        self.layout = _lib.LAYOUT_CANONICAL
+        self.slice_weights: torch.Tensor = None  # [R, Sb] float32
+        self.shifts: torch.Tensor = None         # [R] int32
+        self.Sb = 0
+        self.W = 0
+        self.d = 0
+        self.num_keys = 0
+        self.decimals = 0
+        self.threshold = 0.2
+
+
+class PrebuiltBSIQueryBatchCUDA(_Capsule):
+    """bsi_cuda.cpp:202-211."""
+
+    name = "PrebuiltBSIQueryBatchCUDA"
+
+    def __init__(self):
+        self.words: torch.Tensor = None          # [Q, Sa, W] int64
+        self.slice_weights: torch.Tensor = None  # [Q, Sa] float32
+        self.chunk_scales: Optional[torch.Tensor] = None  # [Q, chunks] float32 or None
+        self.row_scales: Optional[torch.Tensor] = None    # [Q] float32 when there are no chunk scales
+        self.ints8: Optional[torch.Tensor] = None         # [Q, chunks*256] int8 (MFMA operand) or None
+        self.Sa = 0
+        self.W = 0
+        self.decimals = 0
+        self.Q = 0
+        self.mem_bytes = 0
+
+
+class PrebuiltBSIQueryCUDA(_Capsule):
+    """bsi_cuda.cpp:183-192: one query row (a view into its batch)."""
+
+    name = "PrebuiltBSIQueryCUDA"
+
+    def __init__(self):
+        self.dev_words: torch.Tensor = None      # [S, W]
+        self.slice_weights: torch.Tensor = None  # [S]
+        self.chunk_scales: Optional[torch.Tensor] = None  # [chunks]
+        self.row_scale: Optional[torch.Tensor] = None     # [] when no chunk scales
+        self.ints8: Optional[torch.Tensor] = None         # [chunks*256]
+        self.S = 0
+        self.W = 0
+        self.rows = 0
+        self.decimals = 0
+        self.twos_complement = False
+        self.mem_bytes = 0
+        # hybrid builder only
+        self.comp_words: Optional[torch.Tensor] = None
+        self.comp_off: Optional[torch.Tensor] = None
+        self.comp_len: Optional[torch.Tensor] = None
+
+
+def _capsule(obj, cls, what: str):
+    _check(isinstance(obj, cls), what)
+    return obj
+
+
+# --------------------------------------------------------------------------- builder
+
+_last_build_profile = [0, 0, 0]
+
+
+def get_last_query_build_profile_cuda():
+    """(quantize_ns, pack_ns, total_ns) of the last query-batch build; zeros unless BSI_PROFILE=1
+    (bsi_cuda.cpp:1036-1041).  The chunk-scale build is one fused kernel here, reported as pack_ns."""
+    return tuple(_last_build_profile)
+
+
+def reset_last_query_build_profile_cuda() -> None:
+    _last_build_profile[:] = [0, 0, 0]
+
+
+def cuda_builder_version() -> str:
+    return "HIP_BUILDER_GFX950_FIXED76 " + _lib.version()
+
+
+CUDA_BUILDER_VERSION = cuda_builder_version()
+
+
+def _slice_weights(S: int, offset: int, twos: bool, device) -> torch.Tensor:
+    # bsi_cuda.cpp:217-236
+    w = [float(2.0 ** (offset + i)) if offset + i >= 0 else 0.0 for i in range(S)]
+    if twos and S > 0:
+        w[S - 1] = -w[S - 1]
+    return torch.tensor(w, dtype=torch.float32, device=device)
+
+
+def _as_build_input(x: torch.Tensor, device) -> torch.Tensor:
+    x = x.detach()
+    if x.device != device:
+        x = x.to(device)
+    if x.dtype not in (torch.float32, torch.float16, torch.bfloat16):
+        x = x.to(torch.float32)
+    return x.contiguous()
+
+
+def _build_fixed(x2d: torch.Tensor, decimal_places: int, fixed_bits: int, chunk_scale: bool, want_ints8: bool):
+    """One call of bsi_hip_build_fixed -> (words [Q,S,W] int64, shifts, scales, ints8 | None)."""
+    f = _flags()
+    dev = x2d.device
+    Q, d = x2d.shape
+    W = (d + 63) // 64 if d > 0 else 1
+    chunks = (d + 255) // 256 if d > 0 else 0
+    words = torch.zeros((Q, fixed_bits, W), dtype=torch.int64, device=dev)
+    if chunk_scale:
+        shifts = torch.zeros((Q, chunks), dtype=torch.int32, device=dev)
+        scales = torch.ones((Q, chunks), dtype=torch.float32, device=dev)
+    else:
+        shifts = torch.zeros((Q,), dtype=torch.int32, device=dev)
+        scales = torch.ones((Q,), dtype=torch.float32, device=dev)
+    ints8 = None
+    if want_ints8 and fixed_bits <= 8 and Q > 0 and d > 0:
+        ints8 = torch.empty((Q, ((W + 3) // 4) * 256), dtype=torch.int8, device=dev)
+    if Q > 0 and d > 0:
+        check(lib.bsi_hip_build_fixed(x2d.data_ptr(), _dtype_code(x2d), Q, d, int(decimal_places), fixed_bits,
+                                      1 if chunk_scale else 0, f["clip_k"], words.data_ptr(), shifts.data_ptr(),
+                                      scales.data_ptr(), _ptr(ints8), _stream()), "bsi_hip_build_fixed")
+    return words, shifts, scales, ints8
+
+
+def _require_fixed(bits: int, what: str) -> None:
+    _check(bits > 0, f"{what}: BSI_FIXED_BITS*=0 selects the decimal (data-dependent slice count) builder, "
+                     "which this build does not implement; unset it to use the fixed-bit path")
+
+
+def _build_query_batch(q2d: torch.Tensor, decimal_places: int) -> PrebuiltBSIQueryBatchCUDA:
+    """bsi_vector_cuda.cpp:971-1064 (queries): chunk scales iff the flag is on and W64 % 4 == 0."""
+    f = _flags()
+    _require_fixed(f["bits_q"], "build_bsi_queries")
+    dev = _device()
+    x = _as_build_input(q2d, dev)
+    Q, d = x.shape
+    W = (d + 63) // 64 if d > 0 else 1
+    chunk_scale = f["chunk_scale"] and (W % 4 == 0)
+    prof = f["profile"]
+    if prof:
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+    words, _shifts, scales, ints8 = _build_fixed(x, decimal_places, f["bits_q"], chunk_scale, want_ints8=True)
+    if prof:
+        e1.record()
+        e1.synchronize()
+        ns = int(e0.elapsed_time(e1) * 1.0e6)
+        _last_build_profile[:] = [0, ns, ns]
+    else:
+        _last_build_profile[:] = [0, 0, 0]
+    h = PrebuiltBSIQueryBatchCUDA()
+    base = _slice_weights(f["bits_q"], 0, True, dev)
+    h.words = words
+    if chunk_scale:
+        h.slice_weights = base.unsqueeze(0).expand(Q, -1).contiguous()
+        h.chunk_scales = scales
+    else:
+        h.slice_weights = (base.unsqueeze(0) * scales.unsqueeze(1)).contiguous()
+        h.row_scales = scales
+    h.ints8 = ints8
+    h.Sa = f["bits_q"]
+    h.W = W
+    h.decimals = int(decimal_places)
+    h.Q = Q
+    h.mem_bytes = words.numel() * 8 + h.slice_weights.numel() * 4
+    if h.chunk_scales is not None and h.chunk_scales.numel() > 0:
+        h.mem_bytes += h.chunk_scales.numel() * 4
+    if f["debug"]:
+        print(f"[BSI_HIP] build_bsi_queries_cuda_batch_data (fused): Q={Q} slices={h.Sa} words_per_slice={W}")
+    return h
+
+
+def build_bsi_queries_cuda_batch_packed(q2d: torch.Tensor, decimal_places: int, compress_threshold: float = 0.2):
+    """bsi_cuda.cpp:346-379.  ``compress_threshold`` is accepted and unused, as in the reference."""
+    _check(q2d.dim() == 2, "q must be 2D [Q, d]")
+    return _build_query_batch(q2d, int(decimal_places))
+
+
+def build_bsi_queries_cuda_batch(q2d: torch.Tensor, decimal_places: int, compress_threshold: float = 0.2) -> List:
+    """bsi_cuda.cpp:272-344: one handle per row, all views into one batch build."""
+    _check(q2d.dim() == 2, "q must be 2D [Q, d]")
+    b = _build_query_batch(q2d, int(decimal_places))
+    out = []
+    for qi in range(b.Q):
+        h = PrebuiltBSIQueryCUDA()
+        h.S, h.W = b.Sa, b.W
+        h.dev_words = b.words[qi]
+        h.slice_weights = b.slice_weights[qi]
+        if b.chunk_scales is not None and b.chunk_scales.numel() > 0:
+            h.chunk_scales = b.chunk_scales[qi]
+        else:
+            h.row_scale = b.row_scales[qi]
+        h.ints8 = b.ints8[qi] if b.ints8 is not None else None
+        h.mem_bytes = h.dev_words.numel() * 8
+        h.rows = int(q2d.shape[1])
+        h.decimals = int(decimal_places)
+        h.twos_complement = False  # as the reference leaves it (bsi_cuda.cpp:303)
+        out.append(h)
+    return out
+
+
+def _build_query_1d(q: torch.Tensor, decimal_places: int) -> PrebuiltBSIQueryCUDA:
+    """bsi_vector_cuda.cpp:778-852 with fixed bits: one scale for the whole vector."""
+    f = _flags()
+    _require_fixed(f["bits_q"], "build_bsi_query_cuda")
+    dev = _device()
+    x = _as_build_input(q, dev).view(1, -1)
+    words, _shifts, scales, ints8 = _build_fixed(x, decimal_places, f["bits_q"], False, want_ints8=True)
+    h = PrebuiltBSIQueryCUDA()
+    h.S = f["bits_q"]
+    h.W = words.shape[2]
+    h.dev_words = words[0]
+    h.rows = x.shape[1]
+    h.decimals = int(decimal_places)
+    # two's complement only when a negative value is present (bsi_vector_cuda.cpp:843); the top
+    # plane is empty otherwise, so the sign of its weight never matters
+    h.twos_complement = bool((h.dev_words[h.S - 1] != 0).any().item()) if x.shape[1] > 0 else False
+    h.slice_weights = _slice_weights(h.S, 0, h.twos_complement, dev) * scales[0]
+    h.row_scale = scales[0]
+    h.ints8 = ints8[0] if ints8 is not None else None
+    h.mem_bytes = h.dev_words.numel() * 8
+    return h
+
+
+def build_bsi_query_cuda(q: torch.Tensor, decimal_places: int, compress_threshold: float = 0.2):
+    """bsi_cuda.cpp:238-270 -> (handle, mem_bytes, S, W)."""
+    _check(q.dim() == 1, "q must be 1D [d]")
+    h = _build_query_1d(q, int(decimal_places))
+    return h, int(h.mem_bytes), h.S, h.W
+
+
+def ewah_compress_slices(words2d: torch.Tensor, compress_threshold: float):
+    """Density flags + size pass + exclusive scan + emit pass for ``[S, W]`` words
+    (bsi_vector_cuda.cpp:896-951).  Returns (comp_words, comp_off int64 [S], comp_len int32 [S], flags)."""
+    S, W = words2d.shape
+    dev = words2d.device
+    st = _stream()
+    counts = torch.empty((S,), dtype=torch.int64, device=dev)
+    flags = torch.empty((S,), dtype=torch.int32, device=dev)
+    sizes = torch.empty((S,), dtype=torch.int64, device=dev)
+    check(lib.bsi_hip_slice_popcount_sum(words2d.data_ptr(), S, W, counts.data_ptr(), st), "bsi_hip_slice_popcount_sum")
+    check(lib.bsi_hip_compress_flags_from_density(counts.data_ptr(), S, W, float(compress_threshold),
+                                                  flags.data_ptr(), st), "bsi_hip_compress_flags_from_density")
+    check(lib.bsi_hip_ewah_size(words2d.data_ptr(), S, W, flags.data_ptr(), sizes.data_ptr(), st), "bsi_hip_ewah_size")
+    inclusive = sizes.cumsum(0)
+    total = int(inclusive[-1].item()) if S > 0 else 0
+    comp_off = (inclusive - sizes).contiguous()
+    comp_words = torch.empty((max(total, 1),), dtype=torch.int64, device=dev)
+    comp_len = torch.empty((S,), dtype=torch.int32, device=dev)
+    check(lib.bsi_hip_ewah_emit(words2d.data_ptr(), S, W, flags.data_ptr(), comp_off.data_ptr(),
+                                comp_words.data_ptr(), comp_len.data_ptr(), st), "bsi_hip_ewah_emit")
+    return comp_words[:total], comp_off, comp_len, flags
+
+
+def build_bsi_query_cuda_hybrid(q: torch.Tensor, decimal_places: int, compress_threshold: float = 0.2):
+    """bsi_cuda.cpp:386-431: build, EWAH-compress every slice, then decode the streams back into the
+    verbatim words the dot consumes.  mem_bytes counts both the stream and the words."""
+    _check(q.dim() == 1, "q must be 1D [d]")
+    h = _build_query_1d(q, int(decimal_places))
+    planes = h.dev_words.contiguous()
+    comp_words, comp_off, comp_len, _flags_dev = ewah_compress_slices(planes, float(compress_threshold))
+    decoded = torch.zeros_like(planes)
+    if comp_words.numel() > 0:
+        check(lib.bsi_hip_ewah_decompress_batch(comp_words.data_ptr(), comp_off.data_ptr(), comp_len.data_ptr(),
+                                                h.S, h.W, decoded.data_ptr(), _stream()),
+              "bsi_hip_ewah_decompress_batch")
+    else:
+        decoded.copy_(planes)
+    h.dev_words = decoded
+    h.comp_words, h.comp_off, h.comp_len = comp_words, comp_off, comp_len
+    h.mem_bytes = comp_words.numel() * 8 + decoded.numel() * 8
+    return h, int(h.mem_bytes), h.S, h.W
+
+
+def build_bsi_keys_cuda(K: torch.Tensor, decimal_places: int, compress_threshold: float = 0.2):
+    """bsi_cuda.cpp:863-910 (fixed-bit branch): per-row scale, Sb slices, ``Bw[r, j] = w_j * 2^shift_r``.
+    Returns (handle, total_bytes_of_words, num_keys, d, W)."""
+    _check(K.dim() == 2, "K must be 2D [num_keys, d]")
+    f = _flags()
+    _require_fixed(f["bits_k"], "build_bsi_keys_cuda")
+    dev = _device()
+    x = _as_build_input(K, dev)
+    R, d = x.shape
+    words, shifts, scales, _ = _build_fixed(x, int(decimal_places), f["bits_k"], False, want_ints8=False)
+    h = PrebuiltBSIKeysCUDA()
+    h.num_keys, h.d = int(R), int(d)
+    h.W = words.shape[2]
+    h.Sb = f["bits_k"]
+    h.decimals = int(decimal_places)
+    h.threshold = float(compress_threshold)
+    h.shifts = shifts
+    h.slice_weights = (_slice_weights(h.Sb, 0, True, dev).unsqueeze(0) * scales.unsqueeze(1)).contiguous()
+    total_bytes = words.numel() * 8
+    if f["tiled"] and R > 0:
+        chunks = (h.W + 3) // 4
+        tiled = torch.empty(((R + 15) // 16, chunks, h.Sb, 64), dtype=torch.int64, device=dev)
+        check(lib.bsi_hip_tile_key_planes(words.data_ptr(), R, h.Sb, h.W, tiled.data_ptr(), _stream()),
+              "bsi_hip_tile_key_planes")
+        h.words, h.layout = tiled, _lib.LAYOUT_TILED16
+    else:
+        h.words, h.layout = words, _lib.LAYOUT_CANONICAL
+    if f["debug"]:
+        print(f"[BSI_HIP] build_bsi_keys_cuda: R={R} slices={h.Sb} words_per_slice={h.W} layout={h.layout}")
+    return h, int(total_bytes), int(R), int(d), int(h.W)
+
+
+# --------------------------------------------------------------------------- dot
+
+_DOT_DEBUG_PRINTED = [False]
+_workspace: dict = {}
+
+
+def _get_workspace(nbytes: int, dev) -> Optional[torch.Tensor]:
+    if nbytes <= 0:
+        return None
+    ws = _workspace.get(dev)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty((nbytes,), dtype=torch.uint8, device=dev)
+        _workspace[dev] = ws
+    return ws
+
+
+def _scale_inv(dec_q: int, dec_k: int) -> float:
+    # bsi_cuda.cpp:709-711: (float)(1.0 / 10^(dq + dk)); the C ABI takes it as float
+    total = dec_q + dec_k
+    return (1.0 / (10.0 ** total)) if total > 0 else 1.0
+
+
+def _dot(words, ints8, scales, scale_stride, Sa, W, keys: PrebuiltBSIKeysCUDA, Q, decimals_q, chunk_ints=None, core=None):
+    f = _flags()
+    dev = words.device
+    R = keys.num_keys
+    out = torch.empty((Q, R), dtype=torch.float32, device=dev)
+    core = f["core"] if core is None else core
+    ws = None
+    ws_bytes = 0
+    if ints8 is None:
+        ws_bytes = int(lib.bsi_hip_dot_workspace_bytes(Q, W, core)) if (2 <= Sa <= 8 and 2 <= keys.Sb <= 8) else 0
+        ws = _get_workspace(ws_bytes, dev)
+    prof = f["profile"]
+    if prof:
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+    check(lib.bsi_hip_dot(words.data_ptr(), _ptr(ints8), scales.data_ptr(), scale_stride, Sa, W,
+                          keys.words.data_ptr(), keys.layout, keys.slice_weights.data_ptr(), keys.Sb, R, Q,
+                          _scale_inv(decimals_q, keys.decimals), R, out.data_ptr(), _ptr(chunk_ints), core,
+                          _ptr(ws), ws_bytes, _stream()), "bsi_hip_dot")
+    ns = 0
+    if prof:
+        e1.record()
+        e1.synchronize()
+        ns = int(e0.elapsed_time(e1) * 1.0e6)
+    if f["dot_debug"] and not _DOT_DEBUG_PRINTED[0]:
+        _DOT_DEBUG_PRINTED[0] = True
+        print(f"[BSI_DOT] core={core} Sa={Sa} Sb={keys.Sb} Q={Q} R={R} W64={W} chunks={(W + 3) // 4} "
+              f"layout={keys.layout} ints8={'yes' if ints8 is not None else 'no'}", file=sys.stderr)
+    return out, ns
+
+
+def _dot_result(out, ns, Q, R):
+    per_q = float(ns) / float(Q) if Q > 0 else 0.0
+    per_s = float(ns) / (float(Q) * float(R)) if (Q > 0 and R > 0) else 0.0
+    return out, int(ns), per_q, per_s
+
+
+def batch_dot_product_multiquery_cuda_batch_caps(query_batch_cap, keyset_cuda_cap):
+    """bsi_cuda.cpp:658-815 -> (out[Q, R] float32 on the device, dot_ns_total, ns_per_query, ns_per_scalar).
+    The times are zero unless BSI_PROFILE=1 (which synchronises), as in the reference."""
+    keys = _capsule(keyset_cuda_cap, PrebuiltBSIKeysCUDA, "Invalid CUDA keys capsule")
+    qb = _capsule(query_batch_cap, PrebuiltBSIQueryBatchCUDA, "Invalid CUDA query-batch capsule")
+    _check(qb.words is not None and qb.slice_weights is not None, "Query batch tensors are not defined")
+    _check(qb.words.is_cuda and qb.slice_weights.is_cuda, "Query batch tensors must be CUDA tensors")
+    _check(qb.words.dim() == 3, "Query batch words must be [Q, Sa, W]")
+    _check(qb.slice_weights.dim() == 2, "Query batch slice_weights must be [Q, Sa]")
+    Q, Sa, W = qb.words.shape
+    _check(Q > 0 and Sa > 0 and W > 0, "Empty query batch")
+    _check(W == keys.W, "Word count mismatch between query batch and keys")
+    _check(tuple(qb.slice_weights.shape) == (Q, Sa), f"slice_weights shape mismatch: expected [{Q}, {Sa}]")
+    R = keys.num_keys
+    _check(R > 0, "Empty keys")
+    if qb.chunk_scales is not None and qb.chunk_scales.numel() > 0:
+        _check(qb.chunk_scales.is_cuda, "chunk_scales must be a CUDA tensor")
+        _check(qb.chunk_scales.dim() == 2, "Expected [Q, chunks] chunk scales")
+        _check(qb.chunk_scales.shape[0] == Q, "chunk_scales Q mismatch")
+        _check(keys.W % 4 == 0, "Chunk scales require W64 multiple of 4")
+        _check(qb.chunk_scales.shape[1] == keys.W // 4,
+               f"Chunk scale stride mismatch: got {qb.chunk_scales.shape[1]} expected {keys.W // 4}")
+        scales, stride = qb.chunk_scales, int(qb.chunk_scales.shape[1])
+    else:
+        _check(qb.row_scales is not None, "Query batch has neither chunk scales nor row scales")
+        scales, stride = qb.row_scales, 1
+    _check(qb.decimals == keys.decimals,
+           f"Decimal mismatch between queries and keys: q={qb.decimals} k={keys.decimals}")
+    out, ns = _dot(qb.words, qb.ints8, scales, stride, int(Sa), int(W), keys, int(Q), qb.decimals)
+    return _dot_result(out, ns, Q, R)
+
+
+def batch_dot_product_multiquery_cuda_caps(query_caps_list, keyset_cuda_cap):
+    """bsi_cuda.cpp:433-656: list-of-row-handles form; rows are stacked, then the same dot runs."""
+    keys = _capsule(keyset_cuda_cap, PrebuiltBSIKeysCUDA, "Invalid CUDA keys capsule")
+    R = keys.num_keys
+    Q = len(query_caps_list)
+    _check(R > 0 and Q > 0, "Empty keys or queries")
+    rows = []
+    for qi, cap in enumerate(query_caps_list):
+        _check(isinstance(cap, _Capsule), "Each item must be a capsule")
+        q = _capsule(cap, PrebuiltBSIQueryCUDA, f"Invalid BSI query capsule at index {qi}")
+        _check(q.W == keys.W, "Word count mismatch between query and keys")
+        _check(q.decimals == rows[0].decimals if rows else True, "Decimal mismatch across queries not supported")
+        _check(q.S == rows[0].S if rows else True, "Mixed slice counts across queries are not supported in fixed-bit mode")
+        rows.append(q)
+    have_scales = rows[0].chunk_scales is not None and rows[0].chunk_scales.numel() > 0
+    for q in rows:
+        _check((q.chunk_scales is not None and q.chunk_scales.numel() > 0) == have_scales,
+               "Mixed chunk-scale and non-chunk-scale queries in the same group")
+    words = torch.stack([q.dev_words for q in rows]).contiguous()
+    if have_scales:
+        scales = torch.stack([q.chunk_scales for q in rows]).contiguous()
+        _check(keys.W % 4 == 0 and scales.shape[1] == keys.W // 4, "Chunk scale stride mismatch")
+        stride = int(scales.shape[1])
+    else:
+        scales = torch.stack([q.row_scale.reshape(()) for q in rows]).contiguous()
+        stride = 1
+    ints8 = torch.stack([q.ints8 for q in rows]).contiguous() if all(q.ints8 is not None for q in rows) else None
+    _check(rows[0].decimals == keys.decimals,
+           f"Decimal mismatch between queries and keys: q={rows[0].decimals} k={keys.decimals}")
+    out, ns = _dot(words, ints8, scales, stride, rows[0].S, keys.W, keys, Q, rows[0].decimals)
+    return _dot_result(out, ns, Q, R)
+
+
+def bsi_keys_cuda_stats(keyset_cuda_cap) -> dict:
+    """bsi_cuda.cpp:817-832."""
+    keys = _capsule(keyset_cuda_cap, PrebuiltBSIKeysCUDA, "Invalid CUDA keys capsule")
+    return {"W": keys.W, "d": keys.d, "num_keys": keys.num_keys, "decimals": keys.decimals,
+            "threshold": keys.threshold, "Sb_counts": {keys.Sb: keys.num_keys}}
+
+
+def bsi_query_caps_stats(query_caps_list) -> dict:
+    """bsi_cuda.cpp:834-861."""
+    Q = len(query_caps_list)
+    _check(Q > 0, "Empty query capsule list")
+    counts: dict = {}
+    W = -1
+    for qi, cap in enumerate(query_caps_list):
+        _check(isinstance(cap, _Capsule), "Each item must be a capsule")
+        q = _capsule(cap, PrebuiltBSIQueryCUDA, f"Invalid BSI query capsule at index {qi}")
+        counts[q.S] = counts.get(q.S, 0) + 1
+        if W < 0:
+            W = q.W
+        else:
+            _check(q.W == W, "Word count mismatch across queries")
+    return {"Q": Q, "W": W, "S_counts": counts}
+
+
+# --------------------------------------------------------------------------- parity / debug hooks
+
+
+def debug_chunk_ints(query_batch_cap, keyset_cuda_cap, core: str = "auto"):
+    """Integer accumulators I[q, r, c] (int32) and the fp32 output of one dot, for parity checks.
+    No counterpart in the reference (its accumulators never leave the kernel)."""
+    keys = _capsule(keyset_cuda_cap, PrebuiltBSIKeysCUDA, "Invalid CUDA keys capsule")
+    qb = _capsule(query_batch_cap, PrebuiltBSIQueryBatchCUDA, "Invalid CUDA query-batch capsule")
+    Q, Sa, W = qb.words.shape
+    chunks = (W + 3) // 4
+    ints = torch.zeros((Q, keys.num_keys, chunks), dtype=torch.int32, device=qb.words.device)
+    if qb.chunk_scales is not None and qb.chunk_scales.numel() > 0:
+        scales, stride = qb.chunk_scales, int(qb.chunk_scales.shape[1])
+    else:
+        scales, stride = qb.row_scales, 1
+    code = {"auto": _lib.CORE_AUTO, "valu": _lib.CORE_VALU, "mfma": _lib.CORE_MFMA}[core]
+    out, _ = _dot(qb.words, qb.ints8, scales, stride, int(Sa), int(W), keys, int(Q), qb.decimals, chunk_ints=ints, core=code)
+    return ints, out
+
+
+def debug_quantize_int64_cpu(values: torch.Tensor, decimal_places: int) -> torch.Tensor:
+    """bsiFunctions.cpp:760-774: round-half-away quantisation on the host (a CPU function in the
+    reference too; exact for float inputs because the fp64 product and the +0.5 are exact)."""
+    x = values.detach().to("cpu", torch.float32).to(torch.float64) * (10.0 ** int(decimal_places))
+    return torch.where(x >= 0, torch.floor(x + 0.5), -torch.floor(-x + 0.5)).to(torch.int64)
+
+
+def _cpu_path_absent(name: str):
+    def fn(*_a, **_k):
+        raise RuntimeError(
+            f"bsi_ops.{name}: the CPU BSI path of the reference lives in the bsiCPP library, which is not part "
+            "of this build; use the *_cuda functions")
+    fn.__name__ = name
+    fn.__doc__ = "CPU decimal-path entry of the reference (bsiFunctions.cpp:811-846); not built here."
+    return fn
+
+
+for _n in ("dot_product", "dot_product_decimal", "vector_dot_product", "vector_dot_product_no_precison",
+           "random_number_dot_product_vector", "random_number_dot_product_bsi", "batch_dot_product", "build_bsi_keys",
+           "build_bsi_query", "batch_dot_product_prebuilt", "batch_dot_product_prebuilt_capsule", "keyset_slice_stats",
+           "tensor_slice_stats", "keyset_size_on_disk", "save_keyset", "debug_bsi_query_words"):
+    globals()[_n] = _cpu_path_absent(_n)
+del _n

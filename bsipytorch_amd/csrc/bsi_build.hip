@@ -1,0 +1,515 @@
+// BSI builder for gfx950: float -> rounded decimal ints -> block-floating shift -> fixed-bit
+// two's-complement values -> bit-planes in canonical [rows, slices, W64] words.
+//
+// wave64 mapping: one wavefront owns one 256-element chunk of one row.  A lane loads elements
+// lane, lane+64, lane+128, lane+192 of the chunk (four fully coalesced 256-byte wave loads), the
+// chunk maximum is a butterfly reduction across the wave, and one 64-bit `__ballot` per slice per
+// load IS the packed plane word (no lo/hi merge, no LDS, no block barrier).  The chunk-scale
+// build is therefore a single pass over the activations.
+//
+// Arithmetic follows the reference's quantiser kernels (bsi_ops/csrc/cuda/bsi_cuda_kernels_quant.cuh:
+// rounding :24-29, shift :82-108, rounded shift + clamp :205-226) and packer
+// (bsi_cuda_kernels_pack.cuh:129-174).
+#include "bsi_common.h"
+
+namespace bsi {
+
+constexpr int kBlock = 256;
+constexpr int kWavesPerBlock = kBlock / BSI_WAVE;
+
+// Position of element e (0..255) of a chunk inside the chunk's 256 int8 bytes in the MFMA core's
+// order: element 32w + 8m + t sits at byte 32w + 4t + m (see planes_to_int8 in bsi_dot.hip).
+__device__ __forceinline__ int mfma_byte_pos(int e) {
+    const int w = e >> 5, r = e & 31;
+    const int m = r >> 3, t = r & 7;
+    return (w << 5) + (t << 2) + m;
+}
+
+// ---------------------------------------------------------------- elementwise
+
+template <typename T>
+__global__ void round_to_int64_kernel(const T* __restrict__ x, int64_t total, double dec_scale,
+                                      long long* __restrict__ out) {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += stride)
+        out[i] = round_scaled(load_as_float<T>(x, i), dec_scale);
+}
+
+__global__ void apply_shift_clamp_kernel(long long* __restrict__ ints, int64_t total, int64_t d, int chunks,
+                                         const int* __restrict__ shifts, long long qmin, long long qmax) {
+    // chunks == 0: one shift per row; else one per (row, col >> 8)
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const int64_t row = i / d;
+        int shift;
+        if (chunks > 0) {
+            int c = static_cast<int>((i - row * d) >> 8);
+            if (c >= chunks) c = chunks - 1;
+            shift = shifts[row * chunks + c];
+        } else {
+            shift = shifts[row];
+        }
+        ints[i] = shift_clamp(ints[i], shift, qmin, qmax);
+    }
+}
+
+// ---------------------------------------------------------------- shift / scale passes
+
+// Source of rounded ints: either the float input (rounded on the fly) or staged int64.
+template <typename T>
+struct RoundedFromInput {
+    const T* x;
+    double dec_scale;
+    __device__ __forceinline__ long long operator()(int64_t i) const { return round_scaled(load_as_float<T>(x, i), dec_scale); }
+};
+struct RoundedFromInts {
+    const long long* v;
+    __device__ __forceinline__ long long operator()(int64_t i) const { return v[i]; }
+};
+
+// One wave per (row, chunk).
+template <typename Src>
+__global__ void chunk_shift_scale_kernel(Src src, int64_t Q, int64_t d, int chunks, int fixed_bits, float clip_k,
+                                         int* __restrict__ shifts, float* __restrict__ scales) {
+    const int lane = threadIdx.x & (BSI_WAVE - 1);
+    const int64_t wave = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
+    if (wave >= Q * chunks) return;
+    const int64_t row = wave / chunks;
+    const int c = static_cast<int>(wave - row * chunks);
+    const int64_t start = static_cast<int64_t>(c) * BSI_CHUNK_ELEMS;
+    int64_t valid = d - start;
+    if (valid > BSI_CHUNK_ELEMS) valid = BSI_CHUNK_ELEMS;
+    if (valid < 0) valid = 0;
+    unsigned long long mx = 0ULL;
+    double sum = 0.0;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int e = k * BSI_WAVE + lane;
+        if (e < valid) {
+            const unsigned long long av = uabs_ll(src(row * d + start + e));
+            if (av > mx) mx = av;
+            sum += static_cast<double>(av);
+        }
+    }
+    mx = wave_max_u64(mx);
+    sum = wave_sum_f64(sum);
+    if (lane == 0) {
+        const int shift = (valid > 0) ? compute_shift(mx, sum, static_cast<int>(valid), fixed_bits, clip_k) : 0;
+        shifts[wave] = shift;
+        scales[wave] = static_cast<float>(1ULL << shift);
+    }
+}
+
+// One block per row.
+template <typename Src>
+__global__ void row_shift_scale_kernel(Src src, int64_t Q, int64_t d, int fixed_bits, float clip_k,
+                                       int* __restrict__ shifts, float* __restrict__ scales) {
+    __shared__ unsigned long long smax[kWavesPerBlock];
+    __shared__ double ssum[kWavesPerBlock];
+    const int64_t row = blockIdx.x;
+    if (row >= Q) return;
+    unsigned long long mx = 0ULL;
+    double sum = 0.0;
+    for (int64_t e = threadIdx.x; e < d; e += kBlock) {
+        const unsigned long long av = uabs_ll(src(row * d + e));
+        if (av > mx) mx = av;
+        sum += static_cast<double>(av);
+    }
+    mx = wave_max_u64(mx);
+    sum = wave_sum_f64(sum);
+    if ((threadIdx.x & (BSI_WAVE - 1)) == 0) {
+        smax[threadIdx.x >> 6] = mx;
+        ssum[threadIdx.x >> 6] = sum;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < kWavesPerBlock; ++w) {
+            if (smax[w] > mx) mx = smax[w];
+            sum += ssum[w];
+        }
+        const int shift = compute_shift(mx, sum, static_cast<int>(d), fixed_bits, clip_k);
+        shifts[row] = shift;
+        scales[row] = static_cast<float>(1ULL << shift);
+    }
+}
+
+// ---------------------------------------------------------------- pack
+
+// Ballot-pack the four 64-element groups of one chunk held as v[0..3] (low `slices` bits valid) and
+// store words 4c..4c+3 of every slice.  Lane s keeps slice s, so each active lane issues one
+// contiguous run of stores.
+__device__ __forceinline__ void ballot_pack_store(const unsigned long long v[4], int slices, int lane, int c,
+                                                  int words_per_slice, unsigned long long* __restrict__ out_row) {
+    unsigned long long keep[4] = {0ULL, 0ULL, 0ULL, 0ULL};
+    for (int s = 0; s < slices; ++s) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const unsigned long long word = __ballot(((v[k] >> s) & 1ULL) != 0ULL);
+            if (lane == (s & (BSI_WAVE - 1))) keep[k] = word;
+        }
+        if (lane == (s & (BSI_WAVE - 1))) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int w = c * BSI_CHUNK_WORDS + k;
+                if (w < words_per_slice) out_row[static_cast<size_t>(s) * words_per_slice + w] = keep[k];
+            }
+        }
+    }
+}
+
+// Quantise (given shifts) + pack.  chunks > 0: shift per (row, chunk); chunks == 0: shift per row.
+// One wave per (row, group of 4 words).
+template <typename Src, bool kQuantise>
+__global__ void shift_pack_kernel(Src src, int64_t Q, int64_t d, int chunks, int slices, int words_per_slice,
+                                  int fixed_bits, const int* __restrict__ shifts, unsigned long long* __restrict__ out) {
+    const int lane = threadIdx.x & (BSI_WAVE - 1);
+    const int groups = (words_per_slice + BSI_CHUNK_WORDS - 1) / BSI_CHUNK_WORDS;
+    const int64_t wave = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
+    if (wave >= Q * groups) return;
+    const int64_t row = wave / groups;
+    const int c = static_cast<int>(wave - row * groups);
+    const unsigned long long mask = (slices >= 64) ? ~0ULL : ((1ULL << slices) - 1ULL);
+    int shift = 0;
+    long long qmin = 0, qmax = 0;
+    if (kQuantise) {
+        int sc = c;
+        if (chunks > 0 && sc >= chunks) sc = chunks - 1;
+        shift = (chunks > 0) ? shifts[row * chunks + sc] : shifts[row];
+        qmax = (1LL << (fixed_bits - 1)) - 1LL;
+        qmin = -(1LL << (fixed_bits - 1));
+    }
+    unsigned long long v[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int64_t e = static_cast<int64_t>(c) * BSI_CHUNK_ELEMS + k * BSI_WAVE + lane;
+        v[k] = 0ULL;
+        if (e < d) {
+            long long r = src(row * d + e);
+            if (kQuantise) r = shift_clamp(r, shift, qmin, qmax);
+            v[k] = static_cast<unsigned long long>(r) & mask;
+        }
+    }
+    ballot_pack_store(v, slices, lane, c, words_per_slice,
+                      out + static_cast<size_t>(row) * slices * words_per_slice);
+}
+
+// ---------------------------------------------------------------- fused builds
+
+// Chunk-scale build in one pass: one wave per (row, chunk) rounds, reduces, shifts, clamps, packs.
+template <typename T>
+__global__ void build_fixed_chunk_kernel(const T* __restrict__ x, int64_t Q, int64_t d, int chunks, int slices,
+                                         int words_per_slice, double dec_scale, float clip_k,
+                                         unsigned long long* __restrict__ words, int* __restrict__ shifts,
+                                         float* __restrict__ scales, int8_t* __restrict__ ints8) {
+    const int lane = threadIdx.x & (BSI_WAVE - 1);
+    const int64_t wave = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
+    if (wave >= Q * chunks) return;
+    const int64_t row = wave / chunks;
+    const int c = static_cast<int>(wave - row * chunks);
+    const int64_t start = static_cast<int64_t>(c) * BSI_CHUNK_ELEMS;
+    int64_t valid = d - start;
+    if (valid > BSI_CHUNK_ELEMS) valid = BSI_CHUNK_ELEMS;
+    if (valid < 0) valid = 0;
+
+    long long r[4];
+    unsigned long long mx = 0ULL;
+    double sum = 0.0;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int e = k * BSI_WAVE + lane;
+        r[k] = 0;
+        if (e < valid) {
+            r[k] = round_scaled(load_as_float<T>(x, row * d + start + e), dec_scale);
+            const unsigned long long av = uabs_ll(r[k]);
+            if (av > mx) mx = av;
+            sum += static_cast<double>(av);
+        }
+    }
+    mx = wave_max_u64(mx);
+    if (clip_k > 0.0f) sum = wave_sum_f64(sum);
+    const int shift = (valid > 0) ? compute_shift(mx, sum, static_cast<int>(valid), slices, clip_k) : 0;
+    if (lane == 0) {
+        shifts[wave] = shift;
+        scales[wave] = static_cast<float>(1ULL << shift);
+    }
+    const long long qmax = (1LL << (slices - 1)) - 1LL;
+    const long long qmin = -(1LL << (slices - 1));
+    const unsigned long long mask = (1ULL << slices) - 1ULL;
+    unsigned long long v[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int e = k * BSI_WAVE + lane;
+        const long long q = (e < valid) ? shift_clamp(r[k], shift, qmin, qmax) : 0;
+        v[k] = static_cast<unsigned long long>(q) & mask;
+        if (ints8 != nullptr)
+            ints8[(static_cast<size_t>(row) * chunks + c) * BSI_CHUNK_ELEMS + mfma_byte_pos(e)] =
+                static_cast<int8_t>(static_cast<int>(q) << (8 - slices));
+    }
+    ballot_pack_store(v, slices, lane, c, words_per_slice,
+                      words + static_cast<size_t>(row) * slices * words_per_slice);
+}
+
+// Row-scale build: one block per row; pass 1 reduces the row maximum, pass 2 (row now in cache)
+// quantises and packs, one wave per group of 4 words.
+template <typename T>
+__global__ void build_fixed_row_kernel(const T* __restrict__ x, int64_t Q, int64_t d, int slices,
+                                       int words_per_slice, double dec_scale, float clip_k,
+                                       unsigned long long* __restrict__ words, int* __restrict__ shifts,
+                                       float* __restrict__ scales, int8_t* __restrict__ ints8) {
+    __shared__ unsigned long long smax[kWavesPerBlock];
+    __shared__ double ssum[kWavesPerBlock];
+    __shared__ int sshift;
+    const int64_t row = blockIdx.x;
+    if (row >= Q) return;
+    const int lane = threadIdx.x & (BSI_WAVE - 1);
+    const int wid = threadIdx.x >> 6;
+    unsigned long long mx = 0ULL;
+    double sum = 0.0;
+    for (int64_t e = threadIdx.x; e < d; e += kBlock) {
+        const unsigned long long av = uabs_ll(round_scaled(load_as_float<T>(x, row * d + e), dec_scale));
+        if (av > mx) mx = av;
+        sum += static_cast<double>(av);
+    }
+    mx = wave_max_u64(mx);
+    sum = wave_sum_f64(sum);
+    if (lane == 0) {
+        smax[wid] = mx;
+        ssum[wid] = sum;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < kWavesPerBlock; ++w) {
+            if (smax[w] > mx) mx = smax[w];
+            sum += ssum[w];
+        }
+        const int shift = compute_shift(mx, sum, static_cast<int>(d), slices, clip_k);
+        sshift = shift;
+        shifts[row] = shift;
+        scales[row] = static_cast<float>(1ULL << shift);
+    }
+    __syncthreads();
+    const int shift = sshift;
+    const long long qmax = (1LL << (slices - 1)) - 1LL;
+    const long long qmin = -(1LL << (slices - 1));
+    const unsigned long long mask = (1ULL << slices) - 1ULL;
+    const int groups = (words_per_slice + BSI_CHUNK_WORDS - 1) / BSI_CHUNK_WORDS;
+    for (int c = wid; c < groups; c += kWavesPerBlock) {
+        unsigned long long v[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int el = k * BSI_WAVE + lane;
+            const int64_t e = static_cast<int64_t>(c) * BSI_CHUNK_ELEMS + el;
+            long long q = 0;
+            if (e < d) q = shift_clamp(round_scaled(load_as_float<T>(x, row * d + e), dec_scale), shift, qmin, qmax);
+            v[k] = static_cast<unsigned long long>(q) & mask;
+            if (ints8 != nullptr)
+                ints8[(static_cast<size_t>(row) * groups + c) * BSI_CHUNK_ELEMS + mfma_byte_pos(el)] =
+                    static_cast<int8_t>(static_cast<int>(q) << (8 - slices));
+        }
+        ballot_pack_store(v, slices, lane, c, words_per_slice,
+                          words + static_cast<size_t>(row) * slices * words_per_slice);
+    }
+}
+
+static inline unsigned grid_for(int64_t waves) {
+    return static_cast<unsigned>((waves + kWavesPerBlock - 1) / kWavesPerBlock);
+}
+static inline unsigned grid_elementwise(int64_t total) {
+    int64_t b = (total + kBlock - 1) / kBlock;
+    if (b > 65535 * 16) b = 65535 * 16;
+    if (b < 1) b = 1;
+    return static_cast<unsigned>(b);
+}
+
+}  // namespace bsi
+
+using namespace bsi;
+
+#define BSI_DISPATCH_DTYPE(dtype, ...)                                                   \
+    switch (dtype) {                                                                     \
+        case BSI_DTYPE_F32: { using T = float; __VA_ARGS__; break; }                     \
+        case BSI_DTYPE_F16: { using T = __half; __VA_ARGS__; break; }                    \
+        case BSI_DTYPE_BF16: { using T = __hip_bfloat16; __VA_ARGS__; break; }           \
+        default: return fail(BSI_ERR_INVALID, "unknown dtype code %d", dtype);           \
+    }
+
+extern "C" int bsi_hip_quantize_round_to_int64(const void* x, int dtype, int64_t total, double dec_scale,
+                                               int64_t* out, void* stream) {
+    BSI_REQUIRE(total >= 0, "total must be >= 0");
+    if (total == 0) return BSI_OK;
+    BSI_REQUIRE(x && out, "null pointer");
+    BSI_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(round_to_int64_kernel<T>, dim3(grid_elementwise(total)), dim3(kBlock),
+                                                 0, as_stream(stream), static_cast<const T*>(x), total, dec_scale,
+                                                 reinterpret_cast<long long*>(out)));
+    BSI_LAUNCH_CHECK("round_to_int64_kernel");
+    return BSI_OK;
+}
+
+extern "C" int bsi_hip_compute_row_shift_scale(const int64_t* ints, int64_t Q, int64_t d, int fixed_bits, float clip_k,
+                                               int32_t* shifts, float* scales, void* stream) {
+    BSI_REQUIRE(Q >= 0 && d >= 0, "negative size");
+    if (Q == 0) return BSI_OK;
+    BSI_REQUIRE(ints && shifts && scales, "null pointer");
+    RoundedFromInts src{reinterpret_cast<const long long*>(ints)};
+    hipLaunchKernelGGL(row_shift_scale_kernel<RoundedFromInts>, dim3(static_cast<unsigned>(Q)), dim3(kBlock), 0,
+                       as_stream(stream), src, Q, d, fixed_bits, clip_k, shifts, scales);
+    BSI_LAUNCH_CHECK("row_shift_scale_kernel");
+    return BSI_OK;
+}
+
+extern "C" int bsi_hip_compute_chunk_shift_scale(const int64_t* ints, int64_t Q, int64_t d, int chunks, int fixed_bits,
+                                                 float clip_k, int32_t* shifts, float* scales, void* stream) {
+    BSI_REQUIRE(Q >= 0 && d >= 0 && chunks >= 0, "negative size");
+    if (Q == 0 || chunks == 0) return BSI_OK;
+    BSI_REQUIRE(ints && shifts && scales, "null pointer");
+    RoundedFromInts src{reinterpret_cast<const long long*>(ints)};
+    hipLaunchKernelGGL(chunk_shift_scale_kernel<RoundedFromInts>, dim3(grid_for(Q * chunks)), dim3(kBlock), 0,
+                       as_stream(stream), src, Q, d, chunks, fixed_bits, clip_k, shifts, scales);
+    BSI_LAUNCH_CHECK("chunk_shift_scale_kernel");
+    return BSI_OK;
+}
+
+extern "C" int bsi_hip_apply_row_shift_clamp(int64_t* ints, int64_t Q, int64_t d, const int32_t* shifts, int fixed_bits,
+                                             void* stream) {
+    BSI_REQUIRE(Q >= 0 && d >= 0, "negative size");
+    BSI_REQUIRE(fixed_bits >= 2 && fixed_bits <= 63, "fixed_bits must be in [2, 63]");
+    if (Q == 0 || d == 0) return BSI_OK;
+    BSI_REQUIRE(ints && shifts, "null pointer");
+    hipLaunchKernelGGL(apply_shift_clamp_kernel, dim3(grid_elementwise(Q * d)), dim3(kBlock), 0, as_stream(stream),
+                       reinterpret_cast<long long*>(ints), Q * d, d, 0, shifts, -(1LL << (fixed_bits - 1)),
+                       (1LL << (fixed_bits - 1)) - 1LL);
+    BSI_LAUNCH_CHECK("apply_shift_clamp_kernel");
+    return BSI_OK;
+}
+
+extern "C" int bsi_hip_apply_chunk_shift_clamp(int64_t* ints, int64_t Q, int64_t d, int chunks, const int32_t* shifts,
+                                               int fixed_bits, void* stream) {
+    BSI_REQUIRE(Q >= 0 && d >= 0 && chunks > 0, "bad size");
+    BSI_REQUIRE(fixed_bits >= 2 && fixed_bits <= 63, "fixed_bits must be in [2, 63]");
+    if (Q == 0 || d == 0) return BSI_OK;
+    BSI_REQUIRE(ints && shifts, "null pointer");
+    hipLaunchKernelGGL(apply_shift_clamp_kernel, dim3(grid_elementwise(Q * d)), dim3(kBlock), 0, as_stream(stream),
+                       reinterpret_cast<long long*>(ints), Q * d, d, chunks, shifts, -(1LL << (fixed_bits - 1)),
+                       (1LL << (fixed_bits - 1)) - 1LL);
+    BSI_LAUNCH_CHECK("apply_shift_clamp_kernel");
+    return BSI_OK;
+}
+
+extern "C" int bsi_hip_compute_row_shift_scale_from_input(const void* x, int dtype, int64_t Q, int64_t d,
+                                                          double dec_scale, int fixed_bits, float clip_k,
+                                                          int32_t* shifts, float* scales, void* stream) {
+    BSI_REQUIRE(Q >= 0 && d >= 0, "negative size");
+    if (Q == 0) return BSI_OK;
+    BSI_REQUIRE(x && shifts && scales, "null pointer");
+    BSI_DISPATCH_DTYPE(dtype, {
+        RoundedFromInput<T> src{static_cast<const T*>(x), dec_scale};
+        hipLaunchKernelGGL(row_shift_scale_kernel<RoundedFromInput<T>>, dim3(static_cast<unsigned>(Q)), dim3(kBlock),
+                           0, as_stream(stream), src, Q, d, fixed_bits, clip_k, shifts, scales);
+    });
+    BSI_LAUNCH_CHECK("row_shift_scale_kernel");
+    return BSI_OK;
+}
+
+extern "C" int bsi_hip_compute_chunk_shift_scale_from_input(const void* x, int dtype, int64_t Q, int64_t d, int chunks,
+                                                            double dec_scale, int fixed_bits, float clip_k,
+                                                            int32_t* shifts, float* scales, void* stream) {
+    BSI_REQUIRE(Q >= 0 && d >= 0 && chunks >= 0, "negative size");
+    if (Q == 0 || chunks == 0) return BSI_OK;
+    BSI_REQUIRE(x && shifts && scales, "null pointer");
+    BSI_DISPATCH_DTYPE(dtype, {
+        RoundedFromInput<T> src{static_cast<const T*>(x), dec_scale};
+        hipLaunchKernelGGL(chunk_shift_scale_kernel<RoundedFromInput<T>>, dim3(grid_for(Q * chunks)), dim3(kBlock), 0,
+                           as_stream(stream), src, Q, d, chunks, fixed_bits, clip_k, shifts, scales);
+    });
+    BSI_LAUNCH_CHECK("chunk_shift_scale_kernel");
+    return BSI_OK;
+}
+
+static int check_pack_args(int64_t Q, int64_t d, int slices, int words_per_slice) {
+    BSI_REQUIRE(Q >= 0 && d >= 0, "negative size");
+    BSI_REQUIRE(slices >= 1 && slices <= 64, "slices must be in [1, 64]");
+    BSI_REQUIRE(words_per_slice >= 1 && static_cast<int64_t>(words_per_slice) * 64 >= d,
+                "words_per_slice * 64 must cover d");
+    return BSI_OK;
+}
+
+extern "C" int bsi_hip_quantize_shift_pack_row_batch(const void* x, int dtype, int64_t Q, int64_t d, int slices,
+                                                     int words_per_slice, double dec_scale, int fixed_bits,
+                                                     const int32_t* shifts, uint64_t* words, void* stream) {
+    if (int rc = check_pack_args(Q, d, slices, words_per_slice)) return rc;
+    BSI_REQUIRE(fixed_bits >= 2 && fixed_bits <= 63, "fixed_bits must be in [2, 63]");
+    if (Q == 0) return BSI_OK;
+    BSI_REQUIRE(x && shifts && words, "null pointer");
+    const int groups = (words_per_slice + 3) / 4;
+    BSI_DISPATCH_DTYPE(dtype, {
+        RoundedFromInput<T> src{static_cast<const T*>(x), dec_scale};
+        hipLaunchKernelGGL((shift_pack_kernel<RoundedFromInput<T>, true>), dim3(grid_for(Q * groups)), dim3(kBlock), 0,
+                           as_stream(stream), src, Q, d, 0, slices, words_per_slice, fixed_bits, shifts,
+                           reinterpret_cast<unsigned long long*>(words));
+    });
+    BSI_LAUNCH_CHECK("shift_pack_kernel");
+    return BSI_OK;
+}
+
+extern "C" int bsi_hip_quantize_shift_pack_chunk_batch(const void* x, int dtype, int64_t Q, int64_t d, int chunks,
+                                                       int slices, int words_per_slice, double dec_scale,
+                                                       int fixed_bits, const int32_t* shifts, uint64_t* words,
+                                                       void* stream) {
+    if (int rc = check_pack_args(Q, d, slices, words_per_slice)) return rc;
+    BSI_REQUIRE(fixed_bits >= 2 && fixed_bits <= 63, "fixed_bits must be in [2, 63]");
+    BSI_REQUIRE(chunks > 0, "chunks must be > 0");
+    if (Q == 0) return BSI_OK;
+    BSI_REQUIRE(x && shifts && words, "null pointer");
+    const int groups = (words_per_slice + 3) / 4;
+    BSI_DISPATCH_DTYPE(dtype, {
+        RoundedFromInput<T> src{static_cast<const T*>(x), dec_scale};
+        hipLaunchKernelGGL((shift_pack_kernel<RoundedFromInput<T>, true>), dim3(grid_for(Q * groups)), dim3(kBlock), 0,
+                           as_stream(stream), src, Q, d, chunks, slices, words_per_slice, fixed_bits, shifts,
+                           reinterpret_cast<unsigned long long*>(words));
+    });
+    BSI_LAUNCH_CHECK("shift_pack_kernel");
+    return BSI_OK;
+}
+
+extern "C" int bsi_hip_pack_bits_batch(const int64_t* ints, int64_t Q, int64_t d, int slices, int words_per_slice,
+                                       uint64_t* words, void* stream) {
+    if (int rc = check_pack_args(Q, d, slices, words_per_slice)) return rc;
+    if (Q == 0) return BSI_OK;
+    BSI_REQUIRE(ints && words, "null pointer");
+    const int groups = (words_per_slice + 3) / 4;
+    RoundedFromInts src{reinterpret_cast<const long long*>(ints)};
+    hipLaunchKernelGGL((shift_pack_kernel<RoundedFromInts, false>), dim3(grid_for(Q * groups)), dim3(kBlock), 0,
+                       as_stream(stream), src, Q, d, 0, slices, words_per_slice, 0, nullptr,
+                       reinterpret_cast<unsigned long long*>(words));
+    BSI_LAUNCH_CHECK("shift_pack_kernel");
+    return BSI_OK;
+}
+
+extern "C" int bsi_hip_build_fixed(const void* x, int dtype, int64_t Q, int64_t d, int decimal_places, int fixed_bits,
+                                   int chunk_scale, float clip_k, uint64_t* words, int32_t* shifts, float* scales,
+                                   int8_t* ints8, void* stream) {
+    BSI_REQUIRE(Q >= 0 && d >= 0, "negative size");
+    BSI_REQUIRE(fixed_bits >= 2 && fixed_bits <= 32, "fixed_bits must be in [2, 32]");
+    BSI_REQUIRE(ints8 == nullptr || fixed_bits <= 8, "int8 output needs fixed_bits <= 8");
+    if (Q == 0 || d == 0) return BSI_OK;
+    BSI_REQUIRE(x && words && shifts && scales, "null pointer");
+    const int W = static_cast<int>((d + 63) / 64);
+    const int chunks = static_cast<int>((d + 255) / 256);
+    const double dec_scale = pow(10.0, static_cast<double>(decimal_places));
+    if (chunk_scale) {
+        BSI_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(build_fixed_chunk_kernel<T>, dim3(grid_for(Q * chunks)),
+                                                     dim3(kBlock), 0, as_stream(stream), static_cast<const T*>(x), Q,
+                                                     d, chunks, fixed_bits, W, dec_scale, clip_k,
+                                                     reinterpret_cast<unsigned long long*>(words), shifts, scales,
+                                                     ints8));
+        BSI_LAUNCH_CHECK("build_fixed_chunk_kernel");
+    } else {
+        BSI_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(build_fixed_row_kernel<T>, dim3(static_cast<unsigned>(Q)),
+                                                     dim3(kBlock), 0, as_stream(stream), static_cast<const T*>(x), Q,
+                                                     d, fixed_bits, W, dec_scale, clip_k,
+                                                     reinterpret_cast<unsigned long long*>(words), shifts, scales,
+                                                     ints8));
+        BSI_LAUNCH_CHECK("build_fixed_row_kernel");
+    }
+    return BSI_OK;
+}

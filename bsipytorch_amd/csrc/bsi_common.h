@@ -1,0 +1,131 @@
+// Shared host/device helpers of libbsi_hip.so (gfx950 only, wave64).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <hip/hip_bf16.h>
+#include <stdint.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <string>
+
+#include "../../include/bsi_hip.h"
+
+#define BSI_WAVE 64
+#define BSI_CHUNK_ELEMS 256
+#define BSI_CHUNK_WORDS 4
+
+namespace bsi {
+
+// ---- error plumbing: every extern "C" entry returns a code and leaves a message here ----
+std::string& last_error_ref();
+int fail(int code, const char* fmt, ...);
+
+#define BSI_REQUIRE(cond, ...)                                   \
+    do {                                                         \
+        if (!(cond)) return ::bsi::fail(BSI_ERR_INVALID, __VA_ARGS__); \
+    } while (0)
+
+#define BSI_HIP_CHECK(expr)                                                                          \
+    do {                                                                                             \
+        hipError_t _e = (expr);                                                                      \
+        if (_e != hipSuccess)                                                                        \
+            return ::bsi::fail(BSI_ERR_HIP, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(_e), __FILE__, __LINE__); \
+    } while (0)
+
+// After a kernel launch: surface launch-configuration errors immediately.
+#define BSI_LAUNCH_CHECK(name)                                                                       \
+    do {                                                                                             \
+        hipError_t _e = hipGetLastError();                                                           \
+        if (_e != hipSuccess)                                                                        \
+            return ::bsi::fail(BSI_ERR_HIP, "launch of %s failed: %s", name, hipGetErrorString(_e)); \
+    } while (0)
+
+static inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+
+// ---- device helpers ----
+
+template <typename T>
+__device__ __forceinline__ float load_as_float(const T* p, int64_t i);
+template <>
+__device__ __forceinline__ float load_as_float<float>(const float* p, int64_t i) { return p[i]; }
+template <>
+__device__ __forceinline__ float load_as_float<__half>(const __half* p, int64_t i) { return __half2float(p[i]); }
+template <>
+__device__ __forceinline__ float load_as_float<__hip_bfloat16>(const __hip_bfloat16* p, int64_t i) {
+    // bf16 is the top half of an fp32
+    const uint16_t raw = reinterpret_cast<const uint16_t*>(p)[i];
+    return __uint_as_float(static_cast<uint32_t>(raw) << 16);
+}
+
+// round half away from zero of x (x = (double)(float)v * 10^dec); the multiply is done by the
+// caller with __dmul_rn so that it is never contracted with the + 0.5
+__device__ __forceinline__ long long round_half_away(double x) {
+    if (x >= 0.0) return static_cast<long long>(floor(__dadd_rn(x, 0.5)));
+    return -static_cast<long long>(floor(__dadd_rn(-x, 0.5)));
+}
+
+__device__ __forceinline__ long long round_scaled(float f, double dec_scale) {
+    return round_half_away(__dmul_rn(static_cast<double>(f), dec_scale));
+}
+
+__device__ __forceinline__ unsigned long long uabs_ll(long long v) {
+    return static_cast<unsigned long long>(v >= 0 ? v : -v);
+}
+
+// bits needed for max_abs minus the magnitude bits available; optional outlier clipping
+__device__ __forceinline__ int compute_shift(unsigned long long max_abs, double sum_abs, int count, int fixed_bits,
+                                             float clip_k) {
+    if (fixed_bits <= 0) return 0;
+    int bits = 0;
+    if (clip_k > 0.0f && count > 0) {
+        double effective = static_cast<double>(max_abs);
+        const double mean_abs = sum_abs / static_cast<double>(count);
+        const double clip_max = mean_abs * static_cast<double>(clip_k);
+        if (clip_max < effective) effective = clip_max;
+        if (effective > 0.0) {
+            int e = 0;
+            (void)frexp(effective, &e);
+            bits = e;
+        }
+    } else {
+        bits = (max_abs > 0ULL) ? (64 - __clzll(static_cast<long long>(max_abs))) : 0;
+    }
+    int shift = bits - (fixed_bits - 1);
+    if (shift < 0) shift = 0;
+    if (shift > 62) shift = 62;
+    return shift;
+}
+
+__device__ __forceinline__ long long shift_clamp(long long v, int shift, long long qmin, long long qmax) {
+    const unsigned long long av = uabs_ll(v);
+    const unsigned long long round_add = (shift > 0) ? (1ULL << (shift - 1)) : 0ULL;
+    const unsigned long long q = (av + round_add) >> shift;
+    long long out = (v < 0) ? -static_cast<long long>(q) : static_cast<long long>(q);
+    if (out < qmin) out = qmin;
+    if (out > qmax) out = qmax;
+    return out;
+}
+
+// wave64 butterfly reductions (every lane ends with the result)
+__device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const unsigned long long o = __shfl_xor(v, off, BSI_WAVE);
+        if (o > v) v = o;
+    }
+    return v;
+}
+__device__ __forceinline__ double wave_sum_f64(double v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, BSI_WAVE);
+    return v;
+}
+__device__ __forceinline__ unsigned long long wave_sum_u64(unsigned long long v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, BSI_WAVE);
+    return v;
+}
+
+}  // namespace bsi

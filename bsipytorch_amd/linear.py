@@ -1,0 +1,217 @@
+"""``BSIQuantizedLinear``: the BSI-linear drop-in for ``torch.nn.Linear`` and the model-wide
+replacement helper, mirroring ``bsi_ops/benchmarks/verify_accuracy_bsi.py:46-215,217-279,312-368,444-486``
+of the reference (same constructor arguments, attributes, counters and scope rules).
+
+forward(x): flatten to [Q, D] -> build query planes on the GPU -> BSI dot against the prebuilt key
+planes -> cast to x.dtype -> add bias -> restore the leading shape.
+"""
+from __future__ import annotations
+
+import os
+import time
+from typing import Any, Dict, List, Union
+
+import torch
+import torch.nn as nn
+
+from . import bsi_ops
+
+
+class BSIQuantizedLinear(nn.Module):
+    """Linear layer whose weight lives as BSI key planes (verify_accuracy_bsi.py:46-215)."""
+
+    def __init__(self, original_linear, decimalPlaces=2, compress_threshold=0.2, query_threshold=None,
+                 prefer_cuda: bool = True):
+        super().__init__()
+        self.decimalPlaces = int(decimalPlaces)
+        self.compress_threshold = float(compress_threshold)
+        self.query_compress_threshold = float(query_threshold) if query_threshold is not None else float(compress_threshold)
+        self.in_features = original_linear.in_features
+        self.out_features = original_linear.out_features
+
+        dense_weight = original_linear.weight.detach().to(torch.float32)
+        self.weight_fp32 = dense_weight.cpu()
+        self.weight_dense_memory_bytes = dense_weight.numel() * dense_weight.element_size()
+        if original_linear.bias is not None:
+            bias = original_linear.bias.detach().to(torch.float32)
+            self.register_buffer("bias", bias)
+            self.bias_fp32 = bias.cpu()
+            self.bias_memory_bytes = bias.numel() * bias.element_size()
+        else:
+            self.register_buffer("bias", None)
+            self.bias_fp32 = None
+            self.bias_memory_bytes = 0
+
+        assert prefer_cuda and torch.cuda.is_available(), \
+            "CUDA path required: build_bsi_keys_cuda not available or CUDA not present"
+        with torch.no_grad():
+            # build from the tensor where it already lives: no host round trip for device weights
+            src = dense_weight if dense_weight.is_cuda else self.weight_fp32
+            self._bsi_keys_cuda, total_mem_bytes, num_keys, d, _W = bsi_ops.build_bsi_keys_cuda(
+                src, self.decimalPlaces, float(self.compress_threshold))
+        assert num_keys == self.out_features and d == self.in_features
+        self.weight_bsi_memory_bytes = int(total_mem_bytes)
+        self.total_bsi_static_bytes = self.weight_bsi_memory_bytes + self.bias_memory_bytes
+        self.verbose = False
+        self.collect_stats = False
+        self._reset_counters()
+
+    def _reset_counters(self):
+        self.dot_ns_total = 0
+        self.dot_calls = 0
+        self.dot_kernel_ns_per_query_last = 0.0
+        self.dot_kernel_ns_per_scalar_last = 0.0
+        self.dot_query_vectors_total = 0
+        self.dot_output_elements_total = 0
+        self.build_ns_total = 0
+        self.build_quantize_ns_total = 0
+        self.build_pack_ns_total = 0
+        self.build_kernel_ns_total = 0
+        self.build_calls = 0
+
+    def reset_error_stats(self):
+        self.mse_sum = 0.0
+        self.mae_sum = 0.0
+        self.cosine_sum = 0.0
+        self.max_abs_error = 0.0
+        self.samples_tracked = 0
+
+    def forward(self, x):
+        original_dtype = x.dtype
+        original_shape = x.shape
+        if x.dim() != 2:
+            x = x.reshape(-1, x.shape[-1])
+        if os.getenv("BSI_QUERY_FP32", "0") != "0":
+            x = x.to(torch.float32)
+        batch_inputs = x.detach().contiguous()
+        q_rows = int(batch_inputs.shape[0])
+
+        t0 = time.perf_counter_ns()
+        use_packed = os.getenv("BSI_QUERY_PACKED", "1") != "0"
+        if use_packed:
+            qcap = bsi_ops.build_bsi_queries_cuda_batch_packed(batch_inputs, self.decimalPlaces,
+                                                               float(self.query_compress_threshold))
+        else:
+            qcap = bsi_ops.build_bsi_queries_cuda_batch(batch_inputs, self.decimalPlaces,
+                                                        float(self.query_compress_threshold))
+        self.build_ns_total += time.perf_counter_ns() - t0
+        q_ns, p_ns, t_ns = bsi_ops.get_last_query_build_profile_cuda()
+        self.build_quantize_ns_total += int(q_ns)
+        self.build_pack_ns_total += int(p_ns)
+        self.build_kernel_ns_total += int(t_ns)
+        self.build_calls += 1
+
+        if use_packed:
+            scores, ns_total, ns_q, ns_s = bsi_ops.batch_dot_product_multiquery_cuda_batch_caps(qcap, self._bsi_keys_cuda)
+        else:
+            scores, ns_total, ns_q, ns_s = bsi_ops.batch_dot_product_multiquery_cuda_caps(qcap, self._bsi_keys_cuda)
+        self.dot_kernel_ns_per_query_last = float(ns_q)
+        self.dot_kernel_ns_per_scalar_last = float(ns_s)
+        self.dot_query_vectors_total += q_rows
+        self.dot_output_elements_total += q_rows * int(self.out_features)
+        self.dot_ns_total += int(ns_total)
+        self.dot_calls += 1
+
+        scores = scores.to(dtype=original_dtype)
+        if self.bias is not None:
+            scores = scores + self.bias.to(device=scores.device, dtype=original_dtype)
+        if len(original_shape) != 2:
+            scores = scores.view(*original_shape[:-1], -1)
+        return scores
+
+
+_COUNTERS = ("dot_ns_total", "dot_calls", "build_ns_total", "build_quantize_ns_total", "build_pack_ns_total",
+             "build_kernel_ns_total", "build_calls", "dot_query_vectors_total", "dot_output_elements_total")
+
+
+def reset_bsi_dot_counters(model: nn.Module):
+    for m in model.modules():
+        if isinstance(m, BSIQuantizedLinear):
+            for c in _COUNTERS:
+                setattr(m, c, 0)
+
+
+def _sum(model: nn.Module, attr: str) -> int:
+    return sum(int(getattr(m, attr, 0)) for m in model.modules() if isinstance(m, BSIQuantizedLinear))
+
+
+def sum_bsi_dot_counters(model): return _sum(model, "dot_ns_total")
+def sum_bsi_build_counters(model): return _sum(model, "build_ns_total")
+def sum_bsi_build_quantize_counters(model): return _sum(model, "build_quantize_ns_total")
+def sum_bsi_build_pack_counters(model): return _sum(model, "build_pack_ns_total")
+def sum_bsi_build_kernel_counters(model): return _sum(model, "build_kernel_ns_total")
+def sum_bsi_dot_query_vectors(model): return _sum(model, "dot_query_vectors_total")
+def sum_bsi_dot_output_elements(model): return _sum(model, "dot_output_elements_total")
+
+
+def summarize_bsi_model(model: nn.Module) -> Dict[str, Any]:
+    """Per-layer and total byte accounting (verify_accuracy_bsi.py:312-368)."""
+    s: Dict[str, Any] = dict(total_bsi_bytes=0, total_dense_bytes=0, total_bias_bytes=0, total_fp16_linear_bytes=0,
+                             total_static_bytes=0, total_dense_with_bias_bytes=0, num_quantized_layers=0,
+                             total_slices=0, compressed_slices=0, verbatim_slices=0, layers=[])
+    for name, m in model.named_modules():
+        if not isinstance(m, BSIQuantizedLinear):
+            continue
+        fp16_bytes = int(m.in_features * m.out_features * 2)
+        s["layers"].append(dict(name=name, in_features=m.in_features, out_features=m.out_features,
+                                decimalPlaces=m.decimalPlaces, compress_threshold=m.compress_threshold,
+                                weight_bsi_bytes=m.weight_bsi_memory_bytes, weight_dense_bytes=m.weight_dense_memory_bytes,
+                                bias_bytes=m.bias_memory_bytes, weight_fp16_bytes=fp16_bytes))
+        s["total_bsi_bytes"] += m.weight_bsi_memory_bytes
+        s["total_dense_bytes"] += m.weight_dense_memory_bytes
+        s["total_bias_bytes"] += m.bias_memory_bytes
+        s["total_fp16_linear_bytes"] += fp16_bytes
+        s["num_quantized_layers"] += 1
+    s["total_static_bytes"] = s["total_bsi_bytes"] + s["total_bias_bytes"]
+    s["total_dense_with_bias_bytes"] = s["total_dense_bytes"] + s["total_bias_bytes"]
+    s["compressed_pct"] = 0.0
+    s["verbatim_pct"] = 0.0
+    return s
+
+
+def _resolve_layer_value(config: Union[float, Dict[str, float]], layer_kind: str, fallback: float) -> float:
+    if isinstance(config, dict):
+        if layer_kind in ("attention", "mlp"):
+            return float(config.get(layer_kind, config.get("default", fallback)))
+        return float(config.get("default", fallback))
+    return float(config)
+
+
+_ATTN_TOKENS = ("attn", "self_attn", "q_proj", "k_proj", "v_proj", "out_proj")
+_MLP_TOKENS = ("mlp", "ff", "ffn", "fc1", "fc2")
+
+
+def quantize_model_bsi(model, decimalPlaces=2, skip_lm_head=True, scope="all", compress_threshold=0.2,
+                       prefer_cuda: bool = True, verbose: bool = True):
+    """Replace every ``nn.Linear`` (except ``lm_head``) by ``BSIQuantizedLinear``; ``scope`` is
+    'all' | 'attention' | 'mlp', chosen by name tokens (verify_accuracy_bsi.py:444-486)."""
+    default_decimal = float(decimalPlaces if isinstance(decimalPlaces, (int, float)) else decimalPlaces.get("default", 2))
+    default_threshold = float(compress_threshold if isinstance(compress_threshold, (int, float))
+                              else compress_threshold.get("default", 0.2))
+    targets: List[str] = []
+    for name, module in model.named_modules():
+        if not isinstance(module, nn.Linear):
+            continue
+        if skip_lm_head and "lm_head" in name:
+            continue
+        is_attn = any(t in name for t in _ATTN_TOKENS)
+        is_mlp = any(t in name for t in _MLP_TOKENS)
+        if scope == "attention" and not is_attn:
+            continue
+        if scope == "mlp" and not is_mlp:
+            continue
+        targets.append(name)
+    for name in targets:
+        parent = model
+        parts = name.split(".")
+        for part in parts[:-1]:
+            parent = getattr(parent, part)
+        module = getattr(parent, parts[-1])
+        kind = "attention" if any(t in name for t in _ATTN_TOKENS) else "mlp" if any(t in name for t in _MLP_TOKENS) else "other"
+        setattr(parent, parts[-1], BSIQuantizedLinear(
+            module, decimalPlaces=_resolve_layer_value(decimalPlaces, kind, default_decimal),
+            compress_threshold=_resolve_layer_value(compress_threshold, kind, default_threshold),
+            prefer_cuda=prefer_cuda))
+    if verbose:
+        print(f"Quantized {len(targets)} linear layers to BSI with decimalPlaces={decimalPlaces} (scope={scope})")
+    return model

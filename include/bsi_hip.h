@@ -1,0 +1,193 @@
+/*
+ * bsi_hip.h -- C ABI of libbsi_hip.so, the MI355X (gfx950) implementation of the bsi_ops
+ * fixed-bit tensor-dot path: BSI builder, EWAH codec, weighted-popcount dot.
+ *
+ * Plain pointers and sizes only.  Every pointer named "device" must be memory of the current HIP
+ * device; `stream` is a hipStream_t passed as void* (NULL = the default stream).  All work is
+ * enqueued on `stream` and returns without synchronising unless stated.  Every function returns
+ * BSI_OK or an error code; bsi_hip_last_error() gives the message of the calling thread's last
+ * failure.  The caller owns every buffer.
+ *
+ * Each entry point names the reference interface it replaces (paths relative to the reference
+ * tree, bsi_ops/csrc/cuda/).  The reference declares these as `extern "C" void launch_*`
+ * (bsi_vector_cuda.cpp:91-242, bsi_cuda.cpp:29-57); the argument meaning is kept, `cudaStream_t`
+ * becomes `void*`, and an error code is returned instead of nothing.
+ *
+ * Canonical bit-plane layout ("words"): uint64 [rows, slices, W64], W64 = ceil(d / 64); bit b of
+ * word w of slice s is bit s of the two's-complement quantised value of element 64*w + b; bits
+ * past d are zero.  A "chunk" is 256 elements = 4 words; chunk scales are float [rows, chunks].
+ */
+#ifndef BSI_HIP_H
+#define BSI_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BSI_OK 0
+#define BSI_ERR_INVALID 1     /* bad argument (null pointer, negative size, unsupported combination) */
+#define BSI_ERR_HIP 2         /* a HIP runtime call or kernel launch failed */
+#define BSI_ERR_UNSUPPORTED 3 /* valid request that this build has no kernel for */
+
+/* Input element types; same codes as the reference's `input_dtype` (bsi_vector_cuda.cpp:346-351). */
+#define BSI_DTYPE_F32 0
+#define BSI_DTYPE_F16 1
+#define BSI_DTYPE_BF16 2
+
+/* Arithmetic core of the dot. */
+#define BSI_CORE_AUTO 0 /* MFMA when it applies, else VALU */
+#define BSI_CORE_VALU 1 /* v_and_b32 + v_bcnt_u32_b32 on bit-planes staged in LDS */
+#define BSI_CORE_MFMA 2 /* planes recombined to int8 in registers, v_mfma_i32_16x16x64_i8 */
+
+/* Layout of the key planes handed to the dot. */
+#define BSI_LAYOUT_CANONICAL 0 /* [R, Sb, W64] */
+#define BSI_LAYOUT_TILED16 1   /* [ceil(R/16), chunks, Sb, 64, 1] words: see bsi_hip_tile_key_planes */
+
+const char* bsi_hip_version(void);
+const char* bsi_hip_last_error(void);
+/* Name of the device architecture (e.g. "gfx950"), CU count and LDS bytes per workgroup. */
+int bsi_hip_device_info(char* arch, int arch_len, int* cu_count, int* lds_bytes);
+
+/* ---------------------------------------------------------------- builder */
+
+/* out[i] = round_half_away((double)(float)x[i] * dec_scale).
+ * Replaces launch_quantize_round_to_int64_batch (bsi_cuda_kernels_quant.cuh:638-668). */
+int bsi_hip_quantize_round_to_int64(const void* x_device, int dtype, int64_t total, double dec_scale,
+                                    int64_t* out_device, void* stream);
+
+/* Per-row / per-(row, 256-element chunk) shift and power-of-two scale from already rounded ints.
+ * Replace launch_compute_row_shift_scale / launch_compute_chunk_shift_scale
+ * (bsi_cuda_kernels_quant.cuh:670-700). shifts/scales are [Q] or [Q, chunks]. */
+int bsi_hip_compute_row_shift_scale(const int64_t* ints_device, int64_t Q, int64_t d, int fixed_bits, float clip_k,
+                                    int32_t* shifts_device, float* scales_device, void* stream);
+int bsi_hip_compute_chunk_shift_scale(const int64_t* ints_device, int64_t Q, int64_t d, int chunks, int fixed_bits,
+                                      float clip_k, int32_t* shifts_device, float* scales_device, void* stream);
+
+/* In-place rounded right shift and clamp to fixed_bits.
+ * Replace launch_apply_row_shift_clamp / launch_apply_chunk_shift_clamp (quant.cuh:702-734). */
+int bsi_hip_apply_row_shift_clamp(int64_t* ints_device, int64_t Q, int64_t d, const int32_t* shifts_device,
+                                  int fixed_bits, void* stream);
+int bsi_hip_apply_chunk_shift_clamp(int64_t* ints_device, int64_t Q, int64_t d, int chunks,
+                                    const int32_t* shifts_device, int fixed_bits, void* stream);
+
+/* Same shift/scale rule computed straight from the float input (no int64 staging).
+ * Replace launch_compute_row_shift_scale_from_input / launch_compute_chunk_shift_scale_from_input
+ * (quant.cuh:490-557). */
+int bsi_hip_compute_row_shift_scale_from_input(const void* x_device, int dtype, int64_t Q, int64_t d, double dec_scale,
+                                               int fixed_bits, float clip_k, int32_t* shifts_device,
+                                               float* scales_device, void* stream);
+int bsi_hip_compute_chunk_shift_scale_from_input(const void* x_device, int dtype, int64_t Q, int64_t d, int chunks,
+                                                 double dec_scale, int fixed_bits, float clip_k,
+                                                 int32_t* shifts_device, float* scales_device, void* stream);
+
+/* Round, shift, clamp and pack into canonical words [Q, slices, words_per_slice] in one pass.
+ * Replace launch_quantize_shift_pack_row_batch / launch_quantize_shift_pack_chunk_batch
+ * (quant.cuh:559-636). */
+int bsi_hip_quantize_shift_pack_row_batch(const void* x_device, int dtype, int64_t Q, int64_t d, int slices,
+                                          int words_per_slice, double dec_scale, int fixed_bits,
+                                          const int32_t* shifts_device, uint64_t* words_device, void* stream);
+int bsi_hip_quantize_shift_pack_chunk_batch(const void* x_device, int dtype, int64_t Q, int64_t d, int chunks,
+                                            int slices, int words_per_slice, double dec_scale, int fixed_bits,
+                                            const int32_t* shifts_device, uint64_t* words_device, void* stream);
+
+/* int64 [Q, d] -> canonical words [Q, slices, words_per_slice] (low `slices` bits of each value).
+ * Replaces launch_pack_bits_all_ballot_batch / launch_pack_bits_all_ballot (Q = 1)
+ * (bsi_cuda_kernels_pack.cuh:176-230). */
+int bsi_hip_pack_bits_batch(const int64_t* ints_device, int64_t Q, int64_t d, int slices, int words_per_slice,
+                            uint64_t* words_device, void* stream);
+
+/* The whole fixed-bit build of a [Q, d] batch in one call: shift/scale pass + quantise/pack pass
+ * (one fused kernel when chunk_scale != 0).  chunk_scale != 0 gives shifts/scales [Q, ceil(d/256)],
+ * else [Q].  Optional extra output `ints8_device` (may be NULL): the quantised values as int8
+ * [Q, chunks*256] in the MFMA core's in-chunk element order (bsi_hip_planes_to_int8 gives the same).
+ * Replaces the host orchestration bsi_cuda_build_fixed_query_words_fused
+ * (bsi_vector_cuda.cpp:401-557) and, with chunk_scale = 0 and fixed_bits = 6, the key quantiser
+ * + packer (bsi_vector_cuda.cpp:559-744, 1125-1141). */
+int bsi_hip_build_fixed(const void* x_device, int dtype, int64_t Q, int64_t d, int decimal_places, int fixed_bits,
+                        int chunk_scale, float clip_k, uint64_t* words_device, int32_t* shifts_device,
+                        float* scales_device, int8_t* ints8_device, void* stream);
+
+/* ---------------------------------------------------------------- EWAH */
+
+/* counts[s] = popcount of slice s.  Replaces launch_slice_popcount_sum (ewah.cuh:71-81). */
+int bsi_hip_slice_popcount_sum(const uint64_t* words_device, int S, int W, uint64_t* counts_device, void* stream);
+/* flags[s] = (1 - (1-p)^128 - p^128 <= threshold), p = counts[s] / (64 W).
+ * Replaces launch_compress_flags_from_density (ewah.cuh:104-115). */
+int bsi_hip_compress_flags_from_density(const uint64_t* counts_device, int S, int W, double threshold,
+                                        int32_t* flags_device, void* stream);
+/* sizes[s] = number of u64 the encoder emits for slice s.  Replaces launch_ewah_size (ewah.cuh:164-175). */
+int bsi_hip_ewah_size(const uint64_t* words_device, int S, int W, const int32_t* flags_device,
+                      uint64_t* sizes_device, void* stream);
+/* Emit marker + literal words of every slice at off[s]; out_len[s] = words written.
+ * Marker = run_bit | run_len << 1 | literal_count << 33.  Replaces launch_ewah_emit (ewah.cuh:234-247). */
+int bsi_hip_ewah_emit(const uint64_t* words_device, int S, int W, const int32_t* flags_device,
+                      const uint64_t* off_device, uint64_t* out_device, int32_t* out_len_device, void* stream);
+/* One stream -> W literal words.  Replaces launch_ewah_decompress (ewah.cuh:35-42). */
+int bsi_hip_ewah_decompress(const uint64_t* in_device, int in_len, int W, uint64_t* out_device, void* stream);
+/* S streams (stream s at comp + off[s], len[s] words) -> canonical [S, W]; the batched form the
+ * hybrid query builder needs (the reference loops launch_ewah_decompress on the host,
+ * bsi_cuda.cpp:402-414). */
+int bsi_hip_ewah_decompress_batch(const uint64_t* comp_device, const int64_t* off_device, const int32_t* len_device,
+                                  int S, int W, uint64_t* out_device, void* stream);
+
+/* ---------------------------------------------------------------- dot */
+
+/* Permute canonical key words [R, Sb, W64] into the streaming layout of the MFMA core:
+ * word (r, j, 4c+g) goes to ((((r/16) * chunks + c) * Sb + j) * 64 + g*16 + r%16); rows past R and
+ * words past W64 are zero.  out must hold ceil(R/16)*16 * Sb * chunks*4 words.
+ * No counterpart in the reference (its kernels read the canonical layout through cp.async/TMA). */
+int bsi_hip_tile_key_planes(const uint64_t* words_device, int64_t R, int Sb, int W64, uint64_t* out_device,
+                            void* stream);
+
+/* Canonical planes [rows, S, W64] -> int8 [rows, chunks*256]: value << (8 - S), bytes of a chunk in
+ * the MFMA core's element order (element 32w + 8m + t of the chunk at byte 32w + 4t + m).
+ * No counterpart in the reference. */
+int bsi_hip_planes_to_int8(const uint64_t* words_device, int64_t rows, int S, int W64, int8_t* out_device,
+                           void* stream);
+
+/* Bytes of device workspace bsi_hip_dot needs for this shape and core (0 when none). */
+size_t bsi_hip_dot_workspace_bytes(int64_t Q, int W64, int core);
+
+/*
+ * The fixed-bit weighted-popcount dot, out[q, r] = scale_inv * chain_c fmaf((float)I[q,r,c],
+ * qscale[q,c] * Bw[r*Sb], acc), I[q,r,c] = sum_{i,j} +-(popc(A_i & B_j over chunk c) << (i+j)),
+ * negative iff (i == Sa-1) xor (j == Sb-1).
+ * Replaces launch_popcount_weighted_keys_literal_fused_multiq (bsi_cuda_kernels_dot.cuh:2616-3090)
+ * and through it the fixed76 chunk-scale kernels (:1285-2307).
+ *   A              canonical query words [Q, Sa, W64]
+ *   A_ints8        optional int8 [Q, chunks*256] from bsi_hip_build_fixed (NULL: derived from A
+ *                  into `workspace` when the MFMA core runs)
+ *   A_chunk_scales float [Q, A_scale_stride]; A_scale_stride == chunks for per-chunk scales,
+ *                  1 for one scale per row (broadcast over chunks)
+ *   B              key words in `b_layout`; Bw float [R, Sb] slice weights (only Bw[r*Sb] is read)
+ *   out            float [Q, R_total] (row stride R_total >= R); every element [q, r<R] is written
+ *   chunk_ints     optional int32 [Q, R, chunks]: the integer accumulators I (parity checks)
+ * Sa, Sb in [2, 8] for the MFMA core and [1, 16] for the VALU core.
+ */
+int bsi_hip_dot(const uint64_t* A, const int8_t* A_ints8, const float* A_chunk_scales, int A_scale_stride, int Sa,
+                int W64, const uint64_t* B, int b_layout, const float* Bw, int Sb, int64_t R, int64_t Q,
+                float scale_inv, int64_t R_total, float* out, int32_t* chunk_ints, int core, void* workspace,
+                size_t workspace_bytes, void* stream);
+
+/* Runs fn-independent timing of `iters` back-to-back bsi_hip_dot launches between two HIP events
+ * recorded on `stream`, synchronises, and returns the mean launch duration in microseconds.
+ * Mirrors the reference's BSI_PROFILE event pair (bsi_cuda.cpp:713-722,798-806). */
+int bsi_hip_dot_timed(const uint64_t* A, const int8_t* A_ints8, const float* A_chunk_scales, int A_scale_stride,
+                      int Sa, int W64, const uint64_t* B, int b_layout, const float* Bw, int Sb, int64_t R, int64_t Q,
+                      float scale_inv, int64_t R_total, float* out, int core, void* workspace, size_t workspace_bytes,
+                      int iters, float* mean_us, void* stream);
+
+/* Peak probes used by the benchmark to print measured next to published peaks: a pure
+ * v_and/v_bcnt loop (returns lane-ops per second), a pure v_mfma_i32_16x16x64_i8 loop (int8
+ * ops per second) and a streaming read (bytes per second).  Each synchronises. */
+int bsi_hip_probe_valu_popcount(double* lane_ops_per_s, void* stream);
+int bsi_hip_probe_mfma_i8(double* ops_per_s, void* stream);
+int bsi_hip_probe_stream_read(const void* buf_device, size_t bytes, double* bytes_per_s, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BSI_HIP_H */

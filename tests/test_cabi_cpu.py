@@ -1,0 +1,149 @@
+"""CPU-side checks of the C-ABI library and the host logic (no kernel is launched here)."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "bsi_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(bsi_hip_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from bsipytorch_amd import _lib
+
+    names = _declared_symbols()
+    assert len(names) >= 25
+    raw = ctypes.CDLL(_lib.LIB_PATH)
+    for n in names:
+        assert hasattr(raw, n), f"libbsi_hip.so does not export {n}"
+    assert set(names) == set(_lib.PROTOTYPES), set(names) ^ set(_lib.PROTOTYPES)
+    assert "gfx950" in _lib.version()
+
+
+def test_argument_validation_returns_error_codes():
+    from bsipytorch_amd import _lib
+
+    L = _lib.lib
+    # W64 = 0 is rejected before anything touches the device
+    rc = L.bsi_hip_dot(None, None, None, 8, 7, 0, None, 0, None, 6, 4, 4, 1.0, 4, None, None, 0, None, 0, None)
+    assert rc == 1 and b"W64" in L.bsi_hip_last_error()
+    rc = L.bsi_hip_dot(None, None, None, 8, 7, 32, None, 0, None, 6, 4, -1, 1.0, 4, None, None, 0, None, 0, None)
+    assert rc == 1
+    # stride must be chunks or 1
+    rc = L.bsi_hip_dot(1, None, 1, 3, 7, 32, 1, 0, 1, 6, 4, 4, 1.0, 4, 1, None, 0, None, 0, None)
+    assert rc == 1 and b"stride" in L.bsi_hip_last_error()
+    rc = L.bsi_hip_dot(1, None, 1, 8, 7, 32, 1, 0, 1, 6, 8, 4, 1.0, 4, 1, None, 0, None, 0, None)
+    assert rc == 1 and b"R_total" in L.bsi_hip_last_error()
+    rc = L.bsi_hip_build_fixed(None, 0, 4, 4, 2, 1, 1, 0.0, None, None, None, None, None)
+    assert rc == 1 and b"fixed_bits" in L.bsi_hip_last_error()
+    rc = L.bsi_hip_planes_to_int8(None, 4, 9, 4, None, None)
+    assert rc == 1
+    # empty problems are fine and launch nothing
+    assert L.bsi_hip_dot(None, None, None, 8, 7, 32, None, 0, None, 6, 0, 0, 1.0, 0, None, None, 0, None, 0, None) == 0
+    assert L.bsi_hip_build_fixed(None, 0, 0, 128, 2, 7, 1, 0.0, None, None, None, None, None) == 0
+    assert L.bsi_hip_dot_workspace_bytes(512, 32, _lib.CORE_MFMA) == 512 * 8 * 256
+    assert L.bsi_hip_dot_workspace_bytes(512, 32, _lib.CORE_VALU) == 0
+    with pytest.raises(_lib.BsiHipError):
+        _lib.check(rc=1, what="x")
+
+
+def test_flags_defaults_and_overrides(monkeypatch):
+    from bsipytorch_amd import bsi_ops
+
+    for k in list(os.environ):
+        if k.startswith("BSI_"):
+            monkeypatch.delenv(k)
+    bsi_ops._reset_flag_cache()
+    f = dict(bsi_ops._flags())
+    assert (f["bits_q"], f["bits_k"], f["chunk_scale"], f["clip_k"], f["profile"]) == (7, 6, True, 0.0, False)
+    monkeypatch.setenv("BSI_FIXED_BITS", "5")
+    monkeypatch.setenv("BSI_FIXED_BITS_KEYS", "1")   # clamped up to 2
+    monkeypatch.setenv("BSI_FIXED_CHUNK_SCALE", "0")
+    monkeypatch.setenv("BSI_FIXED_CLIP_K", "6.5")
+    monkeypatch.setenv("BSI_DOT_CORE", "valu")
+    bsi_ops._reset_flag_cache()
+    f = dict(bsi_ops._flags())
+    assert (f["bits_q"], f["bits_k"], f["chunk_scale"], f["clip_k"]) == (5, 2, False, 6.5)
+    assert f["core"] == 1
+    monkeypatch.setenv("BSI_FIXED_BITS_QUERIES", "0")
+    bsi_ops._reset_flag_cache()
+    assert bsi_ops._flags()["bits_q"] == 0
+    with pytest.raises(RuntimeError):
+        bsi_ops._require_fixed(0, "x")
+    for k in ("BSI_FIXED_BITS", "BSI_FIXED_BITS_KEYS", "BSI_FIXED_CHUNK_SCALE", "BSI_FIXED_CLIP_K", "BSI_DOT_CORE",
+              "BSI_FIXED_BITS_QUERIES"):
+        monkeypatch.delenv(k)
+    bsi_ops._reset_flag_cache()
+
+
+def test_module_surface_matches_reference_names():
+    import bsi_ops  # the drop-in name
+
+    gpu = ["build_bsi_keys_cuda", "build_bsi_queries_cuda_batch_packed", "build_bsi_queries_cuda_batch",
+           "build_bsi_query_cuda", "build_bsi_query_cuda_hybrid", "batch_dot_product_multiquery_cuda_batch_caps",
+           "batch_dot_product_multiquery_cuda_caps", "bsi_keys_cuda_stats", "bsi_query_caps_stats",
+           "get_last_query_build_profile_cuda", "reset_last_query_build_profile_cuda", "cuda_builder_version"]
+    cpu = ["dot_product", "dot_product_decimal", "vector_dot_product", "vector_dot_product_no_precison",
+           "random_number_dot_product_vector", "random_number_dot_product_bsi", "batch_dot_product", "build_bsi_keys",
+           "build_bsi_query", "batch_dot_product_prebuilt", "batch_dot_product_prebuilt_capsule",
+           "keyset_slice_stats", "tensor_slice_stats", "keyset_size_on_disk", "save_keyset", "debug_bsi_query_words"]
+    for n in gpu + cpu + ["debug_quantize_int64_cpu", "CUDA_BUILDER_VERSION"]:
+        assert hasattr(bsi_ops, n), n
+    for n in cpu:
+        with pytest.raises(RuntimeError, match="bsiCPP"):
+            getattr(bsi_ops, n)(torch.zeros(2), torch.zeros(2))
+    assert bsi_ops.get_last_query_build_profile_cuda() == (0, 0, 0)
+    assert bsi_ops.PrebuiltBSIKeysCUDA.name == "PrebuiltBSIKeysCUDA"
+    assert bsi_ops.PrebuiltBSIQueryBatchCUDA.name == "PrebuiltBSIQueryBatchCUDA"
+    assert bsi_ops.PrebuiltBSIQueryCUDA.name == "PrebuiltBSIQueryCUDA"
+
+
+def test_debug_quantize_cpu_matches_oracle(oracle):
+    from bsipytorch_amd import bsi_ops
+
+    rng = np.random.default_rng(0)
+    x = np.concatenate([rng.standard_normal(500), [0.005, -0.005, 0.125, -2.675, 1e-7]]).astype(np.float32)
+    for dec in (0, 2, 3):
+        got = bsi_ops.debug_quantize_int64_cpu(torch.from_numpy(x), dec).numpy()
+        np.testing.assert_array_equal(got, oracle.round_to_int64(x, dec))
+
+
+def test_slice_weights_host(oracle):
+    from bsipytorch_amd import bsi_ops
+
+    for S, off, twos in [(7, 0, True), (6, 0, True), (4, 0, False), (3, 2, True)]:
+        got = bsi_ops._slice_weights(S, off, twos, "cpu").numpy()
+        np.testing.assert_array_equal(got, oracle.slice_weights(S, off, twos))
+
+
+def test_dot_error_paths_on_host():
+    from bsipytorch_amd import bsi_ops
+
+    with pytest.raises(RuntimeError, match="Invalid CUDA keys capsule"):
+        bsi_ops.batch_dot_product_multiquery_cuda_batch_caps(object(), object())
+    keys = bsi_ops.PrebuiltBSIKeysCUDA()
+    with pytest.raises(RuntimeError, match="Invalid CUDA query-batch capsule"):
+        bsi_ops.batch_dot_product_multiquery_cuda_batch_caps(bsi_ops.PrebuiltBSIQueryCUDA(), keys)
+    qb = bsi_ops.PrebuiltBSIQueryBatchCUDA()
+    with pytest.raises(RuntimeError, match="not defined"):
+        bsi_ops.batch_dot_product_multiquery_cuda_batch_caps(qb, keys)
+    qb.words = torch.zeros(2, 7, 4, dtype=torch.int64)
+    qb.slice_weights = torch.zeros(2, 7)
+    with pytest.raises(RuntimeError, match="must be CUDA tensors"):
+        bsi_ops.batch_dot_product_multiquery_cuda_batch_caps(qb, keys)
+    with pytest.raises(RuntimeError, match="Empty keys or queries"):
+        bsi_ops.batch_dot_product_multiquery_cuda_caps([], keys)
+    with pytest.raises(RuntimeError, match="2D"):
+        bsi_ops.build_bsi_queries_cuda_batch_packed(torch.zeros(4), 2)
+    with pytest.raises(RuntimeError, match="2D"):
+        bsi_ops.build_bsi_keys_cuda(torch.zeros(4), 2)
+    with pytest.raises(RuntimeError, match="1D"):
+        bsi_ops.build_bsi_query_cuda(torch.zeros(4, 4), 2)

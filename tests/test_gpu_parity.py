@@ -1,0 +1,568 @@
+"""GPU parity: every HIP kernel against the CPU oracle on the same seeded inputs, through the C ABI
+(raw entry points) and through the ``bsi_ops`` mirror.  Integer and bit work must be bit-exact; the
+fp32 output is compared bit-for-bit as well (same chunk order, fused multiply-add, power-of-two
+scales), with the 1e-5 relative tolerance of the specification as the stated bar.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "reference_known_answers.json")
+FP32_RTOL = 1e-5  # stated tolerance for the fp32 outputs; the asserts below ask for exact equality first
+
+
+@pytest.fixture(scope="module")
+def hip():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from bsipytorch_amd import _lib
+
+    return _lib
+
+
+@pytest.fixture()
+def ops(monkeypatch):
+    from bsipytorch_amd import bsi_ops
+
+    for k in list(os.environ):
+        if k.startswith("BSI_"):
+            monkeypatch.delenv(k)
+    bsi_ops._reset_flag_cache()
+    yield bsi_ops
+    bsi_ops._reset_flag_cache()
+
+
+def dev(a: np.ndarray) -> torch.Tensor:
+    if a.dtype == np.uint64:
+        a = a.view(np.int64)
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host_u64(t: torch.Tensor) -> np.ndarray:
+    return t.detach().cpu().numpy().view(np.uint64)
+
+
+def st():
+    return torch.cuda.current_stream().cuda_stream
+
+
+# ------------------------------------------------------------------ builder
+
+
+def _inputs(Q, d, seed, kind="randn"):
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((Q, d)).astype(np.float32)
+    if kind == "outliers":
+        cols = rng.permutation(d)[: max(1, d // 1000)]
+        x[:, cols] *= 20.0
+    elif kind == "relu":
+        x = np.maximum(x, 0)
+    elif kind == "small":
+        x *= np.float32(0.02)
+    elif kind == "ties":
+        x = (rng.integers(-3000, 3000, size=(Q, d)) / 200.0).astype(np.float32)  # many x.5 after *100
+    if Q > 2 and d >= 256:
+        x[1, :256] = 0.0       # an all-zero chunk
+        x[2, 5] = 655.35       # a large outlier
+    return x
+
+
+@pytest.mark.parametrize("Q,d,kind", [(64, 2048, "randn"), (33, 2048, "outliers"), (17, 8192, "relu"),
+                                      (5, 256, "ties"), (9, 700, "randn"), (3, 64, "small"), (4, 1000, "ties")])
+@pytest.mark.parametrize("bits,chunk", [(7, True), (6, False), (8, True), (4, False)])
+def test_build_fixed_matches_oracle(hip, oracle, Q, d, kind, bits, chunk):
+    x = _inputs(Q, d, seed=Q * 7 + d, kind=kind)
+    ints, shifts, scales = oracle.quantize_fixed(x, 2, bits, chunk)
+    want_words = oracle.pack(ints, bits)
+    W = (d + 63) // 64
+    chunks = (d + 255) // 256
+    xd = dev(x)
+    words = torch.zeros((Q, bits, W), dtype=torch.int64, device="cuda")
+    sh = torch.zeros(shifts.shape, dtype=torch.int32, device="cuda")
+    sc = torch.zeros(scales.shape, dtype=torch.float32, device="cuda")
+    i8 = torch.full((Q, chunks * 256), 77, dtype=torch.int8, device="cuda")
+    hip.check(hip.lib.bsi_hip_build_fixed(xd.data_ptr(), 0, Q, d, 2, bits, int(chunk), 0.0, words.data_ptr(),
+                                          sh.data_ptr(), sc.data_ptr(), i8.data_ptr(), st()), "build")
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(sh.cpu().numpy(), shifts)
+    np.testing.assert_array_equal(sc.cpu().numpy(), scales)
+    np.testing.assert_array_equal(host_u64(words), want_words)
+    # int8 operand: value << (8 - bits), element 32w + 8m + t of a chunk at byte 32w + 4t + m
+    padded = np.zeros((Q, chunks * 256), dtype=np.int64)
+    padded[:, :d] = ints
+    e = np.arange(chunks * 256)
+    pos = (e // 32) * 32 + ((e % 32) % 8) * 4 + (e % 32) // 8
+    want8 = np.zeros_like(padded)
+    want8[:, pos] = padded << (8 - bits)
+    np.testing.assert_array_equal(i8.cpu().numpy().astype(np.int64), want8)
+    # the planes -> int8 pre-pass gives the same bytes
+    i8b = torch.zeros_like(i8)
+    hip.check(hip.lib.bsi_hip_planes_to_int8(words.data_ptr(), Q, bits, W, i8b.data_ptr(), st()), "p2i8")
+    torch.cuda.synchronize()
+    assert torch.equal(i8, i8b)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_build_half_inputs(hip, oracle, dtype):
+    x = torch.from_numpy(_inputs(12, 1024, 5)).to(dtype)
+    ref = x.to(torch.float32).numpy()
+    ints, shifts, scales = oracle.quantize_fixed(ref, 2, 7, True)
+    xd = x.cuda()
+    words = torch.zeros((12, 7, 16), dtype=torch.int64, device="cuda")
+    sh = torch.zeros((12, 4), dtype=torch.int32, device="cuda")
+    sc = torch.zeros((12, 4), dtype=torch.float32, device="cuda")
+    code = 1 if dtype == torch.float16 else 2
+    hip.check(hip.lib.bsi_hip_build_fixed(xd.data_ptr(), code, 12, 1024, 2, 7, 1, 0.0, words.data_ptr(), sh.data_ptr(),
+                                          sc.data_ptr(), None, st()), "build")
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(sh.cpu().numpy(), shifts)
+    np.testing.assert_array_equal(host_u64(words), oracle.pack(ints, 7))
+
+
+def test_build_clip_k(hip, oracle):
+    x = _inputs(8, 1024, 3, "outliers")
+    for chunk in (True, False):
+        ints, shifts, scales = oracle.quantize_fixed(x, 2, 7, chunk, clip_k=6.0)
+        assert (shifts != oracle.quantize_fixed(x, 2, 7, chunk)[1]).any()  # clipping changes something
+        xd = dev(x)
+        words = torch.zeros((8, 7, 16), dtype=torch.int64, device="cuda")
+        sh = torch.zeros(shifts.shape, dtype=torch.int32, device="cuda")
+        sc = torch.zeros(scales.shape, dtype=torch.float32, device="cuda")
+        hip.check(hip.lib.bsi_hip_build_fixed(xd.data_ptr(), 0, 8, 1024, 2, 7, int(chunk), 6.0, words.data_ptr(),
+                                              sh.data_ptr(), sc.data_ptr(), None, st()), "build")
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(sh.cpu().numpy(), shifts)
+        np.testing.assert_array_equal(host_u64(words), oracle.pack(ints, 7))
+
+
+@pytest.mark.parametrize("Q,d", [(7, 2048), (5, 700), (3, 100)])
+def test_staged_builder_entry_points(hip, oracle, Q, d):
+    """The separate passes the reference exposes: round -> shift/scale -> shift+clamp -> pack."""
+    L = hip.lib
+    x = _inputs(Q, d, 11, "outliers")
+    xd = dev(x)
+    W = (d + 63) // 64
+    chunks = (d + 255) // 256
+    r = torch.zeros((Q, d), dtype=torch.int64, device="cuda")
+    hip.check(L.bsi_hip_quantize_round_to_int64(xd.data_ptr(), 0, Q * d, 100.0, r.data_ptr(), st()), "round")
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(r.cpu().numpy(), oracle.round_to_int64(x, 2))
+    for chunk in (True, False):
+        ints, shifts, scales = oracle.quantize_fixed(x, 2, 7, chunk)
+        sh = torch.zeros(shifts.shape, dtype=torch.int32, device="cuda")
+        sc = torch.zeros(scales.shape, dtype=torch.float32, device="cuda")
+        sh2, sc2 = torch.zeros_like(sh), torch.zeros_like(sc)
+        if chunk:
+            hip.check(L.bsi_hip_compute_chunk_shift_scale(r.data_ptr(), Q, d, chunks, 7, 0.0, sh.data_ptr(), sc.data_ptr(), st()), "css")
+            hip.check(L.bsi_hip_compute_chunk_shift_scale_from_input(xd.data_ptr(), 0, Q, d, chunks, 100.0, 7, 0.0,
+                                                                     sh2.data_ptr(), sc2.data_ptr(), st()), "cssi")
+        else:
+            hip.check(L.bsi_hip_compute_row_shift_scale(r.data_ptr(), Q, d, 7, 0.0, sh.data_ptr(), sc.data_ptr(), st()), "rss")
+            hip.check(L.bsi_hip_compute_row_shift_scale_from_input(xd.data_ptr(), 0, Q, d, 100.0, 7, 0.0,
+                                                                   sh2.data_ptr(), sc2.data_ptr(), st()), "rssi")
+        torch.cuda.synchronize()
+        for a, b in ((sh, sc), (sh2, sc2)):
+            np.testing.assert_array_equal(a.cpu().numpy(), shifts)
+            np.testing.assert_array_equal(b.cpu().numpy(), scales)
+        q = r.clone()
+        if chunk:
+            hip.check(L.bsi_hip_apply_chunk_shift_clamp(q.data_ptr(), Q, d, chunks, sh.data_ptr(), 7, st()), "acsc")
+        else:
+            hip.check(L.bsi_hip_apply_row_shift_clamp(q.data_ptr(), Q, d, sh.data_ptr(), 7, st()), "arsc")
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(q.cpu().numpy(), ints)
+        words = torch.zeros((Q, 7, W), dtype=torch.int64, device="cuda")
+        hip.check(L.bsi_hip_pack_bits_batch(q.data_ptr(), Q, d, 7, W, words.data_ptr(), st()), "pack")
+        words2 = torch.zeros_like(words)
+        if chunk:
+            hip.check(L.bsi_hip_quantize_shift_pack_chunk_batch(xd.data_ptr(), 0, Q, d, chunks, 7, W, 100.0, 7,
+                                                                sh.data_ptr(), words2.data_ptr(), st()), "qspc")
+        else:
+            hip.check(L.bsi_hip_quantize_shift_pack_row_batch(xd.data_ptr(), 0, Q, d, 7, W, 100.0, 7, sh.data_ptr(),
+                                                              words2.data_ptr(), st()), "qspr")
+        torch.cuda.synchronize()
+        want = oracle.pack(ints, 7)
+        np.testing.assert_array_equal(host_u64(words), want)
+        np.testing.assert_array_equal(host_u64(words2), want)
+
+
+# ------------------------------------------------------------------ EWAH
+
+
+def _ewah_planes(seed, S=14, W=96):
+    rng = np.random.default_rng(seed)
+    words = rng.integers(0, 2 ** 63, size=(S, W)).astype(np.uint64)
+    words[0] = 0
+    words[1] = np.uint64(0xFFFFFFFFFFFFFFFF)
+    words[2, rng.random(W) < 0.8] = 0
+    words[3, rng.random(W) < 0.8] = np.uint64(0xFFFFFFFFFFFFFFFF)
+    words[4, 5:50] = 0
+    words[4, 50:60] = np.uint64(0xFFFFFFFFFFFFFFFF)
+    words[5] = 0
+    words[5, 17] = 4096  # 1 bit of 6144: density below the 0.54% cut
+    return words
+
+
+@pytest.mark.parametrize("seed", [0, 1])
+def test_ewah_kernels_match_oracle(hip, oracle, seed):
+    L = hip.lib
+    words = _ewah_planes(seed)
+    S, W = words.shape
+    wd = dev(words)
+    counts = torch.zeros((S,), dtype=torch.int64, device="cuda")
+    hip.check(L.bsi_hip_slice_popcount_sum(wd.data_ptr(), S, W, counts.data_ptr(), st()), "pop")
+    torch.cuda.synchronize()
+    want_counts = np.array([sum(bin(int(v)).count("1") for v in row) for row in words])
+    np.testing.assert_array_equal(counts.cpu().numpy(), want_counts)
+    for thr in (0.5, 0.0, 1.0):
+        flags = torch.zeros((S,), dtype=torch.int32, device="cuda")
+        hip.check(L.bsi_hip_compress_flags_from_density(counts.data_ptr(), S, W, thr, flags.data_ptr(), st()), "flags")
+        torch.cuda.synchronize()
+        want_flags = oracle.compress_flags(words, thr)
+        np.testing.assert_array_equal(flags.cpu().numpy(), want_flags)
+        stream, off, lens = oracle.ewah_encode(words, want_flags)
+        sizes = torch.zeros((S,), dtype=torch.int64, device="cuda")
+        hip.check(L.bsi_hip_ewah_size(wd.data_ptr(), S, W, flags.data_ptr(), sizes.data_ptr(), st()), "size")
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(sizes.cpu().numpy(), lens)
+        offd = dev(off)
+        out = torch.zeros((stream.size,), dtype=torch.int64, device="cuda")
+        out_len = torch.zeros((S,), dtype=torch.int32, device="cuda")
+        hip.check(L.bsi_hip_ewah_emit(wd.data_ptr(), S, W, flags.data_ptr(), offd.data_ptr(), out.data_ptr(),
+                                      out_len.data_ptr(), st()), "emit")
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(host_u64(out), stream)
+        np.testing.assert_array_equal(out_len.cpu().numpy(), lens)
+        back = torch.full((S, W), -1, dtype=torch.int64, device="cuda")
+        hip.check(L.bsi_hip_ewah_decompress_batch(out.data_ptr(), offd.data_ptr(), out_len.data_ptr(), S, W,
+                                                  back.data_ptr(), st()), "decode")
+        one = torch.full((W,), -1, dtype=torch.int64, device="cuda")
+        hip.check(L.bsi_hip_ewah_decompress(out.data_ptr() + 8 * int(off[4]), int(lens[4]), W, one.data_ptr(), st()), "decode1")
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(host_u64(back), words)
+        np.testing.assert_array_equal(host_u64(one), words[4])
+
+
+def test_hybrid_query_builder(ops, oracle):
+    x = np.maximum(_inputs(1, 8192, 4), 0)[0]  # ReLU: sign plane all zero
+    cap, mem, S, W = ops.build_bsi_query_cuda_hybrid(torch.from_numpy(x).cuda(), 2, 0.5)
+    cap2, mem2, S2, W2 = ops.build_bsi_query_cuda(torch.from_numpy(x).cuda(), 2, 0.5)
+    torch.cuda.synchronize()
+    assert (S, W) == (7, 128) == (S2, W2)
+    assert torch.equal(cap.dev_words, cap2.dev_words)  # decode(encode(x)) == x
+    ints, shifts, scales = oracle.quantize_fixed(x[None], 2, 7, False)
+    planes = oracle.pack(ints, 7)[0]
+    np.testing.assert_array_equal(host_u64(cap.dev_words), planes)
+    stream, off, lens = oracle.ewah_encode(planes, oracle.compress_flags(planes, 0.5))
+    np.testing.assert_array_equal(host_u64(cap.comp_words), stream)
+    np.testing.assert_array_equal(cap.comp_len.cpu().numpy(), lens)
+    assert lens[6] == 1 and mem == (stream.size + 7 * 128) * 8 and mem2 == 7 * 128 * 8
+    assert not cap2.twos_complement and float(cap.slice_weights[0]) == float(scales[0])
+
+
+# ------------------------------------------------------------------ dot through the raw C ABI
+
+
+def _oracle_case(oracle, Q, R, d, seed, qkind="randn", ksigma=0.02, bits_q=7, bits_k=6):
+    x = _inputs(Q, d, seed, qkind)
+    rng = np.random.default_rng(seed + 1000)
+    k = (rng.standard_normal((R, d)) * ksigma).astype(np.float32)
+    if R > 3:
+        k[3] *= 50  # one row with a large key shift
+    qb = oracle.build_queries(x, 2, bits_q)
+    kb = oracle.build_keys(k, 2, bits_k)
+    ints, out = oracle.dot_fixed(qb["words"], qb["scales"], kb["words"], kb["scales"], oracle.scale_inv(2, 2))
+    return x, k, qb, kb, ints, out
+
+
+def _run_dot(hip, qb, kb, Q, R, W, Sa, Sb, core, tiled, with_ints8, want_ints=True, R_total=None):
+    L = hip.lib
+    chunks = (W + 3) // 4
+    A = dev(qb["words"])
+    scales = dev(qb["scales"])
+    stride = chunks if qb["chunk_scale"] else 1
+    B = dev(kb["words"])
+    layout = 0
+    if tiled:
+        Bt = torch.full((((R + 15) // 16) * chunks * Sb * 64,), -1, dtype=torch.int64, device="cuda")
+        hip.check(L.bsi_hip_tile_key_planes(B.data_ptr(), R, Sb, W, Bt.data_ptr(), st()), "tile")
+        B, layout = Bt, 1
+    Bw = dev(kb["slice_weights"])
+    a8 = None
+    if with_ints8:
+        a8 = torch.zeros((Q, chunks * 256), dtype=torch.int8, device="cuda")
+        hip.check(L.bsi_hip_planes_to_int8(A.data_ptr(), Q, Sa, W, a8.data_ptr(), st()), "p2i8")
+    R_total = R if R_total is None else R_total
+    out = torch.full((Q, R_total), float("nan"), dtype=torch.float32, device="cuda")
+    ints = torch.full((Q, R, chunks), -7, dtype=torch.int32, device="cuda") if want_ints else None
+    ws_bytes = int(L.bsi_hip_dot_workspace_bytes(Q, W, core))
+    ws = torch.zeros((max(ws_bytes, 16),), dtype=torch.uint8, device="cuda")
+    hip.check(L.bsi_hip_dot(A.data_ptr(), a8.data_ptr() if a8 is not None else None, scales.data_ptr(), stride, Sa, W,
+                            B.data_ptr(), layout, Bw.data_ptr(), Sb, R, Q, float(np.float32(1e-4)), R_total,
+                            out.data_ptr(), ints.data_ptr() if ints is not None else None, core, ws.data_ptr(),
+                            ws_bytes, st()), "dot")
+    torch.cuda.synchronize()
+    return (ints.cpu().numpy() if ints is not None else None), out.cpu().numpy()
+
+
+DOT_SHAPES = [
+    (64, 256, 2048, "randn"),     # the correctness-scale configuration
+    (37, 75, 2048, "outliers"),   # ragged Q and R
+    (130, 129, 512, "relu"),      # tile edges on both sides, ReLU queries
+    (5, 3, 256, "ties"),          # a single chunk
+    (16, 40, 700, "randn"),       # W64 = 11: row scale, partial last chunk
+    (1, 200, 4096, "randn"),      # a single query
+]
+
+
+@pytest.mark.parametrize("Q,R,d,kind", DOT_SHAPES)
+@pytest.mark.parametrize("core,tiled,ints8", [(1, False, False), (1, True, False), (2, False, True), (2, True, False),
+                                              (0, True, True)])
+def test_dot_bit_exact(hip, oracle, Q, R, d, kind, core, tiled, ints8):
+    x, k, qb, kb, want_ints, want_out = _oracle_case(oracle, Q, R, d, seed=Q + R + d, qkind=kind)
+    W = (d + 63) // 64
+    ints, out = _run_dot(hip, qb, kb, Q, R, W, 7, 6, core, tiled, ints8)
+    np.testing.assert_array_equal(ints, want_ints)                     # integer accumulators: bit-exact
+    np.testing.assert_allclose(out, want_out, rtol=FP32_RTOL, atol=0)  # the stated fp32 bar
+    np.testing.assert_array_equal(out, want_out)                       # and in fact identical
+    # independent of the popcount form: the accumulators are the integer dot of the quantised values
+    c0 = qb["ints"][:, :256] @ kb["ints"][:, :256].T
+    np.testing.assert_array_equal(ints[:, :, 0], c0)
+
+
+@pytest.mark.parametrize("Sa,Sb", [(8, 8), (5, 4), (2, 2), (7, 5), (3, 7)])
+@pytest.mark.parametrize("core", [1, 2])
+def test_dot_other_bit_widths(hip, oracle, Sa, Sb, core):
+    Q, R, d = 19, 35, 1024
+    x, k, qb, kb, want_ints, want_out = _oracle_case(oracle, Q, R, d, seed=Sa * 10 + Sb, ksigma=0.05, bits_q=Sa, bits_k=Sb)
+    ints, out = _run_dot(hip, qb, kb, Q, R, 16, Sa, Sb, core, tiled=(core == 2), with_ints8=False)
+    np.testing.assert_array_equal(ints, want_ints)
+    np.testing.assert_array_equal(out, want_out)
+
+
+def test_dot_wide_planes_valu_only(hip, oracle):
+    Q, R, d = 6, 10, 512
+    x, k, qb, kb, want_ints, want_out = _oracle_case(oracle, Q, R, d, seed=99, ksigma=0.5, bits_q=12, bits_k=10)
+    ints, out = _run_dot(hip, qb, kb, Q, R, 8, 12, 10, 0, tiled=False, with_ints8=False)  # auto -> VALU
+    np.testing.assert_array_equal(ints, want_ints)
+    np.testing.assert_array_equal(out, want_out)
+    L = hip.lib
+    t = torch.zeros(8, device="cuda")
+    rc = L.bsi_hip_dot(t.data_ptr(), None, t.data_ptr(), 2, 12, 8, t.data_ptr(), 0, t.data_ptr(), 10, 1, 1, 1.0, 1,
+                       t.data_ptr(), None, 2, None, 0, st())
+    assert rc == 3 and b"MFMA core needs" in L.bsi_hip_last_error()
+
+
+def test_dot_extreme_values(hip, oracle):
+    # every product at its largest magnitude: I = 2^19 per chunk, both signs
+    Q, R, d = 4, 6, 1024
+    a = np.full((Q, d), -64, dtype=np.int64)
+    a[1] = 63
+    b = np.full((R, d), -32, dtype=np.int64)
+    b[2] = 31
+    qb = dict(words=oracle.pack(a, 7), scales=np.full((Q, 4), 8, np.float32), chunk_scale=True)
+    kb = dict(words=oracle.pack(b, 6), slice_weights=(oracle.slice_weights(6)[None] * np.ones((R, 1), np.float32)))
+    want_ints, want_out = oracle.dot_fixed(qb["words"], qb["scales"], kb["words"], np.ones(R, np.float32), np.float32(1e-4))
+    assert want_ints.max() == 1 << 19
+    for core in (1, 2):
+        ints, out = _run_dot(hip, qb, kb, Q, R, 16, 7, 6, core, tiled=True, with_ints8=False)
+        np.testing.assert_array_equal(ints, want_ints)
+        np.testing.assert_array_equal(out, want_out)
+
+
+def test_dot_fp32_rounding_order(hip, oracle):
+    # 40 chunks of same-sign products with mixed scales: the fp32 accumulator rounds, so only the
+    # reference's chunk order reproduces the bits
+    rng = np.random.default_rng(11)
+    Q, R, d = 8, 24, 256 * 40
+    a = rng.integers(40, 64, size=(Q, d)).astype(np.int64)
+    b = rng.integers(20, 32, size=(R, d)).astype(np.int64)
+    a[1] = -a[1]
+    qb = dict(words=oracle.pack(a, 7), scales=(2.0 ** rng.integers(0, 8, size=(Q, 40))).astype(np.float32), chunk_scale=True)
+    bscale = (2.0 ** rng.integers(0, 5, size=R)).astype(np.float32)
+    kb = dict(words=oracle.pack(b, 6), slice_weights=(oracle.slice_weights(6)[None] * bscale[:, None]).astype(np.float32))
+    want_ints, want_out = oracle.dot_fixed(qb["words"], qb["scales"], kb["words"], bscale, np.float32(1e-4))
+    for core in (1, 2):
+        ints, out = _run_dot(hip, qb, kb, Q, R, 160, 7, 6, core, tiled=False, with_ints8=True)
+        np.testing.assert_array_equal(ints, want_ints)
+        np.testing.assert_array_equal(out, want_out)
+
+
+def test_dot_row_stride_and_untouched_columns(hip, oracle):
+    Q, R, d = 10, 20, 512
+    x, k, qb, kb, want_ints, want_out = _oracle_case(oracle, Q, R, d, seed=5)
+    for core in (1, 2):
+        _, out = _run_dot(hip, qb, kb, Q, R, 8, 7, 6, core, tiled=True, with_ints8=False, want_ints=False, R_total=27)
+        np.testing.assert_array_equal(out[:, :R], want_out)
+        assert np.isnan(out[:, R:]).all()  # columns past R are not written
+
+
+# ------------------------------------------------------------------ through the bsi_ops mirror
+
+
+def test_reference_known_answers_gpu(ops, monkeypatch):
+    kat = json.load(open(GOLDEN))
+    for case in kat["vector_dot"] + kat["batch_dot"]:
+        monkeypatch.setenv("BSI_FIXED_BITS_KEYS", str(case["key_bits"]))
+        ops._reset_flag_cache()
+        q = torch.tensor(case["q"] if "K" in case else [case["q"]], dtype=torch.float32)
+        K = torch.tensor(case["K"] if "K" in case else [case["k"]], dtype=torch.float32)
+        dec = case["decimal_places"]
+        kcap, nbytes, nk, d, W = ops.build_bsi_keys_cuda(K, dec, 0.2)
+        assert (nk, d, W) == (K.shape[0], K.shape[1], 1) and nbytes == nk * case["key_bits"] * 8
+        qcap = ops.build_bsi_queries_cuda_batch_packed(q.cuda(), dec, 0.2)
+        out, ns, ns_q, ns_s = ops.batch_dot_product_multiquery_cuda_batch_caps(qcap, kcap)
+        want = torch.tensor(case["expected"], dtype=torch.float32).reshape(out.shape)
+        assert torch.equal(out.cpu(), want), case["cite"]
+        assert (ns, ns_q, ns_s) == (0, 0.0, 0.0)  # BSI_PROFILE unset
+        rows = ops.build_bsi_queries_cuda_batch(q.cuda(), dec, 0.2)
+        out2, *_ = ops.batch_dot_product_multiquery_cuda_caps(rows, kcap)
+        assert torch.equal(out2, out)
+
+
+@pytest.mark.parametrize("layout", ["tiled", "canonical"])
+@pytest.mark.parametrize("core", ["mfma", "valu"])
+def test_ops_pipeline_matches_oracle_c1(ops, oracle, monkeypatch, layout, core):
+    monkeypatch.setenv("BSI_KEY_LAYOUT", layout)
+    monkeypatch.setenv("BSI_DOT_CORE", core)
+    ops._reset_flag_cache()
+    torch.manual_seed(123)
+    Q, R, D = 64, 256, 2048
+    K = torch.randn(R, D) * 0.02
+    X = torch.randn(Q, D)
+    kcap, nbytes, nk, d, W = ops.build_bsi_keys_cuda(K, 2, 0.5)
+    assert (nbytes, nk, d, W) == (R * 6 * 32 * 8, R, D, 32)
+    qcap = ops.build_bsi_queries_cuda_batch_packed(X.cuda(), 2, 0.5)
+    out, *_ = ops.batch_dot_product_multiquery_cuda_batch_caps(qcap, kcap)
+    ints, out_dbg = ops.debug_chunk_ints(qcap, kcap, core)
+    qb, kb = oracle.build_queries(X.numpy()), oracle.build_keys(K.numpy())
+    want_ints, want_out = oracle.dot_fixed(qb["words"], qb["scales"], kb["words"], kb["scales"], oracle.scale_inv(2, 2))
+    np.testing.assert_array_equal(host_u64(qcap.words), qb["words"])
+    np.testing.assert_array_equal(qcap.chunk_scales.cpu().numpy(), qb["scales"])
+    np.testing.assert_array_equal(kcap.slice_weights.cpu().numpy(), kb["slice_weights"])
+    np.testing.assert_array_equal(qcap.slice_weights.cpu().numpy(), np.tile(oracle.slice_weights(7), (Q, 1)))
+    np.testing.assert_array_equal(ints.cpu().numpy(), want_ints)
+    np.testing.assert_array_equal(out.cpu().numpy(), want_out)
+    np.testing.assert_array_equal(out_dbg.cpu().numpy(), want_out)
+    # accuracy against the dense product: a statistical bound (keys sit on a 0.01 grid)
+    dense = X.double() @ K.double().T
+    rel = float(torch.linalg.norm(out.cpu().double() - dense) / torch.linalg.norm(dense))
+    assert rel < 0.25, rel
+    stats = ops.bsi_keys_cuda_stats(kcap)
+    assert stats == {"W": 32, "d": D, "num_keys": R, "decimals": 2, "threshold": 0.5, "Sb_counts": {6: R}}
+    rows = ops.build_bsi_queries_cuda_batch(X[:5].cuda(), 2, 0.5)
+    assert ops.bsi_query_caps_stats(rows) == {"Q": 5, "W": 32, "S_counts": {7: 5}}
+
+
+def test_ops_profile_flag_and_errors(ops, monkeypatch):
+    monkeypatch.setenv("BSI_PROFILE", "1")
+    ops._reset_flag_cache()
+    K = torch.randn(64, 512)
+    X = torch.randn(8, 512).cuda()
+    kcap, *_ = ops.build_bsi_keys_cuda(K, 2)
+    qcap = ops.build_bsi_queries_cuda_batch_packed(X, 2)
+    q_ns, p_ns, t_ns = ops.get_last_query_build_profile_cuda()
+    assert t_ns > 0 and t_ns == q_ns + p_ns
+    out, ns, ns_q, ns_s = ops.batch_dot_product_multiquery_cuda_batch_caps(qcap, kcap)
+    assert ns > 0 and ns_q == ns / 8 and ns_s == ns / (8 * 64)
+    ops.reset_last_query_build_profile_cuda()
+    assert ops.get_last_query_build_profile_cuda() == (0, 0, 0)
+    q_bad = ops.build_bsi_queries_cuda_batch_packed(torch.randn(8, 256).cuda(), 2)
+    with pytest.raises(RuntimeError, match="Word count mismatch"):
+        ops.batch_dot_product_multiquery_cuda_batch_caps(q_bad, kcap)
+    q_dec = ops.build_bsi_queries_cuda_batch_packed(X, 3)
+    with pytest.raises(RuntimeError, match="Decimal mismatch"):
+        ops.batch_dot_product_multiquery_cuda_batch_caps(q_dec, kcap)
+    qcap.chunk_scales = qcap.chunk_scales[:, :1].contiguous()
+    with pytest.raises(RuntimeError, match="Chunk scale stride mismatch"):
+        ops.batch_dot_product_multiquery_cuda_batch_caps(qcap, kcap)
+
+
+def test_full_size_fc1_properties(ops):
+    """Q512 x R8192 x D2048 with outlier columns: too big for the scalar oracle, so the integer
+    accumulators are checked against an fp64 matmul of the quantised values on the GPU (exact:
+    every partial sum is below 2^53), and the two cores against each other bit for bit."""
+    torch.manual_seed(123)
+    Q, R, D = 512, 8192, 2048
+    X = torch.randn(Q, D)
+    cols = torch.randperm(D)[:2]
+    X[:, cols] *= 20.0
+    K = torch.randn(R, D) * 0.02
+    kcap, *_ = ops.build_bsi_keys_cuda(K, 2, 0.5)
+    qcap = ops.build_bsi_queries_cuda_batch_packed(X.cuda(), 2, 0.5)
+    ints_m, out_m = ops.debug_chunk_ints(qcap, kcap, "mfma")
+    ints_v, out_v = ops.debug_chunk_ints(qcap, kcap, "valu")
+    assert torch.equal(ints_m, ints_v) and torch.equal(out_m, out_v)
+    # reconstruct the quantised values from the int8 operand (value << 1 in MFMA element order)
+    e = torch.arange(D, device="cuda")
+    pos = (e // 32) * 32 + ((e % 32) % 8) * 4 + (e % 32) // 8
+    a = (qcap.ints8[:, pos].to(torch.float64) / 2.0)
+    kx = K.cuda().double() * 100.0
+    rk = torch.sign(kx) * torch.floor(kx.abs() + 0.5)  # half away from zero (torch.round is half-to-even)
+    sh = kcap.shifts.to(torch.float64).unsqueeze(1)
+    b = torch.sign(rk) * torch.floor((rk.abs() + torch.where(sh > 0, 2.0 ** (sh - 1), torch.zeros_like(sh))) / 2.0 ** sh)
+    b = b.clamp(-32, 31)
+    for c in (0, 3, 7):
+        want = a[:, c * 256:(c + 1) * 256] @ b[:, c * 256:(c + 1) * 256].T
+        assert torch.equal(ints_m[:, :, c].to(torch.float64), want)
+    assert qcap.chunk_scales.max() > qcap.chunk_scales.median()  # outlier chunks got their own scale
+    out, *_ = ops.batch_dot_product_multiquery_cuda_batch_caps(qcap, kcap)
+    assert torch.equal(out, out_m)
+
+
+def test_linear_drop_in(ops, oracle):
+    from bsipytorch_amd.linear import BSIQuantizedLinear, quantize_model_bsi, sum_bsi_dot_query_vectors
+
+    torch.manual_seed(0)
+    lin = torch.nn.Linear(512, 192, bias=True)
+    blin = BSIQuantizedLinear(lin, decimalPlaces=2, compress_threshold=0.5)
+    x = torch.randn(2, 9, 512)
+    y = blin(x.cuda())
+    assert y.shape == (2, 9, 192) and y.dtype == x.dtype and y.is_cuda
+    # the layer is exactly: BSI dot of the quantised activations and weights, plus the bias
+    qb = oracle.build_queries(x.reshape(18, 512).numpy())
+    kb = oracle.build_keys(lin.weight.detach().numpy())
+    _, want = oracle.dot_fixed(qb["words"], qb["scales"], kb["words"], kb["scales"], oracle.scale_inv(2, 2))
+    want = torch.from_numpy(want) + lin.bias.detach()
+    assert torch.equal(y.cpu().reshape(18, 192), want)
+    # and close to the dense layer built from the de-quantised operands
+    a = torch.from_numpy(qb["ints"] * np.repeat(qb["scales"], 256, axis=1) / 100.0)
+    b = torch.from_numpy(kb["ints"] * kb["scales"][:, None] / 100.0)
+    dense = (a @ b.T).float() + lin.bias.detach()
+    assert torch.allclose(y.cpu().reshape(18, 192), dense, rtol=1e-4, atol=1e-5)
+    # half-precision activations go in natively and come back in their dtype
+    y16 = blin(x.cuda().to(torch.bfloat16))
+    assert y16.dtype == torch.bfloat16 and y16.shape == (2, 9, 192)
+    y2d = blin(x.cuda().reshape(18, 512))
+    assert y2d.shape == (18, 192) and torch.equal(y2d, y.reshape(18, 192))
+    assert blin.dot_calls == 3 and blin.dot_query_vectors_total == 54
+    assert blin.weight_bsi_memory_bytes == 192 * 6 * 8 * 8 and blin.dot_ns_total == 0
+
+    class Tiny(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.q_proj = torch.nn.Linear(256, 256)
+            self.fc1 = torch.nn.Linear(256, 512)
+            self.lm_head = torch.nn.Linear(512, 100)
+
+        def forward(self, t):
+            return self.lm_head(torch.relu(self.fc1(self.q_proj(t))))
+
+    m = Tiny()
+    inp = torch.randn(3, 256)
+    dense = m(inp)
+    quantize_model_bsi(m, decimalPlaces=2, scope="all", compress_threshold=0.5, verbose=False)
+    assert isinstance(m.q_proj, BSIQuantizedLinear) and isinstance(m.fc1, BSIQuantizedLinear)
+    assert isinstance(m.lm_head, torch.nn.Linear)
+    m.cuda()
+    got = m(inp.cuda()).cpu()
+    cos = float((got * dense).sum() / (torch.linalg.norm(got) * torch.linalg.norm(dense)))
+    assert cos > 0.9, cos
+    assert sum_bsi_dot_query_vectors(m) == 6
+    m2 = Tiny()
+    quantize_model_bsi(m2, scope="mlp", verbose=False)
+    assert isinstance(m2.fc1, BSIQuantizedLinear) and isinstance(m2.q_proj, torch.nn.Linear)
