@@ -249,6 +249,203 @@ __global__ __launch_bounds__(kMfmaBlock) void dot_mfma_kernel(
     }
 }
 
+// ------------------------------------------------------------------ MFMA core, producer/consumer form
+//
+// 512 threads: waves 0-3 are consumers (64 keys x 64 queries each, 64 MFMAs per chunk), waves 4-7
+// are producers.  A producer wave owns 32 key rows and 32 query rows of the 128 x 128 tile: per
+// chunk it reads its key planes from the tiled layout (one coalesced 512-byte wave load per plane
+// and 16-key tile: lane (m, g) gets words32 2g, 2g+1 of row m), transposes them to 64 int8 per
+// lane, and copies its query int8 rows; both go to the LDS buffer of the NEXT chunk while the
+// consumers run the MFMAs of the current one out of the other buffer.  The loads for the chunk
+// after that are issued before the barrier, so their latency is covered by a whole iteration.
+// Each SIMD hosts one consumer and one producer wave: the transposes run on the VALU while the
+// matrix pipe works.
+
+constexpr int kWsBlock = 512;
+constexpr int kWsStage = (kTileR + kTileQ) * kRowBytes;  // bytes of one LDS buffer
+
+template <int SB>
+struct WsRegs {
+    uint2 k[2][SB];  // two 16-key tiles x SB planes: words32 (2g, 2g+1) of row m
+    uint4 q[8];      // 8 x 16 B of the wave's 32 query rows
+};
+
+template <int SB>
+__device__ __forceinline__ void ws_load(WsRegs<SB>& rg, const unsigned long long* __restrict__ B64,
+                                        const int8_t* __restrict__ A8, int chunks, int c, int64_t tile0,
+                                        int64_t ntiles, int64_t q0, int64_t Q, int p, int lane) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        const int64_t tile = tile0 + p * 2 + t;
+#pragma unroll
+        for (int j = 0; j < SB; ++j) {
+            uint2 v = make_uint2(0u, 0u);
+            if (tile < ntiles) {
+                const unsigned long long w = B64[((static_cast<size_t>(tile) * chunks + c) * SB + j) * 64 + lane];
+                v = make_uint2(static_cast<uint32_t>(w), static_cast<uint32_t>(w >> 32));
+            }
+            rg.k[t][j] = v;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        // piece = i * 64 + lane of the wave's 32 rows x 16 pieces
+        const int piece = i * 64 + lane;
+        const int64_t q = q0 + p * 32 + (piece >> 4);
+        uint4 v = make_uint4(0u, 0u, 0u, 0u);
+        if (q < Q) v = *reinterpret_cast<const uint4*>(A8 + (static_cast<size_t>(q) * chunks + c) * 256 + (piece & 15) * 16);
+        rg.q[i] = v;
+    }
+}
+
+template <int SB>
+__device__ __forceinline__ void ws_store(const WsRegs<SB>& rg, unsigned char* __restrict__ buf, int p, int lane) {
+    unsigned char* K8 = buf;
+    unsigned char* Q8 = buf + kTileR * kRowBytes;
+    const int m = lane & 15, g = lane >> 4;
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        uint32_t lo[8], hi[8];
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            lo[s] = (s >= 8 - SB) ? rg.k[t][s - (8 - SB)].x : 0u;
+            hi[s] = (s >= 8 - SB) ? rg.k[t][s - (8 - SB)].y : 0u;
+        }
+        transpose8x8(lo);
+        transpose8x8(hi);
+        uint4* dst = reinterpret_cast<uint4*>(K8 + (p * 32 + t * 16 + m) * kRowBytes + g * 64);
+        dst[0] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+        dst[1] = make_uint4(lo[4], lo[5], lo[6], lo[7]);
+        dst[2] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+        dst[3] = make_uint4(hi[4], hi[5], hi[6], hi[7]);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int piece = i * 64 + lane;
+        *reinterpret_cast<uint4*>(Q8 + (p * 32 + (piece >> 4)) * kRowBytes + (piece & 15) * 16) = rg.q[i];
+    }
+}
+
+template <int SB, bool kInts>
+__global__ __launch_bounds__(kWsBlock) void dot_mfma_ws_kernel(
+    const int8_t* __restrict__ A8, const float* __restrict__ qscale, int qscale_stride,
+    const unsigned long long* __restrict__ B64,  // tiled key planes
+    const float* __restrict__ Bw, int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv, int64_t R_total,
+    float* __restrict__ out, int* __restrict__ chunk_ints) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];  // 2 * kWsStage
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const bool consumer = wave < 4;
+    const int64_t r0 = static_cast<int64_t>(blockIdx.x) * kTileR;
+    const int64_t q0 = static_cast<int64_t>(blockIdx.y) * kTileQ;
+    const int64_t ntiles = (R + 15) / 16;
+    const int64_t tile0 = r0 / 16;
+
+    if (consumer) {
+        const int wr = wave & 1, wq = wave >> 1;
+        const int ln = lane & 15, lg = lane >> 4;
+        float accf[4][4][4];
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+            for (int b = 0; b < 4; ++b)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) accf[a][b][e] = 0.0f;
+        const float down = __uint_as_float(static_cast<uint32_t>(127 - down_shift) << 23);
+        const int qstep = (qscale_stride == 1) ? 0 : 1;
+        // this lane's four query columns: their scale pointers
+        const float* qsp[4];
+        bool qok[4];
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const int64_t q = q0 + wq * 64 + b * 16 + ln;
+            qok[b] = q < Q;
+            qsp[b] = qscale + (qok[b] ? q : 0) * qscale_stride;
+        }
+        __syncthreads();  // buffer 0 filled by the producers' prologue
+        for (int c = 0; c < chunks; ++c) {
+            const unsigned char* K8 = lds + (c & 1) * kWsStage;
+            const unsigned char* Q8 = K8 + kTileR * kRowBytes;
+            float qs[4];
+#pragma unroll
+            for (int b = 0; b < 4; ++b) qs[b] = qok[b] ? qsp[b][c * qstep] * down : 0.0f;
+            v4i acc[4][4];
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+#pragma unroll
+                for (int b = 0; b < 4; ++b) acc[a][b] = (v4i){0, 0, 0, 0};
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+                v4i ka[4], qb[4];
+#pragma unroll
+                for (int a = 0; a < 4; ++a)
+                    ka[a] = *reinterpret_cast<const v4i*>(K8 + (wr * 64 + a * 16 + ln) * kRowBytes + ks * 64 + lg * 16);
+#pragma unroll
+                for (int b = 0; b < 4; ++b)
+                    qb[b] = *reinterpret_cast<const v4i*>(Q8 + (wq * 64 + b * 16 + ln) * kRowBytes + ks * 64 + lg * 16);
+#pragma unroll
+                for (int a = 0; a < 4; ++a)
+#pragma unroll
+                    for (int b = 0; b < 4; ++b)
+                        acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ka[a], qb[b], acc[a][b], 0, 0, 0);
+            }
+#pragma unroll
+            for (int b = 0; b < 4; ++b)
+#pragma unroll
+                for (int a = 0; a < 4; ++a)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        accf[a][b][e] = fmaf(static_cast<float>(acc[a][b][e]), qs[b], accf[a][b][e]);
+                        if (kInts) {
+                            const int64_t q = q0 + wq * 64 + b * 16 + ln;
+                            const int64_t r = r0 + wr * 64 + a * 16 + lg * 4 + e;
+                            if (q < Q && r < R)
+                                chunk_ints[(static_cast<size_t>(q) * R + r) * chunks + c] = acc[a][b][e] >> down_shift;
+                        }
+                    }
+            __syncthreads();
+        }
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            const int64_t rb = r0 + wr * 64 + a * 16 + lg * 4;
+            float bs[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) bs[e] = (rb + e < R) ? Bw[(rb + e) * SB] : 0.0f;
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                const int64_t q = q0 + wq * 64 + b * 16 + ln;
+                if (q >= Q) continue;
+                float* dst = out + static_cast<size_t>(q) * R_total + rb;
+                if (rb + 3 < R && ((reinterpret_cast<uintptr_t>(dst) & 15) == 0)) {
+                    *reinterpret_cast<float4*>(dst) =
+                        make_float4((accf[a][b][0] * bs[0]) * scale_inv, (accf[a][b][1] * bs[1]) * scale_inv,
+                                    (accf[a][b][2] * bs[2]) * scale_inv, (accf[a][b][3] * bs[3]) * scale_inv);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (rb + e < R) dst[e] = (accf[a][b][e] * bs[e]) * scale_inv;
+                }
+            }
+        }
+    } else {
+        const int p = wave - 4;
+        WsRegs<SB> rg;
+        ws_load<SB>(rg, B64, A8, chunks, 0, tile0, ntiles, q0, Q, p, lane);
+        ws_store<SB>(rg, lds, p, lane);
+        if (chunks > 1) ws_load<SB>(rg, B64, A8, chunks, 1, tile0, ntiles, q0, Q, p, lane);
+        __syncthreads();
+        for (int c = 0; c < chunks; ++c) {
+            if (c + 1 < chunks) {
+                ws_store<SB>(rg, lds + ((c + 1) & 1) * kWsStage, p, lane);
+                if (c + 2 < chunks) ws_load<SB>(rg, B64, A8, chunks, c + 2, tile0, ntiles, q0, Q, p, lane);
+            }
+            __syncthreads();
+        }
+    }
+}
+
 // ------------------------------------------------------------------ VALU popcount core (Sa = 7, Sb = 6 shape templated)
 
 constexpr int kValuBlock = 256;
@@ -451,6 +648,30 @@ static void launch_mfma(const int8_t* A8, const float* qscale, int stride, const
                            R_total, out, chunk_ints);
 }
 
+template <int SB>
+static void launch_mfma_ws(const int8_t* A8, const float* qscale, int stride, const uint64_t* B, const float* Bw,
+                           int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv, int64_t R_total,
+                           float* out, int32_t* chunk_ints, hipStream_t st) {
+    const dim3 grid(static_cast<unsigned>((R + kTileR - 1) / kTileR), static_cast<unsigned>((Q + kTileQ - 1) / kTileQ));
+    constexpr int kLds = 2 * kWsStage;
+    static bool configured = false;
+    if (!configured) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dot_mfma_ws_kernel<SB, true>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dot_mfma_ws_kernel<SB, false>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+        configured = true;
+    }
+    if (chunk_ints)
+        hipLaunchKernelGGL((dot_mfma_ws_kernel<SB, true>), grid, dim3(kWsBlock), kLds, st, A8, qscale, stride,
+                           reinterpret_cast<const unsigned long long*>(B), Bw, chunks, R, Q, down_shift, scale_inv,
+                           R_total, out, chunk_ints);
+    else
+        hipLaunchKernelGGL((dot_mfma_ws_kernel<SB, false>), grid, dim3(kWsBlock), kLds, st, A8, qscale, stride,
+                           reinterpret_cast<const unsigned long long*>(B), Bw, chunks, R, Q, down_shift, scale_inv,
+                           R_total, out, chunk_ints);
+}
+
 template <bool kTiled>
 static void launch_valu76(const uint64_t* A, const float* qscale, int stride, const uint64_t* B, const float* Bw,
                           int W64, int chunks, int64_t R, int64_t Q, float scale_inv, int64_t R_total, float* out,
@@ -532,6 +753,11 @@ extern "C" int bsi_hip_dot(const uint64_t* A, const int8_t* A_ints8, const float
         }
         const int down_shift = 16 - Sa - Sb;
         const bool tiled = (b_layout == BSI_LAYOUT_TILED16);
+        if (Sb == 6 && tiled) {
+            launch_mfma_ws<6>(A8, A_chunk_scales, A_scale_stride, B, Bw, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, st);
+            BSI_LAUNCH_CHECK("dot_mfma_ws_kernel");
+            return BSI_OK;
+        }
         if (Sb == 6) {
             if (tiled) launch_mfma<6, true>(A8, A_chunk_scales, A_scale_stride, B, Bw, Sb, W64, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, st);
             else launch_mfma<6, false>(A8, A_chunk_scales, A_scale_stride, B, Bw, Sb, W64, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, st);
