@@ -1,0 +1,86 @@
+"""Microbenchmark of the BSI dot kernel on one GPU (same flags as the reference's
+``bsi_ops/benchmarks/benchmark_dot_kernel_micro.py``, plus the core, key layout and input shaping
+of the FC1/FC2-like configurations).
+
+    python -m bsipytorch_amd.benchmarks.benchmark_dot_kernel_micro --Q 512 --R 8192 --D 2048 --outliers
+    python -m bsipytorch_amd.benchmarks.benchmark_dot_kernel_micro --Q 512 --R 2048 --D 8192 --relu
+
+The kernel time is measured with HIP events around ``iters`` back-to-back launches on the launch
+stream; no environment flag is needed (the reference prints zeros unless BSI_PROFILE=1).
+"""
+import argparse
+import ctypes
+import json
+
+import torch
+
+from bsipytorch_amd import _lib, bsi_ops
+
+
+def run(Q, R, D, decimal_places=2, compress_threshold=0.5, warmup=10, iters=50, seed=123, core="auto",
+        key_sigma=0.02, outliers=False, relu=False, use_ints8=True, report_stats=False):
+    torch.manual_seed(seed)
+    K = torch.randn(R, D, dtype=torch.float32) * key_sigma
+    X = torch.randn(Q, D, dtype=torch.float32)
+    if outliers:
+        X[:, torch.randperm(D)[: max(1, D // 1000)]] *= 20.0
+    if relu:
+        X = torch.relu(X)
+    kcap, key_bytes, _, _, W = bsi_ops.build_bsi_keys_cuda(K, decimal_places, float(compress_threshold))
+    qcap = bsi_ops.build_bsi_queries_cuda_batch_packed(X.cuda(), decimal_places, float(compress_threshold))
+    if report_stats:
+        print("[Keys]", bsi_ops.bsi_keys_cuda_stats(kcap))
+    chunks = (W + 3) // 4
+    if qcap.chunk_scales is not None:
+        scales, stride = qcap.chunk_scales, chunks
+    else:
+        scales, stride = qcap.row_scales, 1
+    code = {"auto": _lib.CORE_AUTO, "mfma": _lib.CORE_MFMA, "valu": _lib.CORE_VALU}[core]
+    out = torch.empty((Q, R), dtype=torch.float32, device="cuda")
+    ws_bytes = 0 if use_ints8 else int(_lib.lib.bsi_hip_dot_workspace_bytes(Q, W, code))
+    ws = torch.empty((max(ws_bytes, 16),), dtype=torch.uint8, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    args = (qcap.words.data_ptr(), qcap.ints8.data_ptr() if use_ints8 else None, scales.data_ptr(), stride, qcap.Sa, W,
+            kcap.words.data_ptr(), kcap.layout, kcap.slice_weights.data_ptr(), kcap.Sb, R, Q, 1.0 / 10.0 ** (2 * decimal_places),
+            R, out.data_ptr(), code, ws.data_ptr(), ws_bytes)
+    us = ctypes.c_float(0.0)
+    if warmup > 0:
+        _lib.check(_lib.lib.bsi_hip_dot_timed(*args, warmup, ctypes.byref(us), st), "warmup")
+    _lib.check(_lib.lib.bsi_hip_dot_timed(*args, iters, ctypes.byref(us), st), "timed")
+    t = float(us.value) * 1e-6
+    bit_ops = 2.0 * qcap.Sa * kcap.Sb * Q * R * D
+    alg_bytes = Q * qcap.Sa * W * 8 + Q * chunks * 4 + R * kcap.Sb * W * 8 + R * 4 + Q * R * 4
+    return {"Q": Q, "R": R, "D": D, "core": core, "layout": "tiled16" if kcap.layout else "canonical",
+            "avg_dot_us": t * 1e6, "dot_q_us": t * 1e6 / Q, "dot_s_ns": t * 1e9 / (Q * R),
+            "effective_bitop_TOPS": bit_ops / t / 1e12, "int8_TOPS": 2.0 * Q * R * D / t / 1e12,
+            "algorithmic_GBps": alg_bytes / t / 1e9, "key_plane_GBps": key_bytes / t / 1e9, "iters": iters}
+
+
+def main() -> None:
+    p = argparse.ArgumentParser(description="Microbench BSI dot kernel (HIP, gfx950)")
+    p.add_argument("--Q", type=int, default=128)
+    p.add_argument("--R", type=int, default=256)
+    p.add_argument("--D", type=int, default=2048)
+    p.add_argument("--decimal_places", type=int, default=2)
+    p.add_argument("--compress_threshold", type=float, default=0.5)
+    p.add_argument("--warmup", type=int, default=5)
+    p.add_argument("--iters", type=int, default=20)
+    p.add_argument("--seed", type=int, default=123)
+    p.add_argument("--core", default="auto", choices=["auto", "mfma", "valu"])
+    p.add_argument("--key_sigma", type=float, default=0.02)
+    p.add_argument("--outliers", action="store_true", help="scale 0.1%% of the query columns by 20")
+    p.add_argument("--relu", action="store_true", help="ReLU the queries (about half exact zeros)")
+    p.add_argument("--planes_only", action="store_true", help="do not hand the builder's int8 queries to the dot")
+    p.add_argument("--report_stats", action="store_true")
+    a = p.parse_args()
+    if not torch.cuda.is_available():
+        raise RuntimeError("a GPU is required for this microbench")
+    r = run(a.Q, a.R, a.D, a.decimal_places, a.compress_threshold, a.warmup, a.iters, a.seed, a.core, a.key_sigma,
+            a.outliers, a.relu, not a.planes_only, a.report_stats)
+    print(f"[Microbench] Q={a.Q} R={a.R} D={a.D} iters={a.iters} core={r['core']} layout={r['layout']}")
+    print(f"[Kernel] avg_dot_ms={r['avg_dot_us'] / 1e3:.4f}  dot_q_us={r['dot_q_us']:.3f}  dot_s_ns={r['dot_s_ns']:.4f}")
+    print(json.dumps(r))
+
+
+if __name__ == "__main__":
+    main()
