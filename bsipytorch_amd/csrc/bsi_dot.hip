@@ -666,6 +666,120 @@ __global__ __launch_bounds__(kWsBlock) void dot_mfma_ws_kernel(
     }
 }
 
+// ------------------------------------------------------------------ MFMA core, few query rows
+//
+// Decode-like shapes (a handful of query rows against a large key matrix) are bound by reading the
+// packed key planes once.  One workgroup owns one 16-key tile of the tiled layout over all chunks
+// and up to 16 * NT query rows; its waves take the chunks round-robin.  A lane loads the six plane
+// words of (key row lane % 16, 64-bit word lane / 16), transposes them in registers into the four
+// 16-byte MFMA operands of that row (no LDS staging: with a k permutation shared by both operands
+// any assignment of chunk elements to MFMA k-slots gives the same integer), loads the matching 64
+// int8 query bytes from L2, and issues 4 MFMAs per query tile.  The int32 results go to LDS
+// indexed by chunk; after a workgroup barrier 256 * NT lanes run the fp32 chain of their (query,
+// key) pair over the chunks in order, so the result is bit-identical to a sequential pass
+// whatever the number of waves.  Problems with more chunks than LDS slots run in several passes.
+constexpr int kStreamMaxQ = 32;        // above this the 128 x 128 tiled kernel takes over
+constexpr int kStreamLdsInts = 16384;  // 64 KiB of chunk accumulators: 64 / NT chunks per pass
+
+template <int NT, bool kInts>
+__global__ __launch_bounds__(1024) void dot_mfma_stream_kernel(
+    const int8_t* __restrict__ A8, const float* __restrict__ qscale, int qscale_stride,
+    const unsigned long long* __restrict__ B64,  // tiled key planes, Sb = 6
+    const float* __restrict__ Bw, int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv, int64_t R_total,
+    float* __restrict__ out, int* __restrict__ chunk_ints) {
+    __shared__ __attribute__((aligned(16))) int ints[kStreamLdsInts];
+    constexpr int kPass = kStreamLdsInts / (NT * 256);  // chunk slots
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nwaves = static_cast<int>(blockDim.x >> 6);
+    const int ln = lane & 15, lg = lane >> 4;
+    const int64_t tile = blockIdx.x;
+    const int64_t r0 = tile * 16;
+    const int64_t q0 = static_cast<int64_t>(blockIdx.y) * (16 * NT);
+    const unsigned long long* ksrc = B64 + static_cast<size_t>(tile) * chunks * (6 * 64) + lane;
+    const size_t arow = static_cast<size_t>(chunks) * 256;
+
+    // the chain lanes: (query tile t, query n, key) <-> tid, keys fastest so output stores are contiguous
+    const bool chain = tid < NT * 256;
+    const int ct = tid >> 8, cn = (tid >> 4) & 15, ckey = tid & 15;
+    const int64_t cq = q0 + ct * 16 + cn, cr = r0 + ckey;
+    const bool cvalid = chain && cq < Q && cr < R;
+    const float down = __uint_as_float(static_cast<uint32_t>(127 - down_shift) << 23);
+    const float* csrc = qscale + (cvalid ? cq : 0) * qscale_stride;
+    const int sstep = (qscale_stride == 1) ? 0 : 1;
+    float accf = 0.0f;
+
+    for (int p0 = 0; p0 < chunks; p0 += kPass) {
+        const int pend = (p0 + kPass < chunks) ? p0 + kPass : chunks;
+        int c = p0 + wave;
+        uint2 kc[6];
+        if (c < pend) {
+#pragma unroll
+            for (int j = 0; j < 6; ++j) {
+                const unsigned long long w = ksrc[(static_cast<size_t>(c) * 6 + j) * 64];
+                kc[j] = make_uint2(static_cast<uint32_t>(w), static_cast<uint32_t>(w >> 32));
+            }
+        }
+        for (; c < pend; c += nwaves) {
+            // query operands of this chunk (L2 resident), then the key planes of the wave's next chunk
+            v4i qb[NT][4];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                const int64_t q = q0 + t * 16 + ln;
+                if (q < Q) {
+                    const v4i* src = reinterpret_cast<const v4i*>(A8 + static_cast<size_t>(q) * arow + c * 256 + lg * 64);
+#pragma unroll
+                    for (int m = 0; m < 4; ++m) qb[t][m] = src[m];
+                } else {
+#pragma unroll
+                    for (int m = 0; m < 4; ++m) qb[t][m] = (v4i){0, 0, 0, 0};
+                }
+            }
+            uint2 kn[6];
+            const int cnext = c + nwaves;
+            if (cnext < pend) {
+#pragma unroll
+                for (int j = 0; j < 6; ++j) {
+                    const unsigned long long w = ksrc[(static_cast<size_t>(cnext) * 6 + j) * 64];
+                    kn[j] = make_uint2(static_cast<uint32_t>(w), static_cast<uint32_t>(w >> 32));
+                }
+            }
+            uint32_t lo[8], hi[8];
+            transpose_6planes(kc[0].x, kc[1].x, kc[2].x, kc[3].x, kc[4].x, kc[5].x, lo);
+            transpose_6planes(kc[0].y, kc[1].y, kc[2].y, kc[3].y, kc[4].y, kc[5].y, hi);
+            v4i ka[4];
+            ka[0] = (v4i){static_cast<int>(lo[0]), static_cast<int>(lo[1]), static_cast<int>(lo[2]), static_cast<int>(lo[3])};
+            ka[1] = (v4i){static_cast<int>(lo[4]), static_cast<int>(lo[5]), static_cast<int>(lo[6]), static_cast<int>(lo[7])};
+            ka[2] = (v4i){static_cast<int>(hi[0]), static_cast<int>(hi[1]), static_cast<int>(hi[2]), static_cast<int>(hi[3])};
+            ka[3] = (v4i){static_cast<int>(hi[4]), static_cast<int>(hi[5]), static_cast<int>(hi[6]), static_cast<int>(hi[7])};
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                v4i acc = {0, 0, 0, 0};
+#pragma unroll
+                for (int m = 0; m < 4; ++m) acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(ka[m], qb[t][m], acc, 0, 0, 0);
+                // lane holds keys 4*lg .. 4*lg+3 of query ln: slot layout [t][query][key]
+                *reinterpret_cast<v4i*>(&ints[((c - p0) * NT + t) * 256 + ln * 16 + lg * 4]) = acc;
+            }
+            if (cnext < pend) {
+#pragma unroll
+                for (int j = 0; j < 6; ++j) kc[j] = kn[j];
+            }
+        }
+        __syncthreads();
+        if (cvalid) {
+            for (int cc = p0; cc < pend; ++cc) {
+                const int v = ints[(cc - p0) * (NT * 256) + tid];
+                accf = fmaf(static_cast<float>(v), csrc[cc * sstep] * down, accf);
+                if (kInts) chunk_ints[(cq * R + cr) * chunks + cc] = v >> down_shift;
+            }
+        }
+        if (pend < chunks) __syncthreads();
+    }
+    if (cvalid) out[static_cast<size_t>(cq) * R_total + cr] = (accf * Bw[cr * 6]) * scale_inv;
+}
+
 // ------------------------------------------------------------------ VALU popcount core (Sa = 7, Sb = 6 shape templated)
 
 constexpr int kValuBlock = 256;
@@ -892,6 +1006,23 @@ static void launch_mfma_ws(const int8_t* A8, const float* qscale, int stride, co
                            R_total, out, chunk_ints);
 }
 
+template <int NT>
+static void launch_mfma_stream(const int8_t* A8, const float* qscale, int stride, const uint64_t* B, const float* Bw,
+                               int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv, int64_t R_total,
+                               float* out, int32_t* chunk_ints, hipStream_t st) {
+    const dim3 grid(static_cast<unsigned>((R + 15) / 16), static_cast<unsigned>((Q + 16 * NT - 1) / (16 * NT)));
+    int waves = chunks < 16 ? chunks : 16;  // one chunk per wave and pass at least
+    if (waves < 4 * NT) waves = 4 * NT;     // the chain needs 256 * NT lanes
+    if (chunk_ints)
+        hipLaunchKernelGGL((dot_mfma_stream_kernel<NT, true>), grid, dim3(waves * 64), 0, st, A8, qscale, stride,
+                           reinterpret_cast<const unsigned long long*>(B), Bw, chunks, R, Q, down_shift, scale_inv,
+                           R_total, out, chunk_ints);
+    else
+        hipLaunchKernelGGL((dot_mfma_stream_kernel<NT, false>), grid, dim3(waves * 64), 0, st, A8, qscale, stride,
+                           reinterpret_cast<const unsigned long long*>(B), Bw, chunks, R, Q, down_shift, scale_inv,
+                           R_total, out, chunk_ints);
+}
+
 template <bool kTiled>
 static void launch_valu76(const uint64_t* A, const float* qscale, int stride, const uint64_t* B, const float* Bw,
                           int W64, int chunks, int64_t R, int64_t Q, float scale_inv, int64_t R_total, float* out,
@@ -973,6 +1104,12 @@ extern "C" int bsi_hip_dot(const uint64_t* A, const int8_t* A_ints8, const float
         }
         const int down_shift = 16 - Sa - Sb;
         const bool tiled = (b_layout == BSI_LAYOUT_TILED16);
+        if (Sb == 6 && tiled && Q <= kStreamMaxQ) {
+            if (Q <= 16) launch_mfma_stream<1>(A8, A_chunk_scales, A_scale_stride, B, Bw, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, st);
+            else launch_mfma_stream<2>(A8, A_chunk_scales, A_scale_stride, B, Bw, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, st);
+            BSI_LAUNCH_CHECK("dot_mfma_stream_kernel");
+            return BSI_OK;
+        }
         if (Sb == 6 && tiled) {
             launch_mfma_ws<6>(A8, A_chunk_scales, A_scale_stride, B, Bw, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, st);
             BSI_LAUNCH_CHECK("dot_mfma_ws_kernel");

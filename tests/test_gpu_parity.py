@@ -316,6 +316,9 @@ DOT_SHAPES = [
     (5, 3, 256, "ties"),          # a single chunk
     (16, 40, 700, "randn"),       # W64 = 11: row scale, partial last chunk
     (1, 200, 4096, "randn"),      # a single query
+    (17, 50, 1024, "randn"),      # two query tiles of the few-rows kernel, ragged in both
+    (32, 33, 8704, "relu"),       # 34 chunks: more than one pass of the few-rows kernel with two query tiles
+    (3, 20, 16640, "randn"),      # 65 chunks: more than one pass with one query tile
 ]
 
 
