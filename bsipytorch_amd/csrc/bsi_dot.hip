@@ -679,48 +679,56 @@ __global__ __launch_bounds__(kWsBlock) void dot_mfma_ws_kernel(
 // key) pair over the chunks in order, so the result is bit-identical to a sequential pass
 // whatever the number of waves.  Problems with more chunks than LDS slots run in several passes.
 constexpr int kStreamMaxQ = 32;        // above this the 128 x 128 tiled kernel takes over
-constexpr int kStreamLdsInts = 16384;  // 64 KiB of chunk accumulators: 64 / NT chunks per pass
+constexpr int kStreamLdsInts = 16384;  // at most 64 KiB of chunk accumulators per pass
 
-template <int NT, bool kInts>
+template <int NT, int KT, bool kInts>
 __global__ __launch_bounds__(1024) void dot_mfma_stream_kernel(
     const int8_t* __restrict__ A8, const float* __restrict__ qscale, int qscale_stride,
     const unsigned long long* __restrict__ B64,  // tiled key planes, Sb = 6
-    const float* __restrict__ Bw, int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv, int64_t R_total,
-    float* __restrict__ out, int* __restrict__ chunk_ints) {
-    __shared__ __attribute__((aligned(16))) int ints[kStreamLdsInts];
-    constexpr int kPass = kStreamLdsInts / (NT * 256);  // chunk slots
+    const float* __restrict__ Bw, int chunks, int pass_chunks, int64_t R, int64_t Q, int down_shift, float scale_inv,
+    int64_t R_total, float* __restrict__ out, int* __restrict__ chunk_ints) {
+    extern __shared__ __attribute__((aligned(16))) int ints[];  // [pass_chunks][KT][NT][16 queries][16 keys]
+    constexpr int kSlot = KT * NT * 256;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nwaves = static_cast<int>(blockDim.x >> 6);
     const int ln = lane & 15, lg = lane >> 4;
-    const int64_t tile = blockIdx.x;
-    const int64_t r0 = tile * 16;
+    const int64_t ntiles = (R + 15) / 16;
+    const int64_t tile0 = static_cast<int64_t>(blockIdx.x) * KT;
     const int64_t q0 = static_cast<int64_t>(blockIdx.y) * (16 * NT);
-    const unsigned long long* ksrc = B64 + static_cast<size_t>(tile) * chunks * (6 * 64) + lane;
+    const size_t ktile = static_cast<size_t>(chunks) * (6 * 64);  // words per key tile
+    const unsigned long long* ksrc[KT];
+#pragma unroll
+    for (int k = 0; k < KT; ++k) {
+        const int64_t t = (tile0 + k < ntiles) ? tile0 + k : ntiles - 1;  // clamped: its outputs are never stored
+        ksrc[k] = B64 + static_cast<size_t>(t) * ktile + lane;
+    }
     const size_t arow = static_cast<size_t>(chunks) * 256;
 
-    // the chain lanes: (query tile t, query n, key) <-> tid, keys fastest so output stores are contiguous
-    const bool chain = tid < NT * 256;
-    const int ct = tid >> 8, cn = (tid >> 4) & 15, ckey = tid & 15;
-    const int64_t cq = q0 + ct * 16 + cn, cr = r0 + ckey;
+    // the chain lanes: tid <-> (key tile, query tile, query, key), keys fastest so output stores are contiguous
+    float accf = 0.0f;
+    const bool chain = tid < kSlot;
+    const int ck = tid / (NT * 256), ct = (tid >> 8) % NT, cn = (tid >> 4) & 15, ckey = tid & 15;
+    const int64_t cq = q0 + ct * 16 + cn, cr = (tile0 + ck) * 16 + ckey;
     const bool cvalid = chain && cq < Q && cr < R;
     const float down = __uint_as_float(static_cast<uint32_t>(127 - down_shift) << 23);
     const float* csrc = qscale + (cvalid ? cq : 0) * qscale_stride;
     const int sstep = (qscale_stride == 1) ? 0 : 1;
-    float accf = 0.0f;
 
-    for (int p0 = 0; p0 < chunks; p0 += kPass) {
-        const int pend = (p0 + kPass < chunks) ? p0 + kPass : chunks;
+    for (int p0 = 0; p0 < chunks; p0 += pass_chunks) {
+        const int pend = (p0 + pass_chunks < chunks) ? p0 + pass_chunks : chunks;
         int c = p0 + wave;
-        uint2 kc[6];
+        uint2 kc[KT][6];
         if (c < pend) {
 #pragma unroll
-            for (int j = 0; j < 6; ++j) {
-                const unsigned long long w = ksrc[(static_cast<size_t>(c) * 6 + j) * 64];
-                kc[j] = make_uint2(static_cast<uint32_t>(w), static_cast<uint32_t>(w >> 32));
-            }
+            for (int k = 0; k < KT; ++k)
+#pragma unroll
+                for (int j = 0; j < 6; ++j) {
+                    const unsigned long long w = ksrc[k][(static_cast<size_t>(c) * 6 + j) * 64];
+                    kc[k][j] = make_uint2(static_cast<uint32_t>(w), static_cast<uint32_t>(w >> 32));
+                }
         }
         for (; c < pend; c += nwaves) {
             // query operands of this chunk (L2 resident), then the key planes of the wave's next chunk
@@ -737,40 +745,47 @@ __global__ __launch_bounds__(1024) void dot_mfma_stream_kernel(
                     for (int m = 0; m < 4; ++m) qb[t][m] = (v4i){0, 0, 0, 0};
                 }
             }
-            uint2 kn[6];
+            uint2 kn[KT][6];
             const int cnext = c + nwaves;
             if (cnext < pend) {
 #pragma unroll
-                for (int j = 0; j < 6; ++j) {
-                    const unsigned long long w = ksrc[(static_cast<size_t>(cnext) * 6 + j) * 64];
-                    kn[j] = make_uint2(static_cast<uint32_t>(w), static_cast<uint32_t>(w >> 32));
-                }
+                for (int k = 0; k < KT; ++k)
+#pragma unroll
+                    for (int j = 0; j < 6; ++j) {
+                        const unsigned long long w = ksrc[k][(static_cast<size_t>(cnext) * 6 + j) * 64];
+                        kn[k][j] = make_uint2(static_cast<uint32_t>(w), static_cast<uint32_t>(w >> 32));
+                    }
             }
-            uint32_t lo[8], hi[8];
-            transpose_6planes(kc[0].x, kc[1].x, kc[2].x, kc[3].x, kc[4].x, kc[5].x, lo);
-            transpose_6planes(kc[0].y, kc[1].y, kc[2].y, kc[3].y, kc[4].y, kc[5].y, hi);
-            v4i ka[4];
-            ka[0] = (v4i){static_cast<int>(lo[0]), static_cast<int>(lo[1]), static_cast<int>(lo[2]), static_cast<int>(lo[3])};
-            ka[1] = (v4i){static_cast<int>(lo[4]), static_cast<int>(lo[5]), static_cast<int>(lo[6]), static_cast<int>(lo[7])};
-            ka[2] = (v4i){static_cast<int>(hi[0]), static_cast<int>(hi[1]), static_cast<int>(hi[2]), static_cast<int>(hi[3])};
-            ka[3] = (v4i){static_cast<int>(hi[4]), static_cast<int>(hi[5]), static_cast<int>(hi[6]), static_cast<int>(hi[7])};
 #pragma unroll
-            for (int t = 0; t < NT; ++t) {
-                v4i acc = {0, 0, 0, 0};
+            for (int k = 0; k < KT; ++k) {
+                uint32_t lo[8], hi[8];
+                transpose_6planes(kc[k][0].x, kc[k][1].x, kc[k][2].x, kc[k][3].x, kc[k][4].x, kc[k][5].x, lo);
+                transpose_6planes(kc[k][0].y, kc[k][1].y, kc[k][2].y, kc[k][3].y, kc[k][4].y, kc[k][5].y, hi);
+                v4i ka[4];
+                ka[0] = (v4i){static_cast<int>(lo[0]), static_cast<int>(lo[1]), static_cast<int>(lo[2]), static_cast<int>(lo[3])};
+                ka[1] = (v4i){static_cast<int>(lo[4]), static_cast<int>(lo[5]), static_cast<int>(lo[6]), static_cast<int>(lo[7])};
+                ka[2] = (v4i){static_cast<int>(hi[0]), static_cast<int>(hi[1]), static_cast<int>(hi[2]), static_cast<int>(hi[3])};
+                ka[3] = (v4i){static_cast<int>(hi[4]), static_cast<int>(hi[5]), static_cast<int>(hi[6]), static_cast<int>(hi[7])};
 #pragma unroll
-                for (int m = 0; m < 4; ++m) acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(ka[m], qb[t][m], acc, 0, 0, 0);
-                // lane holds keys 4*lg .. 4*lg+3 of query ln: slot layout [t][query][key]
-                *reinterpret_cast<v4i*>(&ints[((c - p0) * NT + t) * 256 + ln * 16 + lg * 4]) = acc;
+                for (int t = 0; t < NT; ++t) {
+                    v4i acc = {0, 0, 0, 0};
+#pragma unroll
+                    for (int m = 0; m < 4; ++m) acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(ka[m], qb[t][m], acc, 0, 0, 0);
+                    // the lane holds keys 4*lg .. 4*lg+3 of query ln
+                    *reinterpret_cast<v4i*>(&ints[(c - p0) * kSlot + (k * NT + t) * 256 + ln * 16 + lg * 4]) = acc;
+                }
             }
             if (cnext < pend) {
 #pragma unroll
-                for (int j = 0; j < 6; ++j) kc[j] = kn[j];
+                for (int k = 0; k < KT; ++k)
+#pragma unroll
+                    for (int j = 0; j < 6; ++j) kc[k][j] = kn[k][j];
             }
         }
         __syncthreads();
         if (cvalid) {
             for (int cc = p0; cc < pend; ++cc) {
-                const int v = ints[(cc - p0) * (NT * 256) + tid];
+                const int v = ints[(cc - p0) * kSlot + tid];
                 accf = fmaf(static_cast<float>(v), csrc[cc * sstep] * down, accf);
                 if (kInts) chunk_ints[(cq * R + cr) * chunks + cc] = v >> down_shift;
             }
@@ -1006,21 +1021,29 @@ static void launch_mfma_ws(const int8_t* A8, const float* qscale, int stride, co
                            R_total, out, chunk_ints);
 }
 
-template <int NT>
+template <int NT, int KT>
 static void launch_mfma_stream(const int8_t* A8, const float* qscale, int stride, const uint64_t* B, const float* Bw,
                                int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv, int64_t R_total,
                                float* out, int32_t* chunk_ints, hipStream_t st) {
-    const dim3 grid(static_cast<unsigned>((R + 15) / 16), static_cast<unsigned>((Q + 16 * NT - 1) / (16 * NT)));
-    int waves = chunks < 16 ? chunks : 16;  // one chunk per wave and pass at least
-    if (waves < 4 * NT) waves = 4 * NT;     // the chain needs 256 * NT lanes
+    constexpr int kSlot = KT * NT * 256;
+    const int64_t ntiles = (R + 15) / 16;
+    const dim3 grid(static_cast<unsigned>((ntiles + KT - 1) / KT), static_cast<unsigned>((Q + 16 * NT - 1) / (16 * NT)));
+    // one workgroup per CU at most: more waves each streaming their own chunks; else 8 and several workgroups
+    int waves = (grid.x * grid.y <= 256) ? 16 : 8;
+    if (waves > chunks) waves = chunks;             // one chunk per wave and pass at least
+    if (waves < kSlot / 64) waves = kSlot / 64;     // the chain needs one lane per output
+    if (waves > 16) waves = 16;
+    int pass_chunks = kStreamLdsInts / kSlot;
+    if (pass_chunks > chunks) pass_chunks = chunks;
+    const size_t lds = static_cast<size_t>(pass_chunks) * kSlot * sizeof(int);
     if (chunk_ints)
-        hipLaunchKernelGGL((dot_mfma_stream_kernel<NT, true>), grid, dim3(waves * 64), 0, st, A8, qscale, stride,
-                           reinterpret_cast<const unsigned long long*>(B), Bw, chunks, R, Q, down_shift, scale_inv,
-                           R_total, out, chunk_ints);
+        hipLaunchKernelGGL((dot_mfma_stream_kernel<NT, KT, true>), grid, dim3(waves * 64), lds, st, A8, qscale, stride,
+                           reinterpret_cast<const unsigned long long*>(B), Bw, chunks, pass_chunks, R, Q, down_shift,
+                           scale_inv, R_total, out, chunk_ints);
     else
-        hipLaunchKernelGGL((dot_mfma_stream_kernel<NT, false>), grid, dim3(waves * 64), 0, st, A8, qscale, stride,
-                           reinterpret_cast<const unsigned long long*>(B), Bw, chunks, R, Q, down_shift, scale_inv,
-                           R_total, out, chunk_ints);
+        hipLaunchKernelGGL((dot_mfma_stream_kernel<NT, KT, false>), grid, dim3(waves * 64), lds, st, A8, qscale, stride,
+                           reinterpret_cast<const unsigned long long*>(B), Bw, chunks, pass_chunks, R, Q, down_shift,
+                           scale_inv, R_total, out, chunk_ints);
 }
 
 template <bool kTiled>
@@ -1105,8 +1128,12 @@ extern "C" int bsi_hip_dot(const uint64_t* A, const int8_t* A_ints8, const float
         const int down_shift = 16 - Sa - Sb;
         const bool tiled = (b_layout == BSI_LAYOUT_TILED16);
         if (Sb == 6 && tiled && Q <= kStreamMaxQ) {
-            if (Q <= 16) launch_mfma_stream<1>(A8, A_chunk_scales, A_scale_stride, B, Bw, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, st);
-            else launch_mfma_stream<2>(A8, A_chunk_scales, A_scale_stride, B, Bw, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, st);
+            // two key tiles per workgroup halve the query re-reads once there are enough tiles to fill the GPU
+            const bool two = (R + 15) / 16 >= 1024;
+#define BSI_STREAM_ARGS A8, A_chunk_scales, A_scale_stride, B, Bw, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, st
+            if (Q <= 16) { if (two) launch_mfma_stream<1, 2>(BSI_STREAM_ARGS); else launch_mfma_stream<1, 1>(BSI_STREAM_ARGS); }
+            else { if (two) launch_mfma_stream<2, 2>(BSI_STREAM_ARGS); else launch_mfma_stream<2, 1>(BSI_STREAM_ARGS); }
+#undef BSI_STREAM_ARGS
             BSI_LAUNCH_CHECK("dot_mfma_stream_kernel");
             return BSI_OK;
         }

@@ -319,6 +319,8 @@ DOT_SHAPES = [
     (17, 50, 1024, "randn"),      # two query tiles of the few-rows kernel, ragged in both
     (32, 33, 8704, "relu"),       # 34 chunks: more than one pass of the few-rows kernel with two query tiles
     (3, 20, 16640, "randn"),      # 65 chunks: more than one pass with one query tile
+    (3, 16400, 256, "randn"),     # many key tiles: two per workgroup in the few-rows kernel, last tile ragged
+    (20, 16390, 512, "relu"),     # the same with two query tiles
 ]
 
 
