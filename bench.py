@@ -64,10 +64,11 @@ def main() -> int:
     stream = torch.cuda.current_stream().cuda_stream
     scale_inv = 1.0 / 10.0 ** 4
 
+    kptr, klayout = bsi_ops.key_operand(kcap, Q, SA, core)
+
     def dot_args():
         return (qcap.words.data_ptr(), qcap.ints8.data_ptr(), qcap.chunk_scales.data_ptr(), chunks, SA, W,
-                kcap.words.data_ptr(), kcap.layout, kcap.slice_weights.data_ptr(), SB, R, Q, scale_inv, R,
-                out.data_ptr())
+                kptr, klayout, kcap.slice_weights.data_ptr(), SB, R, Q, scale_inv, R, out.data_ptr())
 
     def step():
         _lib.check(_lib.lib.bsi_hip_dot(*dot_args(), None, core, None, 0, stream), "bsi_hip_dot")
@@ -135,7 +136,7 @@ def main() -> int:
                       if used_core == "mfma" else "u32 and/popcount -> int32 per chunk, fp32 fmaf chunk-scale epilogue",
         "data": "synthetic",
         "config": {"workload": "FC1-like fixed76 chunk-scale dot Q512 R8192 D2048, 0.1% outlier columns x20, dec=2",
-                   "core": used_core, "key_layout": "tiled16" if kcap.layout else "canonical",
+                   "core": used_core, "key_layout": {0: "canonical planes", 1: "tiled16 planes", 2: "cached int8 image of the planes"}[klayout],
                    "algorithmic_bytes": alg_bytes, "bit_ops": bit_ops},
         "roofline": roof,
     }

@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(_HERE, "libbsi_hip.so")
 BSI_OK = 0
 DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
 CORE_AUTO, CORE_VALU, CORE_MFMA = 0, 1, 2
-LAYOUT_CANONICAL, LAYOUT_TILED16 = 0, 1
+LAYOUT_CANONICAL, LAYOUT_TILED16, LAYOUT_INT8 = 0, 1, 2
 
 _vp = ctypes.c_void_p
 _i = ctypes.c_int

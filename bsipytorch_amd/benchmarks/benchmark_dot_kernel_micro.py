@@ -40,8 +40,9 @@ def run(Q, R, D, decimal_places=2, compress_threshold=0.5, warmup=10, iters=50, 
     ws_bytes = 0 if use_ints8 else int(_lib.lib.bsi_hip_dot_workspace_bytes(Q, W, code))
     ws = torch.empty((max(ws_bytes, 16),), dtype=torch.uint8, device="cuda")
     st = torch.cuda.current_stream().cuda_stream
+    kptr, klayout = bsi_ops.key_operand(kcap, Q, qcap.Sa, code)
     args = (qcap.words.data_ptr(), qcap.ints8.data_ptr() if use_ints8 else None, scales.data_ptr(), stride, qcap.Sa, W,
-            kcap.words.data_ptr(), kcap.layout, kcap.slice_weights.data_ptr(), kcap.Sb, R, Q, 1.0 / 10.0 ** (2 * decimal_places),
+            kptr, klayout, kcap.slice_weights.data_ptr(), kcap.Sb, R, Q, 1.0 / 10.0 ** (2 * decimal_places),
             R, out.data_ptr(), code, ws.data_ptr(), ws_bytes)
     us = ctypes.c_float(0.0)
     if warmup > 0:
@@ -50,7 +51,7 @@ def run(Q, R, D, decimal_places=2, compress_threshold=0.5, warmup=10, iters=50, 
     t = float(us.value) * 1e-6
     bit_ops = 2.0 * qcap.Sa * kcap.Sb * Q * R * D
     alg_bytes = Q * qcap.Sa * W * 8 + Q * chunks * 4 + R * kcap.Sb * W * 8 + R * 4 + Q * R * 4
-    return {"Q": Q, "R": R, "D": D, "core": core, "layout": "tiled16" if kcap.layout else "canonical",
+    return {"Q": Q, "R": R, "D": D, "core": core, "layout": {0: "canonical", 1: "tiled16", 2: "int8 image"}[klayout],
             "avg_dot_us": t * 1e6, "dot_q_us": t * 1e6 / Q, "dot_s_ns": t * 1e9 / (Q * R),
             "effective_bitop_TOPS": bit_ops / t / 1e12, "int8_TOPS": 2.0 * Q * R * D / t / 1e12,
             "algorithmic_GBps": alg_bytes / t / 1e9, "key_plane_GBps": key_bytes / t / 1e9, "iters": iters}

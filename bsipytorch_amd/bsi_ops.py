@@ -78,6 +78,7 @@ def _flags() -> dict:
         dot_debug=(_env_int("BSI_DOT_DEBUG", 0) or 0) != 0,
         core={"auto": _lib.CORE_AUTO, "valu": _lib.CORE_VALU, "mfma": _lib.CORE_MFMA}.get(core, _lib.CORE_AUTO),
         tiled=(layout != "canonical"),
+        key_image=(_env_int("BSI_KEY_INT8_IMAGE", 1) or 0) != 0,
     )
     return _flag_cache
 
@@ -131,6 +132,7 @@ class PrebuiltBSIKeysCUDA(_Capsule):
     def __init__(self):
         self.words: torch.Tensor = None          # canonical [R, Sb, W] or tiled [ceil(R/16), chunks, Sb, 64]
         self.layout = _lib.LAYOUT_CANONICAL
+        self.ints8: Optional[torch.Tensor] = None  # cached int8 image [R, chunks*256] of the same integers, or None
         self.slice_weights: torch.Tensor = None  # [R, Sb] float32
         self.shifts: torch.Tensor = None         # [R] int32
         self.Sb = 0
@@ -419,6 +421,11 @@ def build_bsi_keys_cuda(K: torch.Tensor, decimal_places: int, compress_threshold
     h.shifts = shifts
     h.slice_weights = (_slice_weights(h.Sb, 0, True, dev).unsqueeze(0) * scales.unsqueeze(1)).contiguous()
     total_bytes = words.numel() * 8
+    if f["key_image"] and R > 0 and 2 <= h.Sb <= 8:
+        # compute-bound shapes contract this image on the matrix cores; the planes stay the stored form
+        h.ints8 = torch.empty((R, ((h.W + 3) // 4) * 256), dtype=torch.int8, device=dev)
+        check(lib.bsi_hip_planes_to_int8(words.data_ptr(), R, h.Sb, h.W, h.ints8.data_ptr(), _stream()),
+              "bsi_hip_planes_to_int8")
     if f["tiled"] and R > 0:
         chunks = (h.W + 3) // 4
         tiled = torch.empty(((R + 15) // 16, chunks, h.Sb, 64), dtype=torch.int64, device=dev)
@@ -436,6 +443,7 @@ def build_bsi_keys_cuda(K: torch.Tensor, decimal_places: int, compress_threshold
 
 _DOT_DEBUG_PRINTED = [False]
 _workspace: dict = {}
+_FEW_ROWS_MAX_Q = 32  # up to here the dot streams the packed planes (bandwidth-bound); above, the int8 image
 
 
 def _get_workspace(nbytes: int, dev) -> Optional[torch.Tensor]:
@@ -454,6 +462,14 @@ def _scale_inv(dec_q: int, dec_k: int) -> float:
     return (1.0 / (10.0 ** total)) if total > 0 else 1.0
 
 
+def key_operand(keys: "PrebuiltBSIKeysCUDA", Q: int, Sa: int, core: int):
+    """(device pointer, layout code) of the key representation the dot should read for Q query rows:
+    the packed planes while the call is bound by streaming them, the cached int8 image above."""
+    if keys.ints8 is not None and core != _lib.CORE_VALU and Q > _FEW_ROWS_MAX_Q and 2 <= Sa <= 8:
+        return keys.ints8.data_ptr(), _lib.LAYOUT_INT8
+    return keys.words.data_ptr(), keys.layout
+
+
 def _dot(words, ints8, scales, scale_stride, Sa, W, keys: PrebuiltBSIKeysCUDA, Q, decimals_q, chunk_ints=None, core=None):
     f = _flags()
     dev = words.device
@@ -469,8 +485,9 @@ def _dot(words, ints8, scales, scale_stride, Sa, W, keys: PrebuiltBSIKeysCUDA, Q
     if prof:
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
+    kptr, klayout = key_operand(keys, Q, Sa, core)
     check(lib.bsi_hip_dot(words.data_ptr(), _ptr(ints8), scales.data_ptr(), scale_stride, Sa, W,
-                          keys.words.data_ptr(), keys.layout, keys.slice_weights.data_ptr(), keys.Sb, R, Q,
+                          kptr, klayout, keys.slice_weights.data_ptr(), keys.Sb, R, Q,
                           _scale_inv(decimals_q, keys.decimals), R, out.data_ptr(), _ptr(chunk_ints), core,
                           _ptr(ws), ws_bytes, _stream()), "bsi_hip_dot")
     ns = 0
@@ -481,7 +498,7 @@ def _dot(words, ints8, scales, scale_stride, Sa, W, keys: PrebuiltBSIKeysCUDA, Q
     if f["dot_debug"] and not _DOT_DEBUG_PRINTED[0]:
         _DOT_DEBUG_PRINTED[0] = True
         print(f"[BSI_DOT] core={core} Sa={Sa} Sb={keys.Sb} Q={Q} R={R} W64={W} chunks={(W + 3) // 4} "
-              f"layout={keys.layout} ints8={'yes' if ints8 is not None else 'no'}", file=sys.stderr)
+              f"layout={klayout} ints8={'yes' if ints8 is not None else 'no'}", file=sys.stderr)
     return out, ns
 
 

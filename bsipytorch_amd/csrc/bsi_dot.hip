@@ -666,6 +666,270 @@ __global__ __launch_bounds__(kWsBlock) void dot_mfma_ws_kernel(
     }
 }
 
+// ------------------------------------------------------------------ MFMA core on the cached int8 key image
+//
+// Compute-bound shapes (hundreds of query rows) pay for the plane -> int8 recombination of the keys
+// on the vector ALU in every workgroup that touches a key tile.  A keyset can therefore carry,
+// next to its packed planes, the recombined int8 image of the same integers (built once by
+// bsi_hip_planes_to_int8, 1 byte per weight); this kernel contracts that image with the int8
+// query image.
+//   * workgroup = 128 keys x 128 queries over all chunks; 8 MFMA waves of 64 keys x 32 queries
+//     and 4 loader waves (one per SIMD).  Only the loader waves issue global loads: a wave that
+//     issues them blocks while the memory queue is full, which the MFMA waves must never do;
+//   * LDS is a ring of four half-chunk stages (keys 128 x 128 B + queries 128 x 128 B = 32 KiB
+//     each), filled by buffer loads that write LDS directly (a loader wave issues 4 + 4 per
+//     stage, 1 KiB each); the 16-byte columns of a row are XOR-swizzled with (row >> 1) & 7 so
+//     that the 16 rows a ds_read_b128 touches hit distinct banks;
+//   * loads of half h+3 are issued when half h starts; the wait before the barrier that ends half
+//     h only covers the loads of half h+1, so two stages stay in flight across barriers;
+//   * the fp32 epilogue of chunk c-1 (one cvt + one fma per output and chunk, in chunk order)
+//     is interleaved element by element with the MFMAs of chunk c (two accumulator sets).
+typedef __amdgpu_buffer_rsrc_t bsi_rsrc;
+__device__ __forceinline__ bsi_rsrc make_rsrc(const void* base, size_t bytes) {
+    const size_t capped = bytes > 0x7FFFFFFFull ? 0x7FFFFFFFull : bytes;
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, static_cast<int>(capped), 0x00020000);
+}
+// 64 lanes x 16 bytes from `r` (byte offset lane_off per lane + wave_off) to 1 KiB of LDS at dst (wave-uniform)
+__device__ __forceinline__ void load16_to_lds(bsi_rsrc r, uint32_t lane_off, uint32_t wave_off, unsigned char* dst) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r, BSI_LDS_PTR(dst), 16, static_cast<int>(lane_off),
+                                             static_cast<int>(wave_off), 0, 0);
+}
+
+constexpr int kI8Consumers = 8;                     // MFMA waves: 64 keys x 32 queries each
+constexpr int kI8Block = (kI8Consumers + 4) * 64;   // + 4 loader waves
+constexpr int kI8ScaleBytes = 4 * 4 * 256;          // chunk scales: ring of 4 chunks x 4 loader regions x 64 floats
+constexpr int kI8Operand = 128 * 128;               // bytes of one operand tile of one half-chunk
+constexpr int kI8Stage = 2 * kI8Operand;            // keys then queries
+constexpr int kI8Stages = 4;
+
+// One half-chunk (two k-steps) of an MFMA wave: 16 MFMAs into `acc`, 12 operand reads, and 16
+// epilogue elements of the previous chunk (held in `prev`).  kHalf: first or second half of the chunk.
+template <int kHalf, bool kInts>
+__device__ __forceinline__ void i8_consume_half(const unsigned char* __restrict__ krow,
+                                                const unsigned char* __restrict__ qrow, const int (&pcol)[2],
+                                                v4i (&acc)[4][2], const v4i (&prev)[4][2], float (&accf)[4][2][4],
+                                                const float (&qs_prev)[2], int* __restrict__ ints_prev,
+                                                const int64_t (&int_off)[4][2], const int (&int_rows)[4],
+                                                int down_shift, int chunks) {
+    v4i ka[2][4], qb[2][2];
+    // operands of the first k-step, in the order its MFMAs need them
+    ka[0][0] = *reinterpret_cast<const v4i*>(krow + pcol[0]);
+    qb[0][0] = *reinterpret_cast<const v4i*>(qrow + pcol[0]);
+    qb[0][1] = *reinterpret_cast<const v4i*>(qrow + 16 * 128 + pcol[0]);
+    ka[0][1] = *reinterpret_cast<const v4i*>(krow + 16 * 128 + pcol[0]);
+    ka[0][2] = *reinterpret_cast<const v4i*>(krow + 32 * 128 + pcol[0]);
+    ka[0][3] = *reinterpret_cast<const v4i*>(krow + 48 * 128 + pcol[0]);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                const int ks = kHalf * 2 + kk, t = a * 2 + b;
+                const v4i c0 = (ks == 0) ? (v4i){0, 0, 0, 0} : acc[a][b];
+                acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ka[kk][a], qb[kk][b], c0, 0, 0, 0);
+                {
+                    const int idx = ks * 8 + t, tt = idx >> 2, e = idx & 3, ea = tt >> 1, eb = tt & 1;
+                    accf[ea][eb][e] = fmaf(static_cast<float>(prev[ea][eb][e]), qs_prev[eb], accf[ea][eb][e]);
+                    if (kInts && ints_prev != nullptr && int_off[ea][eb] >= 0 && e < int_rows[ea])
+                        ints_prev[int_off[ea][eb] + static_cast<int64_t>(e) * chunks] = prev[ea][eb][e] >> down_shift;
+                }
+                if (kk == 0) {  // operands of the second k-step, one read behind each of the first six MFMAs
+                    if (t == 0) ka[1][0] = *reinterpret_cast<const v4i*>(krow + pcol[1]);
+                    if (t == 1) qb[1][0] = *reinterpret_cast<const v4i*>(qrow + pcol[1]);
+                    if (t == 2) qb[1][1] = *reinterpret_cast<const v4i*>(qrow + 16 * 128 + pcol[1]);
+                    if (t == 3) ka[1][1] = *reinterpret_cast<const v4i*>(krow + 16 * 128 + pcol[1]);
+                    if (t == 4) ka[1][2] = *reinterpret_cast<const v4i*>(krow + 32 * 128 + pcol[1]);
+                    if (t == 5) ka[1][3] = *reinterpret_cast<const v4i*>(krow + 48 * 128 + pcol[1]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+    }
+}
+
+template <bool kInts>
+__global__ __launch_bounds__(kI8Block) void dot_mfma_i8_kernel(
+    const int8_t* __restrict__ A8, const float* __restrict__ qscale, int qscale_stride,
+    const int8_t* __restrict__ K8,  // int8 key image [R, chunks * 256]
+    const float* __restrict__ Bw, int Sb, int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv,
+    int64_t R_total, float* __restrict__ out, int* __restrict__ chunk_ints) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];  // kI8Stages * kI8Stage + kI8ScaleBytes
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int64_t r0 = static_cast<int64_t>(blockIdx.x) * 128;
+    const int64_t q0 = static_cast<int64_t>(blockIdx.y) * 128;
+    const size_t rowbytes = static_cast<size_t>(chunks) * 256;
+    const int halves = chunks * 2;
+    unsigned char* const scale_lds = lds + kI8Stages * kI8Stage;  // ring of four chunks x 4 loader waves x 64 floats
+
+    if (wave >= kI8Consumers) {
+        // ---- loader wave lw: rows 32 lw .. 32 lw + 31 of both operand tiles of every stage (4 + 4 loads of
+        // 1 KiB), plus the chunk scales of 64 queries once per chunk.
+        const int lw = wave - kI8Consumers;
+        const bsi_rsrc rk = make_rsrc(K8 + static_cast<size_t>(r0) * rowbytes, static_cast<size_t>(R - r0) * rowbytes);
+        const bsi_rsrc rq = make_rsrc(A8 + static_cast<size_t>(q0) * rowbytes, static_cast<size_t>(Q - q0) * rowbytes);
+        const bsi_rsrc rs = make_rsrc(qscale + q0 * qscale_stride, static_cast<size_t>(Q - q0) * qscale_stride * 4);
+        uint32_t koff[4], qoff[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int rowl = (4 * lw + i) * 8 + (lane >> 3);                                 // tile row this lane fetches
+            const uint32_t col = static_cast<uint32_t>((lane & 7) ^ ((rowl >> 1) & 7)) * 16;  // logical column landing here
+            const int64_t kr = (r0 + rowl < R) ? rowl : (R - 1 - r0);                         // past the end: clamp (never stored)
+            const int64_t qr = (q0 + rowl < Q) ? rowl : (Q - 1 - q0);
+            koff[i] = static_cast<uint32_t>(kr * rowbytes) + col;
+            qoff[i] = static_cast<uint32_t>(qr * rowbytes) + col;
+        }
+        // scales: loader wave lw fetches queries 64 (lw & 1) + lane (the two pairs of waves fetch the same
+        // data into their own regions so that every loader wave has the same number of loads in flight)
+        const int sq = (lw & 1) * 64 + lane;
+        const uint32_t soff = static_cast<uint32_t>(((q0 + sq < Q) ? sq : (Q - 1 - q0)) * qscale_stride * 4);
+        const int sstep = (qscale_stride == 1) ? 0 : 4;
+        auto issue = [&](int h) {  // stage of half-chunk h (clamped to the last) into its ring slot
+            const int hc = h < halves ? h : halves - 1;
+            unsigned char* slot = lds + (h & 3) * kI8Stage + (4 * lw) * 1024;
+            const uint32_t so = static_cast<uint32_t>(hc) * 128;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) load16_to_lds(rk, koff[i], so, slot + i * 1024);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) load16_to_lds(rq, qoff[i], so, slot + kI8Operand + i * 1024);
+            if (h & 1) {  // with the second half of chunk c = h / 2: its scales
+                const int c = hc >> 1;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, BSI_LDS_PTR(scale_lds + ((c & 3) * 4 + lw) * 256), 4,
+                                                         static_cast<int>(soff), c * sstep, 0, 0);
+            }
+        };
+        issue(0);
+        issue(1);
+        issue(2);
+        asm volatile("s_waitcnt vmcnt(17)" ::: "memory");  // stage 0 landed (stage 1 + scales + stage 2 may be in flight)
+        lds_barrier();
+        for (int h = 0; h < halves; ++h) {
+            issue(h + 3);  // its slot was released by the barrier that ended half h - 1
+            // stage h + 1 (and the scales issued right behind it) landed; stages h + 2, h + 3 and one
+            // scale load, 17 instructions, may still be in flight
+            asm volatile("s_waitcnt vmcnt(17)" ::: "memory");
+            lds_barrier();
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still be writing LDS when the workgroup ends
+        return;
+    }
+
+    // ---- MFMA waves
+    const int wr = wave & 1, wq = wave >> 1;  // 64-key half, 32-query quarter
+    const int ln = lane & 15, lg = lane >> 4;
+    const int krow_off = (wr * 64 + ln) * 128;
+    const int qrow_off = kI8Operand + (wq * 32 + ln) * 128;
+    int pcol[2];
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) pcol[kk] = ((kk * 4 + lg) ^ (ln >> 1)) * 16;
+    float accf[4][2][4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) accf[a][b][e] = 0.0f;
+    v4i acc0[4][2], acc1[4][2];
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b) acc0[a][b] = acc1[a][b] = (v4i){0, 0, 0, 0};
+    // the MFMA accumulators hold 2^down_shift times the integer dot; the chain runs on them unscaled
+    // (a power of two commutes with every rounding) and the factor is taken out once at the end
+    const float down = __uint_as_float(static_cast<uint32_t>(127 - down_shift) << 23);
+    int64_t int_off[4][2];
+    int int_rows[4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+        const int64_t r = r0 + wr * 64 + a * 16 + lg * 4;
+        int_rows[a] = static_cast<int>((R - r) < 4 ? (R - r) : 4);
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            const int64_t q = q0 + wq * 32 + b * 16 + ln;
+            int_off[a][b] = (kInts && q < Q && r < R) ? (q * R + r) * chunks : -1;
+        }
+    }
+    // chunk scales of the lane's two query columns, from the loaders' ring: region (wq >> 1) holds queries
+    // 64 (wq >> 1) .. + 63
+    const unsigned char* sread = scale_lds + (wq >> 1) * 256 + ((wq & 1) * 32 + ln) * 4;
+    float qsa[2] = {0.0f, 0.0f}, qsb[2] = {0.0f, 0.0f};  // even / odd chunks
+#define BSI_I8_SCALES(dst, c)                                                            \
+    {                                                                                    \
+        dst[0] = *reinterpret_cast<const float*>(sread + ((c) & 3) * 1024);              \
+        dst[1] = *reinterpret_cast<const float*>(sread + ((c) & 3) * 1024 + 64);         \
+    }
+#define BSI_I8_HALF(kHalf, slot, acc, prev, qs, ip)                                                                   \
+    i8_consume_half<kHalf, kInts>(lds + (slot) * kI8Stage + krow_off, lds + (slot) * kI8Stage + qrow_off, pcol, acc,   \
+                                  prev, accf, qs, ip, int_off, int_rows, down_shift, chunks);                         \
+    lds_barrier();
+
+    lds_barrier();  // stage 0 is there
+    int c = 0;
+    for (; c + 1 < chunks; c += 2) {
+        int* const ip = c > 0 ? chunk_ints + (c - 1) : nullptr;
+        // even chunk c -> acc0, ring slots 0 and 1; epilogue of chunk c-1 (acc1, scales qsb)
+        BSI_I8_HALF(0, 0, acc0, acc1, qsb, ip);
+        BSI_I8_HALF(1, 1, acc0, acc1, qsb, ip);
+        BSI_I8_SCALES(qsa, c);  // landed with the second half of chunk c
+        // odd chunk c+1 -> acc1, ring slots 2 and 3; epilogue of chunk c (acc0, scales qsa)
+        BSI_I8_HALF(0, 2, acc1, acc0, qsa, chunk_ints + c);
+        BSI_I8_HALF(1, 3, acc1, acc0, qsa, chunk_ints + c);
+        BSI_I8_SCALES(qsb, c + 1);
+    }
+    bool last_in_acc0 = false;
+    if (c < chunks) {  // odd number of chunks: one more even chunk; its halves sit in slots 0 and 1
+        int* const ip = c > 0 ? chunk_ints + (c - 1) : nullptr;
+        BSI_I8_HALF(0, 0, acc0, acc1, qsb, ip);
+        BSI_I8_HALF(1, 1, acc0, acc1, qsb, ip);
+        BSI_I8_SCALES(qsa, c);
+        last_in_acc0 = true;
+    }
+#undef BSI_I8_SCALES
+#undef BSI_I8_HALF
+    // epilogue of the last chunk
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int v = last_in_acc0 ? acc0[a][b][e] : acc1[a][b][e];
+                const float qsv = last_in_acc0 ? qsa[b] : qsb[b];
+                accf[a][b][e] = fmaf(static_cast<float>(v), qsv, accf[a][b][e]);
+                if (kInts && int_off[a][b] >= 0 && e < int_rows[a])
+                    chunk_ints[int_off[a][b] + static_cast<int64_t>(e) * chunks + (chunks - 1)] = v >> down_shift;
+            }
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+        const int64_t rb = r0 + wr * 64 + a * 16 + lg * 4;
+        float bs[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) bs[e] = (rb + e < R) ? Bw[(rb + e) * Sb] : 0.0f;
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) accf[a][b][e] *= down;
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            const int64_t q = q0 + wq * 32 + b * 16 + ln;
+            if (q >= Q) continue;
+            float* dst = out + static_cast<size_t>(q) * R_total + rb;
+            if (rb + 3 < R && ((reinterpret_cast<uintptr_t>(dst) & 15) == 0)) {
+                *reinterpret_cast<float4*>(dst) =
+                    make_float4((accf[a][b][0] * bs[0]) * scale_inv, (accf[a][b][1] * bs[1]) * scale_inv,
+                                (accf[a][b][2] * bs[2]) * scale_inv, (accf[a][b][3] * bs[3]) * scale_inv);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (rb + e < R) dst[e] = (accf[a][b][e] * bs[e]) * scale_inv;
+            }
+        }
+    }
+}
+
 // ------------------------------------------------------------------ MFMA core, few query rows
 //
 // Decode-like shapes (a handful of query rows against a large key matrix) are bound by reading the
@@ -1021,6 +1285,27 @@ static void launch_mfma_ws(const int8_t* A8, const float* qscale, int stride, co
                            R_total, out, chunk_ints);
 }
 
+static void launch_mfma_i8(const int8_t* A8, const float* qscale, int stride, const int8_t* K8, const float* Bw, int Sb,
+                           int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv, int64_t R_total,
+                           float* out, int32_t* chunk_ints, hipStream_t st) {
+    const dim3 grid(static_cast<unsigned>((R + 127) / 128), static_cast<unsigned>((Q + 127) / 128));
+    constexpr int kLds = kI8Stages * kI8Stage + kI8ScaleBytes;
+    static bool configured = false;
+    if (!configured) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dot_mfma_i8_kernel<true>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dot_mfma_i8_kernel<false>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+        configured = true;
+    }
+    if (chunk_ints)
+        hipLaunchKernelGGL((dot_mfma_i8_kernel<true>), grid, dim3(kI8Block), kLds, st, A8, qscale, stride, K8, Bw, Sb,
+                           chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints);
+    else
+        hipLaunchKernelGGL((dot_mfma_i8_kernel<false>), grid, dim3(kI8Block), kLds, st, A8, qscale, stride, K8, Bw, Sb,
+                           chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints);
+}
+
 template <int NT, int KT>
 static void launch_mfma_stream(const int8_t* A8, const float* qscale, int stride, const uint64_t* B, const float* Bw,
                                int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv, int64_t R_total,
@@ -1100,7 +1385,8 @@ extern "C" int bsi_hip_dot(const uint64_t* A, const int8_t* A_ints8, const float
     BSI_REQUIRE(W64 >= 1, "W64 must be >= 1");
     BSI_REQUIRE(Sa >= 1 && Sa <= 16 && Sb >= 1 && Sb <= 16, "Sa and Sb must be in [1, 16]");
     BSI_REQUIRE(R_total >= R, "R_total must be >= R");
-    BSI_REQUIRE(b_layout == BSI_LAYOUT_CANONICAL || b_layout == BSI_LAYOUT_TILED16, "unknown key layout %d", b_layout);
+    BSI_REQUIRE(b_layout == BSI_LAYOUT_CANONICAL || b_layout == BSI_LAYOUT_TILED16 || b_layout == BSI_LAYOUT_INT8,
+                "unknown key layout %d", b_layout);
     if (Q == 0 || R == 0) return BSI_OK;
     const int chunks = (W64 + 3) / 4;
     BSI_REQUIRE(A_chunk_scales != nullptr, "A_chunk_scales is required (pass a [Q,1] array of row scales if there are no chunk scales)");
@@ -1126,6 +1412,13 @@ extern "C" int bsi_hip_dot(const uint64_t* A, const int8_t* A_ints8, const float
             A8 = static_cast<const int8_t*>(workspace);
         }
         const int down_shift = 16 - Sa - Sb;
+        if (b_layout == BSI_LAYOUT_INT8) {
+            BSI_REQUIRE((reinterpret_cast<uintptr_t>(B) & 15) == 0, "int8 key image must be 16-byte aligned");
+            launch_mfma_i8(A8, A_chunk_scales, A_scale_stride, reinterpret_cast<const int8_t*>(B), Bw, Sb, chunks, R, Q,
+                           down_shift, scale_inv, R_total, out, chunk_ints, st);
+            BSI_LAUNCH_CHECK("dot_mfma_i8_kernel");
+            return BSI_OK;
+        }
         const bool tiled = (b_layout == BSI_LAYOUT_TILED16);
         if (Sb == 6 && tiled && Q <= kStreamMaxQ) {
             // two key tiles per workgroup halve the query re-reads once there are enough tiles to fill the GPU
@@ -1154,6 +1447,7 @@ extern "C" int bsi_hip_dot(const uint64_t* A, const int8_t* A_ints8, const float
     }
 
     if (core != BSI_CORE_VALU) return fail(BSI_ERR_INVALID, "unknown core %d", core);
+    if (b_layout == BSI_LAYOUT_INT8) return fail(BSI_ERR_UNSUPPORTED, "the popcount core reads key planes, not the int8 image");
     BSI_REQUIRE(A != nullptr, "VALU core needs the query planes");
     if (Sa == 7 && Sb == 6) {
         if (b_layout == BSI_LAYOUT_TILED16)

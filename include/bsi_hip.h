@@ -45,6 +45,7 @@ extern "C" {
 /* Layout of the key planes handed to the dot. */
 #define BSI_LAYOUT_CANONICAL 0 /* [R, Sb, W64] */
 #define BSI_LAYOUT_TILED16 1   /* [ceil(R/16), chunks, Sb, 64, 1] words: see bsi_hip_tile_key_planes */
+#define BSI_LAYOUT_INT8 2      /* int8 [R, chunks*256]: the recombined image bsi_hip_planes_to_int8 writes */
 
 const char* bsi_hip_version(void);
 const char* bsi_hip_last_error(void);

@@ -287,7 +287,11 @@ def _run_dot(hip, qb, kb, Q, R, W, Sa, Sb, core, tiled, with_ints8, want_ints=Tr
     stride = chunks if qb["chunk_scale"] else 1
     B = dev(kb["words"])
     layout = 0
-    if tiled:
+    if tiled == "int8":   # the cached int8 image of the key integers
+        Bi = torch.full((R, chunks * 256), 77, dtype=torch.int8, device="cuda")
+        hip.check(L.bsi_hip_planes_to_int8(B.data_ptr(), R, Sb, W, Bi.data_ptr(), st()), "key image")
+        B, layout = Bi, 2
+    elif tiled:
         Bt = torch.full((((R + 15) // 16) * chunks * Sb * 64,), -1, dtype=torch.int64, device="cuda")
         hip.check(L.bsi_hip_tile_key_planes(B.data_ptr(), R, Sb, W, Bt.data_ptr(), st()), "tile")
         B, layout = Bt, 1
@@ -326,7 +330,7 @@ DOT_SHAPES = [
 
 @pytest.mark.parametrize("Q,R,d,kind", DOT_SHAPES)
 @pytest.mark.parametrize("core,tiled,ints8", [(1, False, False), (1, True, False), (2, False, True), (2, True, False),
-                                              (0, True, True)])
+                                              (0, True, True), (2, "int8", True), (0, "int8", False)])
 def test_dot_bit_exact(hip, oracle, Q, R, d, kind, core, tiled, ints8):
     x, k, qb, kb, want_ints, want_out = _oracle_case(oracle, Q, R, d, seed=Q + R + d, qkind=kind)
     W = (d + 63) // 64
@@ -337,14 +341,18 @@ def test_dot_bit_exact(hip, oracle, Q, R, d, kind, core, tiled, ints8):
     # independent of the popcount form: the accumulators are the integer dot of the quantised values
     c0 = qb["ints"][:, :256] @ kb["ints"][:, :256].T
     np.testing.assert_array_equal(ints[:, :, 0], c0)
+    if core != 1:
+        # the production launch (no accumulator dump) is a different kernel instance: same floats
+        _, out2 = _run_dot(hip, qb, kb, Q, R, W, 7, 6, core, tiled, ints8, want_ints=False)
+        np.testing.assert_array_equal(out2, want_out)
 
 
 @pytest.mark.parametrize("Sa,Sb", [(8, 8), (5, 4), (2, 2), (7, 5), (3, 7)])
-@pytest.mark.parametrize("core", [1, 2])
-def test_dot_other_bit_widths(hip, oracle, Sa, Sb, core):
+@pytest.mark.parametrize("core,tiled", [(1, False), (2, True), (2, "int8")])
+def test_dot_other_bit_widths(hip, oracle, Sa, Sb, core, tiled):
     Q, R, d = 19, 35, 1024
     x, k, qb, kb, want_ints, want_out = _oracle_case(oracle, Q, R, d, seed=Sa * 10 + Sb, ksigma=0.05, bits_q=Sa, bits_k=Sb)
-    ints, out = _run_dot(hip, qb, kb, Q, R, 16, Sa, Sb, core, tiled=(core == 2), with_ints8=False)
+    ints, out = _run_dot(hip, qb, kb, Q, R, 16, Sa, Sb, core, tiled=tiled, with_ints8=False)
     np.testing.assert_array_equal(ints, want_ints)
     np.testing.assert_array_equal(out, want_out)
 
