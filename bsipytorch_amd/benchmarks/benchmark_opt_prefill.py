@@ -7,8 +7,8 @@ token ids are uniform random from a seed, and no accuracy is computed.
 
     python -m bsipytorch_amd.benchmarks.benchmark_opt_prefill --model opt-1.3b --seq_len 512
 
-Reports tokens/s of one prefill (batch 1), the share of the forward spent in the BSI dot kernels
-(device-event time per call, collected in a second pass with BSI_PROFILE=1 because per-call events
+Reports tokens/s of one prefill (batch 1), run eagerly and as a replayed HIP graph, the share of
+the forward spent in the BSI dot kernels (device-event time per call, collected in a second pass with BSI_PROFILE=1 because per-call events
 synchronise), the query-build time, and the dense fp32 forward of the same model for context.
 """
 from __future__ import annotations
@@ -119,7 +119,7 @@ def time_forward(model, input_ids, iters: int, warmup: int):
 
 
 def run(model_name="opt-1.3b", seq_len=512, batch=1, iters=5, warmup=2, decimal_places=2, compress_threshold=0.5,
-        seed=123, dense=True):
+        seed=123, dense=True, graph=True):
     from bsipytorch_amd import bsi_ops, linear
 
     assert torch.cuda.is_available(), "needs the GPU"
@@ -154,6 +154,41 @@ def run(model_name="opt-1.3b", seq_len=512, batch=1, iters=5, warmup=2, decimal_
     res["bsi_fwd_ms_min"] = best
     res["bsi_tokens_per_s"] = tokens / (med * 1e-3)
 
+    # pass 1b: the same forward captured once into a HIP graph and replayed (no host work per layer).
+    # Replays are checked against the eager logits, with eager work in between, as graph replays must be.
+    if graph:
+        with torch.no_grad():
+            eager = model(input_ids).clone()
+            linear._last_query_build.clear()
+            static_in = input_ids.clone()
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                for _ in range(2):
+                    model(static_in)
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            linear._last_query_build.clear()
+            hip_graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(hip_graph):
+                static_out = model(static_in)
+            linear._last_query_build.clear()
+            same = True
+            times = []
+            for _ in range(max(iters, 3)):
+                s_evt, e_evt = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                s_evt.record()
+                hip_graph.replay()
+                e_evt.record()
+                torch.cuda.synchronize()
+                times.append(s_evt.elapsed_time(e_evt))
+                same = same and bool(torch.equal(static_out, eager))
+                same = same and bool(torch.equal(model(input_ids), eager))  # eager work between replays
+            times.sort()
+            res["bsi_graph_fwd_ms"] = times[len(times) // 2]
+            res["bsi_graph_tokens_per_s"] = tokens / (times[len(times) // 2] * 1e-3)
+            res["graph_replays_match_eager"] = same
+
     # pass 2: per-call device events on the dot and the builder -> shares
     os.environ["BSI_PROFILE"] = "1"
     bsi_ops._reset_flag_cache()
@@ -187,9 +222,10 @@ def main():
     ap.add_argument("--compress_threshold", type=float, default=0.5)
     ap.add_argument("--seed", type=int, default=123)
     ap.add_argument("--no_dense", action="store_true")
+    ap.add_argument("--no_graph", action="store_true", help="skip the HIP-graph replay leg")
     a = ap.parse_args()
     print(json.dumps(run(a.model, a.seq_len, a.batch, a.iters, a.warmup, a.decimal_places, a.compress_threshold,
-                         a.seed, not a.no_dense)))
+                         a.seed, not a.no_dense, not a.no_graph)))
 
 
 if __name__ == "__main__":

@@ -211,12 +211,21 @@ def cuda_builder_version() -> str:
 CUDA_BUILDER_VERSION = cuda_builder_version()
 
 
+_slice_weight_cache: dict = {}
+
+
 def _slice_weights(S: int, offset: int, twos: bool, device) -> torch.Tensor:
-    # bsi_cuda.cpp:217-236
-    w = [float(2.0 ** (offset + i)) if offset + i >= 0 else 0.0 for i in range(S)]
-    if twos and S > 0:
-        w[S - 1] = -w[S - 1]
-    return torch.tensor(w, dtype=torch.float32, device=device)
+    # bsi_cuda.cpp:217-236; cached per device like make_slice_weights_cuda_cached (bsi_vector_cuda.cpp:48-88).
+    # Callers must not modify the returned tensor.
+    key = (int(S), int(offset), bool(twos), str(device))
+    t = _slice_weight_cache.get(key)
+    if t is None:
+        w = [float(2.0 ** (offset + i)) if offset + i >= 0 else 0.0 for i in range(S)]
+        if twos and S > 0:
+            w[S - 1] = -w[S - 1]
+        t = torch.tensor(w, dtype=torch.float32, device=device)
+        _slice_weight_cache[key] = t
+    return t
 
 
 def _as_build_input(x: torch.Tensor, device) -> torch.Tensor:
@@ -235,13 +244,17 @@ def _build_fixed(x2d: torch.Tensor, decimal_places: int, fixed_bits: int, chunk_
     Q, d = x2d.shape
     W = (d + 63) // 64 if d > 0 else 1
     chunks = (d + 255) // 256 if d > 0 else 0
-    words = torch.zeros((Q, fixed_bits, W), dtype=torch.int64, device=dev)
-    if chunk_scale:
-        shifts = torch.zeros((Q, chunks), dtype=torch.int32, device=dev)
-        scales = torch.ones((Q, chunks), dtype=torch.float32, device=dev)
+    if Q > 0 and d > 0:   # the build kernels write every word, shift and scale: no fill passes
+        alloc_i, alloc_f = torch.empty, torch.empty
     else:
-        shifts = torch.zeros((Q,), dtype=torch.int32, device=dev)
-        scales = torch.ones((Q,), dtype=torch.float32, device=dev)
+        alloc_i, alloc_f = torch.zeros, torch.ones
+    words = alloc_i((Q, fixed_bits, W), dtype=torch.int64, device=dev)
+    if chunk_scale:
+        shifts = alloc_i((Q, chunks), dtype=torch.int32, device=dev)
+        scales = alloc_f((Q, chunks), dtype=torch.float32, device=dev)
+    else:
+        shifts = alloc_i((Q,), dtype=torch.int32, device=dev)
+        scales = alloc_f((Q,), dtype=torch.float32, device=dev)
     ints8 = None
     if want_ints8 and fixed_bits <= 8 and Q > 0 and d > 0:
         ints8 = torch.empty((Q, ((W + 3) // 4) * 256), dtype=torch.int8, device=dev)
@@ -255,6 +268,22 @@ def _build_fixed(x2d: torch.Tensor, decimal_places: int, fixed_bits: int, chunk_
 def _require_fixed(bits: int, what: str) -> None:
     _check(bits > 0, f"{what}: BSI_FIXED_BITS*=0 selects the decimal (data-dependent slice count) builder, "
                      "which this build does not implement; unset it to use the fixed-bit path")
+
+
+_expanded_cache: dict = {}
+
+
+def _expanded_slice_weights(base: torch.Tensor, Q: int, bits: int, dev) -> torch.Tensor:
+    """[Q, bits] copies of the base slice weights; constant per (Q, bits, device), so built once
+    (the reference caches its slice weights the same way, bsi_vector_cuda.cpp:48-88)."""
+    key = (int(Q), int(bits), str(dev))
+    t = _expanded_cache.get(key)
+    if t is None:
+        if len(_expanded_cache) > 64:
+            _expanded_cache.clear()
+        t = base.unsqueeze(0).expand(Q, -1).contiguous()
+        _expanded_cache[key] = t
+    return t
 
 
 def _build_query_batch(q2d: torch.Tensor, decimal_places: int) -> PrebuiltBSIQueryBatchCUDA:
@@ -282,7 +311,7 @@ def _build_query_batch(q2d: torch.Tensor, decimal_places: int) -> PrebuiltBSIQue
     base = _slice_weights(f["bits_q"], 0, True, dev)
     h.words = words
     if chunk_scale:
-        h.slice_weights = base.unsqueeze(0).expand(Q, -1).contiguous()
+        h.slice_weights = _expanded_slice_weights(base, Q, f["bits_q"], dev)
         h.chunk_scales = scales
     else:
         h.slice_weights = (base.unsqueeze(0) * scales.unsqueeze(1)).contiguous()

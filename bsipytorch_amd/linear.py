@@ -17,6 +17,26 @@ import torch.nn as nn
 from . import bsi_ops
 
 
+# Layers fed by the same activation tensor (q_proj / k_proj / v_proj) share one query build: the last built
+# batch is kept with a reference to its input (so its address cannot be reused) and its version counter.
+_last_query_build: Dict[str, Any] = {}
+
+
+def _cached_query_build(batch_inputs: torch.Tensor, decimal_places: int, threshold: float, packed: bool):
+    use_cache = os.getenv("BSI_QUERY_CACHE", "1") != "0"
+    key = (batch_inputs.data_ptr(), tuple(batch_inputs.shape), batch_inputs.dtype, batch_inputs._version,
+           int(decimal_places), bool(packed))
+    if use_cache and _last_query_build.get("key") == key and _last_query_build.get("src") is not None:
+        return _last_query_build["cap"], True
+    if packed:
+        cap = bsi_ops.build_bsi_queries_cuda_batch_packed(batch_inputs, decimal_places, threshold)
+    else:
+        cap = bsi_ops.build_bsi_queries_cuda_batch(batch_inputs, decimal_places, threshold)
+    if use_cache:
+        _last_query_build.update(key=key, src=batch_inputs, cap=cap)
+    return cap, False
+
+
 class BSIQuantizedLinear(nn.Module):
     """Linear layer whose weight lives as BSI key planes (verify_accuracy_bsi.py:46-215)."""
 
@@ -88,18 +108,15 @@ class BSIQuantizedLinear(nn.Module):
 
         t0 = time.perf_counter_ns()
         use_packed = os.getenv("BSI_QUERY_PACKED", "1") != "0"
-        if use_packed:
-            qcap = bsi_ops.build_bsi_queries_cuda_batch_packed(batch_inputs, self.decimalPlaces,
-                                                               float(self.query_compress_threshold))
-        else:
-            qcap = bsi_ops.build_bsi_queries_cuda_batch(batch_inputs, self.decimalPlaces,
-                                                        float(self.query_compress_threshold))
+        qcap, reused = _cached_query_build(batch_inputs, self.decimalPlaces, float(self.query_compress_threshold),
+                                           use_packed)
         self.build_ns_total += time.perf_counter_ns() - t0
-        q_ns, p_ns, t_ns = bsi_ops.get_last_query_build_profile_cuda()
-        self.build_quantize_ns_total += int(q_ns)
-        self.build_pack_ns_total += int(p_ns)
-        self.build_kernel_ns_total += int(t_ns)
-        self.build_calls += 1
+        if not reused:
+            q_ns, p_ns, t_ns = bsi_ops.get_last_query_build_profile_cuda()
+            self.build_quantize_ns_total += int(q_ns)
+            self.build_pack_ns_total += int(p_ns)
+            self.build_kernel_ns_total += int(t_ns)
+            self.build_calls += 1
 
         if use_packed:
             scores, ns_total, ns_q, ns_s = bsi_ops.batch_dot_product_multiquery_cuda_batch_caps(qcap, self._bsi_keys_cuda)

@@ -555,6 +555,21 @@ def test_linear_drop_in(ops, oracle):
     assert blin.dot_calls == 3 and blin.dot_query_vectors_total == 54
     assert blin.weight_bsi_memory_bytes == 192 * 6 * 8 * 8 and blin.dot_ns_total == 0
 
+    # layers fed the same tensor share one query build; an in-place change of the tensor forces a new one
+    lin2 = torch.nn.Linear(512, 64, bias=False)
+    blin2 = BSIQuantizedLinear(lin2, decimalPlaces=2, compress_threshold=0.5)
+    xs = x.cuda().reshape(18, 512).contiguous()
+    b0, b1 = blin.build_calls, blin2.build_calls
+    ya, yb = blin(xs), blin2(xs)
+    assert blin.build_calls == b0 + 1 and blin2.build_calls == b1  # second layer reused the planes
+    kb2 = oracle.build_keys(lin2.weight.detach().numpy())
+    _, want2 = oracle.dot_fixed(qb["words"], qb["scales"], kb2["words"], kb2["scales"], oracle.scale_inv(2, 2))
+    assert torch.equal(yb.cpu(), torch.from_numpy(want2)) and torch.equal(ya, y.reshape(18, 192))
+    xs.mul_(2.0)
+    yc = blin2(xs)
+    assert blin2.build_calls == b1 + 1 and not torch.equal(yc, yb)
+    blin.dot_calls -= 1  # keep the call accounting below as it was
+
     class Tiny(torch.nn.Module):
         def __init__(self):
             super().__init__()
