@@ -15,6 +15,7 @@ BSI_OK = 0
 DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
 CORE_AUTO, CORE_VALU, CORE_MFMA = 0, 1, 2
 LAYOUT_CANONICAL, LAYOUT_TILED16, LAYOUT_INT8 = 0, 1, 2
+OPT_I8_SMALL_TILE_BELOW = 1
 
 _vp = ctypes.c_void_p
 _i = ctypes.c_int
@@ -45,6 +46,7 @@ PROTOTYPES = {
     "bsi_hip_ewah_decompress_batch": [_vp, _vp, _vp, _i, _i, _vp, _vp],
     "bsi_hip_tile_key_planes": [_vp, _i64, _i, _i, _vp, _vp],
     "bsi_hip_planes_to_int8": [_vp, _i64, _i, _i, _vp, _vp],
+    "bsi_hip_set_option": [_i, _i],
     "bsi_hip_dot_workspace_bytes": [_i64, _i, _i],
     "bsi_hip_dot": [_vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _i, _i64, _i64, _f, _i64, _vp, _vp, _i, _vp, _sz, _vp],
     "bsi_hip_dot_timed": [_vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _i, _i64, _i64, _f, _i64, _vp, _i, _vp, _sz, _i,

@@ -695,80 +695,90 @@ __device__ __forceinline__ void load16_to_lds(bsi_rsrc r, uint32_t lane_off, uin
                                              static_cast<int>(wave_off), 0, 0);
 }
 
-constexpr int kI8Consumers = 8;                     // MFMA waves: 64 keys x 32 queries each
-constexpr int kI8Block = (kI8Consumers + 4) * 64;   // + 4 loader waves
-constexpr int kI8ScaleBytes = 4 * 4 * 256;          // chunk scales: ring of 4 chunks x 4 loader regions x 64 floats
-constexpr int kI8Operand = 128 * 128;               // bytes of one operand tile of one half-chunk
-constexpr int kI8Stage = 2 * kI8Operand;            // keys then queries
-constexpr int kI8Stages = 4;
+// Tile configuration: T keys x T queries per workgroup (T = 128, or 64 for grids that would leave
+// most CUs without a workgroup), MFMA waves arranged 2 (keys) x kWavesN (queries), each WM x WN
+// tiles of 16 x 16; one loader wave per 32 rows.
+static int g_i8_small_tile_below = 100;  // workgroups of 128 x 128 below which 64 x 64 tiles are used (tunable)
 
-// One half-chunk (two k-steps) of an MFMA wave: 16 MFMAs into `acc`, 12 operand reads, and 16
-// epilogue elements of the previous chunk (held in `prev`).  kHalf: first or second half of the chunk.
-template <int kHalf, bool kInts>
+template <int T>
+struct I8Cfg {
+    static constexpr int kWM = T / 32;                 // 16-key tiles per wave (2 waves along the keys)
+    static constexpr int kWN = 2;                      // 16-query tiles per wave
+    static constexpr int kWavesN = T / 32;             // waves along the queries
+    static constexpr int kConsumers = 2 * kWavesN;
+    static constexpr int kLoaders = T / 32;
+    static constexpr int kBlock = (kConsumers + kLoaders) * 64;
+    static constexpr int kOperand = T * 128;           // bytes of one operand tile of one half-chunk
+    static constexpr int kStage = 2 * kOperand;        // keys then queries
+    static constexpr int kScaleBytes = 4 * kLoaders * 256;  // chunk scales: ring of 4 chunks x loader regions x 64 floats
+    static constexpr int kLds = 4 * kStage + kScaleBytes;
+};
+
+// One half-chunk (two k-steps) of an MFMA wave: 2 WM WN MFMAs into `acc`, 2 (WM + WN) operand
+// reads, and as many epilogue elements of the previous chunk (held in `prev`) as MFMAs.
+// kHalf: first or second half of the chunk.
+template <int WM, int WN, int kHalf, bool kInts>
 __device__ __forceinline__ void i8_consume_half(const unsigned char* __restrict__ krow,
                                                 const unsigned char* __restrict__ qrow, const int (&pcol)[2],
-                                                v4i (&acc)[4][2], const v4i (&prev)[4][2], float (&accf)[4][2][4],
-                                                const float (&qs_prev)[2], int* __restrict__ ints_prev,
-                                                const int64_t (&int_off)[4][2], const int (&int_rows)[4],
-                                                int down_shift, int chunks) {
-    v4i ka[2][4], qb[2][2];
-    // operands of the first k-step, in the order its MFMAs need them
-    ka[0][0] = *reinterpret_cast<const v4i*>(krow + pcol[0]);
-    qb[0][0] = *reinterpret_cast<const v4i*>(qrow + pcol[0]);
-    qb[0][1] = *reinterpret_cast<const v4i*>(qrow + 16 * 128 + pcol[0]);
-    ka[0][1] = *reinterpret_cast<const v4i*>(krow + 16 * 128 + pcol[0]);
-    ka[0][2] = *reinterpret_cast<const v4i*>(krow + 32 * 128 + pcol[0]);
-    ka[0][3] = *reinterpret_cast<const v4i*>(krow + 48 * 128 + pcol[0]);
+                                                v4i (&acc)[WM][WN], const v4i (&prev)[WM][WN],
+                                                float (&accf)[WM][WN][4], const float (&qs_prev)[WN],
+                                                int* __restrict__ ints_prev, const int64_t (&int_off)[WM][WN],
+                                                const int (&int_rows)[WM], int down_shift, int chunks) {
+    static_assert(WM + WN <= WM * WN, "one operand read behind each MFMA of a k-step");
+    v4i ka[2][WM], qb[2][WN];
+    // read number t of a k-step, in the order its MFMAs first need them: ka[0], qb[0..], ka[1..]
+    auto read = [&](int set, int t) {
+        if (t == 0) ka[set][0] = *reinterpret_cast<const v4i*>(krow + pcol[set]);
+        else if (t <= WN) qb[set][t - 1] = *reinterpret_cast<const v4i*>(qrow + (t - 1) * 16 * 128 + pcol[set]);
+        else ka[set][t - WN] = *reinterpret_cast<const v4i*>(krow + (t - WN) * 16 * 128 + pcol[set]);
+    };
+#pragma unroll
+    for (int t = 0; t < WM + WN; ++t) read(0, t);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) {
 #pragma unroll
-        for (int a = 0; a < 4; ++a)
+        for (int a = 0; a < WM; ++a)
 #pragma unroll
-            for (int b = 0; b < 2; ++b) {
-                const int ks = kHalf * 2 + kk, t = a * 2 + b;
+            for (int b = 0; b < WN; ++b) {
+                const int ks = kHalf * 2 + kk, t = a * WN + b;
                 const v4i c0 = (ks == 0) ? (v4i){0, 0, 0, 0} : acc[a][b];
                 acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ka[kk][a], qb[kk][b], c0, 0, 0, 0);
                 {
-                    const int idx = ks * 8 + t, tt = idx >> 2, e = idx & 3, ea = tt >> 1, eb = tt & 1;
+                    const int idx = ks * (WM * WN) + t, tt = idx >> 2, e = idx & 3, ea = tt / WN, eb = tt % WN;
                     accf[ea][eb][e] = fmaf(static_cast<float>(prev[ea][eb][e]), qs_prev[eb], accf[ea][eb][e]);
                     if (kInts && ints_prev != nullptr && int_off[ea][eb] >= 0 && e < int_rows[ea])
                         ints_prev[int_off[ea][eb] + static_cast<int64_t>(e) * chunks] = prev[ea][eb][e] >> down_shift;
                 }
-                if (kk == 0) {  // operands of the second k-step, one read behind each of the first six MFMAs
-                    if (t == 0) ka[1][0] = *reinterpret_cast<const v4i*>(krow + pcol[1]);
-                    if (t == 1) qb[1][0] = *reinterpret_cast<const v4i*>(qrow + pcol[1]);
-                    if (t == 2) qb[1][1] = *reinterpret_cast<const v4i*>(qrow + 16 * 128 + pcol[1]);
-                    if (t == 3) ka[1][1] = *reinterpret_cast<const v4i*>(krow + 16 * 128 + pcol[1]);
-                    if (t == 4) ka[1][2] = *reinterpret_cast<const v4i*>(krow + 32 * 128 + pcol[1]);
-                    if (t == 5) ka[1][3] = *reinterpret_cast<const v4i*>(krow + 48 * 128 + pcol[1]);
-                }
+                if (kk == 0 && t < WM + WN) read(1, t);  // operands of the second k-step
                 __builtin_amdgcn_sched_barrier(0);
             }
     }
 }
 
-template <bool kInts>
-__global__ __launch_bounds__(kI8Block) void dot_mfma_i8_kernel(
+template <int T, bool kInts>
+__global__ __launch_bounds__(I8Cfg<T>::kBlock) void dot_mfma_i8_kernel(
     const int8_t* __restrict__ A8, const float* __restrict__ qscale, int qscale_stride,
     const int8_t* __restrict__ K8,  // int8 key image [R, chunks * 256]
     const float* __restrict__ Bw, int Sb, int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv,
     int64_t R_total, float* __restrict__ out, int* __restrict__ chunk_ints) {
-    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];  // kI8Stages * kI8Stage + kI8ScaleBytes
+    using C = I8Cfg<T>;
+    constexpr int WM = C::kWM, WN = C::kWN;
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];  // C::kLds
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int64_t r0 = static_cast<int64_t>(blockIdx.x) * 128;
-    const int64_t q0 = static_cast<int64_t>(blockIdx.y) * 128;
+    const int64_t r0 = static_cast<int64_t>(blockIdx.x) * T;
+    const int64_t q0 = static_cast<int64_t>(blockIdx.y) * T;
     const size_t rowbytes = static_cast<size_t>(chunks) * 256;
     const int halves = chunks * 2;
-    unsigned char* const scale_lds = lds + kI8Stages * kI8Stage;  // ring of four chunks x 4 loader waves x 64 floats
+    unsigned char* const scale_lds = lds + 4 * C::kStage;  // [chunk & 3][loader][64] floats
 
-    if (wave >= kI8Consumers) {
+    if (wave >= C::kConsumers) {
         // ---- loader wave lw: rows 32 lw .. 32 lw + 31 of both operand tiles of every stage (4 + 4 loads of
         // 1 KiB), plus the chunk scales of 64 queries once per chunk.
-        const int lw = wave - kI8Consumers;
+        const int lw = wave - C::kConsumers;
         const bsi_rsrc rk = make_rsrc(K8 + static_cast<size_t>(r0) * rowbytes, static_cast<size_t>(R - r0) * rowbytes);
         const bsi_rsrc rq = make_rsrc(A8 + static_cast<size_t>(q0) * rowbytes, static_cast<size_t>(Q - q0) * rowbytes);
         const bsi_rsrc rs = make_rsrc(qscale + q0 * qscale_stride, static_cast<size_t>(Q - q0) * qscale_stride * 4);
@@ -782,23 +792,25 @@ __global__ __launch_bounds__(kI8Block) void dot_mfma_i8_kernel(
             koff[i] = static_cast<uint32_t>(kr * rowbytes) + col;
             qoff[i] = static_cast<uint32_t>(qr * rowbytes) + col;
         }
-        // scales: loader wave lw fetches queries 64 (lw & 1) + lane (the two pairs of waves fetch the same
-        // data into their own regions so that every loader wave has the same number of loads in flight)
-        const int sq = (lw & 1) * 64 + lane;
+        // scales: loader wave lw fetches the 64 queries of group lw % (T / 64) (with T = 128 two pairs of
+        // waves fetch the same data into their own regions, so that every loader wave has the same number
+        // of loads in flight)
+        const int sq = (lw % (T / 64)) * 64 + lane;
         const uint32_t soff = static_cast<uint32_t>(((q0 + sq < Q) ? sq : (Q - 1 - q0)) * qscale_stride * 4);
         const int sstep = (qscale_stride == 1) ? 0 : 4;
         auto issue = [&](int h) {  // stage of half-chunk h (clamped to the last) into its ring slot
             const int hc = h < halves ? h : halves - 1;
-            unsigned char* slot = lds + (h & 3) * kI8Stage + (4 * lw) * 1024;
+            unsigned char* slot = lds + (h & 3) * C::kStage + (4 * lw) * 1024;
             const uint32_t so = static_cast<uint32_t>(hc) * 128;
 #pragma unroll
             for (int i = 0; i < 4; ++i) load16_to_lds(rk, koff[i], so, slot + i * 1024);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) load16_to_lds(rq, qoff[i], so, slot + kI8Operand + i * 1024);
+            for (int i = 0; i < 4; ++i) load16_to_lds(rq, qoff[i], so, slot + C::kOperand + i * 1024);
             if (h & 1) {  // with the second half of chunk c = h / 2: its scales
                 const int c = hc >> 1;
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, BSI_LDS_PTR(scale_lds + ((c & 3) * 4 + lw) * 256), 4,
-                                                         static_cast<int>(soff), c * sstep, 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                    rs, BSI_LDS_PTR(scale_lds + ((c & 3) * C::kLoaders + lw) * 256), 4, static_cast<int>(soff),
+                    c * sstep, 0, 0);
             }
         };
         issue(0);
@@ -818,52 +830,54 @@ __global__ __launch_bounds__(kI8Block) void dot_mfma_i8_kernel(
     }
 
     // ---- MFMA waves
-    const int wr = wave & 1, wq = wave >> 1;  // 64-key half, 32-query quarter
+    const int wr = wave & 1, wq = wave >> 1;  // half of the keys, group of 32 queries
     const int ln = lane & 15, lg = lane >> 4;
-    const int krow_off = (wr * 64 + ln) * 128;
-    const int qrow_off = kI8Operand + (wq * 32 + ln) * 128;
+    const int krow_off = (wr * (WM * 16) + ln) * 128;
+    const int qrow_off = C::kOperand + (wq * (WN * 16) + ln) * 128;
     int pcol[2];
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) pcol[kk] = ((kk * 4 + lg) ^ (ln >> 1)) * 16;
-    float accf[4][2][4];
+    float accf[WM][WN][4];
 #pragma unroll
-    for (int a = 0; a < 4; ++a)
+    for (int a = 0; a < WM; ++a)
 #pragma unroll
-        for (int b = 0; b < 2; ++b)
+        for (int b = 0; b < WN; ++b)
 #pragma unroll
             for (int e = 0; e < 4; ++e) accf[a][b][e] = 0.0f;
-    v4i acc0[4][2], acc1[4][2];
+    v4i acc0[WM][WN], acc1[WM][WN];
 #pragma unroll
-    for (int a = 0; a < 4; ++a)
+    for (int a = 0; a < WM; ++a)
 #pragma unroll
-        for (int b = 0; b < 2; ++b) acc0[a][b] = acc1[a][b] = (v4i){0, 0, 0, 0};
+        for (int b = 0; b < WN; ++b) acc0[a][b] = acc1[a][b] = (v4i){0, 0, 0, 0};
     // the MFMA accumulators hold 2^down_shift times the integer dot; the chain runs on them unscaled
     // (a power of two commutes with every rounding) and the factor is taken out once at the end
     const float down = __uint_as_float(static_cast<uint32_t>(127 - down_shift) << 23);
-    int64_t int_off[4][2];
-    int int_rows[4];
+    int64_t int_off[WM][WN];
+    int int_rows[WM];
 #pragma unroll
-    for (int a = 0; a < 4; ++a) {
-        const int64_t r = r0 + wr * 64 + a * 16 + lg * 4;
+    for (int a = 0; a < WM; ++a) {
+        const int64_t r = r0 + wr * (WM * 16) + a * 16 + lg * 4;
         int_rows[a] = static_cast<int>((R - r) < 4 ? (R - r) : 4);
 #pragma unroll
-        for (int b = 0; b < 2; ++b) {
-            const int64_t q = q0 + wq * 32 + b * 16 + ln;
+        for (int b = 0; b < WN; ++b) {
+            const int64_t q = q0 + wq * (WN * 16) + b * 16 + ln;
             int_off[a][b] = (kInts && q < Q && r < R) ? (q * R + r) * chunks : -1;
         }
     }
-    // chunk scales of the lane's two query columns, from the loaders' ring: region (wq >> 1) holds queries
-    // 64 (wq >> 1) .. + 63
+    // chunk scales of the lane's query columns, from the loaders' ring: region wq / 2 holds queries
+    // 64 (wq / 2) .. + 63 (WN = 2: a wave spans 32 queries)
     const unsigned char* sread = scale_lds + (wq >> 1) * 256 + ((wq & 1) * 32 + ln) * 4;
-    float qsa[2] = {0.0f, 0.0f}, qsb[2] = {0.0f, 0.0f};  // even / odd chunks
-#define BSI_I8_SCALES(dst, c)                                                            \
-    {                                                                                    \
-        dst[0] = *reinterpret_cast<const float*>(sread + ((c) & 3) * 1024);              \
-        dst[1] = *reinterpret_cast<const float*>(sread + ((c) & 3) * 1024 + 64);         \
+    float qsa[WN], qsb[WN];  // scales of even / odd chunks
+#pragma unroll
+    for (int b = 0; b < WN; ++b) qsa[b] = qsb[b] = 0.0f;
+#define BSI_I8_SCALES(dst, c)                                                                                  \
+    {                                                                                                          \
+        _Pragma("unroll") for (int b = 0; b < WN; ++b) dst[b] =                                                \
+            *reinterpret_cast<const float*>(sread + ((c) & 3) * (C::kLoaders * 256) + b * 64);                 \
     }
-#define BSI_I8_HALF(kHalf, slot, acc, prev, qs, ip)                                                                   \
-    i8_consume_half<kHalf, kInts>(lds + (slot) * kI8Stage + krow_off, lds + (slot) * kI8Stage + qrow_off, pcol, acc,   \
-                                  prev, accf, qs, ip, int_off, int_rows, down_shift, chunks);                         \
+#define BSI_I8_HALF(kHalf, slot, acc, prev, qs, ip)                                                                  \
+    i8_consume_half<WM, WN, kHalf, kInts>(lds + (slot) * C::kStage + krow_off, lds + (slot) * C::kStage + qrow_off,  \
+                                          pcol, acc, prev, accf, qs, ip, int_off, int_rows, down_shift, chunks);     \
     lds_barrier();
 
     lds_barrier();  // stage 0 is there
@@ -891,9 +905,9 @@ __global__ __launch_bounds__(kI8Block) void dot_mfma_i8_kernel(
 #undef BSI_I8_HALF
     // epilogue of the last chunk
 #pragma unroll
-    for (int a = 0; a < 4; ++a)
+    for (int a = 0; a < WM; ++a)
 #pragma unroll
-        for (int b = 0; b < 2; ++b)
+        for (int b = 0; b < WN; ++b)
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int v = last_in_acc0 ? acc0[a][b][e] : acc1[a][b][e];
@@ -903,18 +917,18 @@ __global__ __launch_bounds__(kI8Block) void dot_mfma_i8_kernel(
                     chunk_ints[int_off[a][b] + static_cast<int64_t>(e) * chunks + (chunks - 1)] = v >> down_shift;
             }
 #pragma unroll
-    for (int a = 0; a < 4; ++a) {
-        const int64_t rb = r0 + wr * 64 + a * 16 + lg * 4;
+    for (int a = 0; a < WM; ++a) {
+        const int64_t rb = r0 + wr * (WM * 16) + a * 16 + lg * 4;
         float bs[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) bs[e] = (rb + e < R) ? Bw[(rb + e) * Sb] : 0.0f;
 #pragma unroll
-        for (int b = 0; b < 2; ++b)
+        for (int b = 0; b < WN; ++b)
 #pragma unroll
             for (int e = 0; e < 4; ++e) accf[a][b][e] *= down;
 #pragma unroll
-        for (int b = 0; b < 2; ++b) {
-            const int64_t q = q0 + wq * 32 + b * 16 + ln;
+        for (int b = 0; b < WN; ++b) {
+            const int64_t q = q0 + wq * (WN * 16) + b * 16 + ln;
             if (q >= Q) continue;
             float* dst = out + static_cast<size_t>(q) * R_total + rb;
             if (rb + 3 < R && ((reinterpret_cast<uintptr_t>(dst) & 15) == 0)) {
@@ -1285,25 +1299,39 @@ static void launch_mfma_ws(const int8_t* A8, const float* qscale, int stride, co
                            R_total, out, chunk_ints);
 }
 
-static void launch_mfma_i8(const int8_t* A8, const float* qscale, int stride, const int8_t* K8, const float* Bw, int Sb,
-                           int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv, int64_t R_total,
-                           float* out, int32_t* chunk_ints, hipStream_t st) {
-    const dim3 grid(static_cast<unsigned>((R + 127) / 128), static_cast<unsigned>((Q + 127) / 128));
-    constexpr int kLds = kI8Stages * kI8Stage + kI8ScaleBytes;
+template <int T>
+static void launch_mfma_i8_t(const int8_t* A8, const float* qscale, int stride, const int8_t* K8, const float* Bw,
+                             int Sb, int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv,
+                             int64_t R_total, float* out, int32_t* chunk_ints, hipStream_t st) {
+    using C = I8Cfg<T>;
+    const dim3 grid(static_cast<unsigned>((R + T - 1) / T), static_cast<unsigned>((Q + T - 1) / T));
     static bool configured = false;
     if (!configured) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dot_mfma_i8_kernel<true>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dot_mfma_i8_kernel<false>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dot_mfma_i8_kernel<T, true>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, C::kLds);
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dot_mfma_i8_kernel<T, false>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, C::kLds);
         configured = true;
     }
     if (chunk_ints)
-        hipLaunchKernelGGL((dot_mfma_i8_kernel<true>), grid, dim3(kI8Block), kLds, st, A8, qscale, stride, K8, Bw, Sb,
-                           chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints);
+        hipLaunchKernelGGL((dot_mfma_i8_kernel<T, true>), grid, dim3(C::kBlock), C::kLds, st, A8, qscale, stride, K8,
+                           Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints);
     else
-        hipLaunchKernelGGL((dot_mfma_i8_kernel<false>), grid, dim3(kI8Block), kLds, st, A8, qscale, stride, K8, Bw, Sb,
-                           chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints);
+        hipLaunchKernelGGL((dot_mfma_i8_kernel<T, false>), grid, dim3(C::kBlock), C::kLds, st, A8, qscale, stride, K8,
+                           Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints);
+}
+
+static void launch_mfma_i8(const int8_t* A8, const float* qscale, int stride, const int8_t* K8, const float* Bw, int Sb,
+                           int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv, int64_t R_total,
+                           float* out, int32_t* chunk_ints, hipStream_t st) {
+    // 128 x 128 tiles unless they would leave most of the 256 CUs without a workgroup
+    const int64_t big = ((R + 127) / 128) * ((Q + 127) / 128);
+    if (big >= g_i8_small_tile_below)
+        launch_mfma_i8_t<128>(A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out,
+                              chunk_ints, st);
+    else
+        launch_mfma_i8_t<64>(A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out,
+                             chunk_ints, st);
 }
 
 template <int NT, int KT>
@@ -1370,6 +1398,17 @@ extern "C" int bsi_hip_planes_to_int8(const uint64_t* words, int64_t rows, int S
     if (rows == 0) return BSI_OK;
     BSI_REQUIRE(words && out, "null pointer");
     return launch_planes_to_int8(words, rows, S, W64, out, as_stream(stream));
+}
+
+extern "C" int bsi_hip_set_option(int option, int value) {
+    switch (option) {
+        case BSI_OPT_I8_SMALL_TILE_BELOW:
+            BSI_REQUIRE(value >= 0, "threshold must be >= 0");
+            g_i8_small_tile_below = value;
+            return BSI_OK;
+        default:
+            return fail(BSI_ERR_INVALID, "unknown option %d", option);
+    }
 }
 
 extern "C" size_t bsi_hip_dot_workspace_bytes(int64_t Q, int W64, int core) {

@@ -287,7 +287,9 @@ def _run_dot(hip, qb, kb, Q, R, W, Sa, Sb, core, tiled, with_ints8, want_ints=Tr
     stride = chunks if qb["chunk_scale"] else 1
     B = dev(kb["words"])
     layout = 0
-    if tiled == "int8":   # the cached int8 image of the key integers
+    if tiled in ("int8", "int8-128", "int8-64"):   # the cached int8 image of the key integers; tile size forced or automatic
+        hip.check(L.bsi_hip_set_option(hip.OPT_I8_SMALL_TILE_BELOW, {"int8": 100, "int8-128": 0, "int8-64": 1 << 30}[tiled]),
+                  "set_option")
         Bi = torch.full((R, chunks * 256), 77, dtype=torch.int8, device="cuda")
         hip.check(L.bsi_hip_planes_to_int8(B.data_ptr(), R, Sb, W, Bi.data_ptr(), st()), "key image")
         B, layout = Bi, 2
@@ -310,6 +312,7 @@ def _run_dot(hip, qb, kb, Q, R, W, Sa, Sb, core, tiled, with_ints8, want_ints=Tr
                             out.data_ptr(), ints.data_ptr() if ints is not None else None, core, ws.data_ptr(),
                             ws_bytes, st()), "dot")
     torch.cuda.synchronize()
+    hip.check(L.bsi_hip_set_option(hip.OPT_I8_SMALL_TILE_BELOW, 100), "set_option")
     return (ints.cpu().numpy() if ints is not None else None), out.cpu().numpy()
 
 
@@ -330,7 +333,7 @@ DOT_SHAPES = [
 
 @pytest.mark.parametrize("Q,R,d,kind", DOT_SHAPES)
 @pytest.mark.parametrize("core,tiled,ints8", [(1, False, False), (1, True, False), (2, False, True), (2, True, False),
-                                              (0, True, True), (2, "int8", True), (0, "int8", False)])
+                                              (0, True, True), (2, "int8-128", True), (0, "int8-64", False)])
 def test_dot_bit_exact(hip, oracle, Q, R, d, kind, core, tiled, ints8):
     x, k, qb, kb, want_ints, want_out = _oracle_case(oracle, Q, R, d, seed=Q + R + d, qkind=kind)
     W = (d + 63) // 64
@@ -348,7 +351,7 @@ def test_dot_bit_exact(hip, oracle, Q, R, d, kind, core, tiled, ints8):
 
 
 @pytest.mark.parametrize("Sa,Sb", [(8, 8), (5, 4), (2, 2), (7, 5), (3, 7)])
-@pytest.mark.parametrize("core,tiled", [(1, False), (2, True), (2, "int8")])
+@pytest.mark.parametrize("core,tiled", [(1, False), (2, True), (2, "int8-128"), (2, "int8-64")])
 def test_dot_other_bit_widths(hip, oracle, Sa, Sb, core, tiled):
     Q, R, d = 19, 35, 1024
     x, k, qb, kb, want_ints, want_out = _oracle_case(oracle, Q, R, d, seed=Sa * 10 + Sb, ksigma=0.05, bits_q=Sa, bits_k=Sb)
