@@ -79,6 +79,7 @@ def _flags() -> dict:
         core={"auto": _lib.CORE_AUTO, "valu": _lib.CORE_VALU, "mfma": _lib.CORE_MFMA}.get(core, _lib.CORE_AUTO),
         tiled=(layout != "canonical"),
         key_image=(_env_int("BSI_KEY_INT8_IMAGE", 1) or 0) != 0,
+        ewah_inline=(_env_int("BSI_EWAH_INLINE", 1) or 0) != 0,
     )
     return _flag_cache
 
@@ -587,6 +588,33 @@ def batch_dot_product_multiquery_cuda_caps(query_caps_list, keyset_cuda_cap):
     for q in rows:
         _check((q.chunk_scales is not None and q.chunk_scales.numel() > 0) == have_scales,
                "Mixed chunk-scale and non-chunk-scale queries in the same group")
+    f = _flags()
+    q0 = rows[0]
+    if (Q == 1 and getattr(q0, "comp_words", None) is not None and q0.comp_words.numel() > 0 and f["ewah_inline"]
+            and keys.layout == _lib.LAYOUT_TILED16 and keys.Sb == 6 and 2 <= q0.S <= 8
+            and f["core"] != _lib.CORE_VALU and q0.S * ((keys.W + 3) // 4) * 32 <= 96 * 1024):
+        # a hybrid query: its EWAH streams are decoded inside the dot's load stage
+        _check(q0.decimals == keys.decimals, f"Decimal mismatch between queries and keys: q={q0.decimals} k={keys.decimals}")
+        if have_scales:
+            sc, stride = q0.chunk_scales.contiguous(), int(q0.chunk_scales.numel())
+            _check(keys.W % 4 == 0 and stride == keys.W // 4, "Chunk scale stride mismatch")
+        else:
+            sc, stride = q0.row_scale.reshape(1).contiguous(), 1
+        out = torch.empty((1, R), dtype=torch.float32, device=q0.comp_words.device)
+        prof = f["profile"]
+        if prof:
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+        check(lib.bsi_hip_dot_ewah_query(q0.comp_words.data_ptr(), q0.comp_off.data_ptr(), q0.comp_len.data_ptr(),
+                                         q0.S, keys.W, sc.data_ptr(), stride, keys.words.data_ptr(),
+                                         keys.slice_weights.data_ptr(), keys.Sb, R, _scale_inv(q0.decimals, keys.decimals),
+                                         out.data_ptr(), None, _stream()), "bsi_hip_dot_ewah_query")
+        ns = 0
+        if prof:
+            e1.record()
+            e1.synchronize()
+            ns = int(e0.elapsed_time(e1) * 1.0e6)
+        return _dot_result(out, ns, 1, R)
     words = torch.stack([q.dev_words for q in rows]).contiguous()
     if have_scales:
         scales = torch.stack([q.chunk_scales for q in rows]).contiguous()

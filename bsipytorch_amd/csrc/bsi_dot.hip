@@ -1073,6 +1073,122 @@ __global__ __launch_bounds__(1024) void dot_mfma_stream_kernel(
     if (cvalid) out[static_cast<size_t>(cq) * R_total + cr] = (accf * Bw[cr * 6]) * scale_inv;
 }
 
+// ------------------------------------------------------------------ one EWAH-compressed query, decode inline
+//
+// The hybrid query form keeps each of its Sa slices as an EWAH stream ([marker][literals...],
+// marker = run_bit | run_len << 1 | literal_count << 33; bsi_cuda_kernels_ewah.cuh:5-33 is the
+// decoder this follows, including its bounds: output clipped at W words, input at the stream's
+// length, the rest zero).  This kernel is the few-rows kernel for that one query with the decode
+// folded into its load stage: every workgroup first expands the streams into bit planes in LDS
+// (wave s walks the markers of slice s; its lanes write a run or copy a literal block in
+// parallel), then recombines the planes of each chunk into the int8 MFMA operand in registers,
+// exactly as it does for the key planes it streams from HBM.
+template <bool kInts>
+__global__ __launch_bounds__(1024) void dot_mfma_stream_ewah_kernel(
+    const unsigned long long* __restrict__ comp, const long long* __restrict__ comp_off,
+    const int* __restrict__ comp_len, int Sa, int W64, const float* __restrict__ qscale, int qscale_stride,
+    const unsigned long long* __restrict__ B64,  // tiled key planes, Sb = 6
+    const float* __restrict__ Bw, int chunks, int pass_chunks, int64_t R, int down_shift, float scale_inv,
+    float* __restrict__ out, int* __restrict__ chunk_ints) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    // [Sa][4 * chunks] query plane words (zero-padded to whole chunks), then the chunk accumulators
+    unsigned long long* planes = reinterpret_cast<unsigned long long*>(smem);
+    const int wpad = chunks * 4;
+    int* ints = reinterpret_cast<int*>(smem + static_cast<size_t>(Sa) * wpad * 8);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nwaves = static_cast<int>(blockDim.x >> 6);
+    const int ln = lane & 15, lg = lane >> 4;
+    const int64_t tile = blockIdx.x;
+    const unsigned long long* ksrc = B64 + static_cast<size_t>(tile) * chunks * (6 * 64) + lane;
+
+    // ---- inline EWAH decode: slices round-robin over the waves
+    for (int s = wave; s < Sa; s += nwaves) {
+        const unsigned long long* in = comp + comp_off[s];
+        const int in_len = comp_len[s];
+        unsigned long long* dst = planes + static_cast<size_t>(s) * wpad;
+        int idx = 0, o = 0;
+        while (idx < in_len && o < W64) {
+            const unsigned long long rlw = in[idx++];
+            const unsigned long long run_val = (rlw & 1ULL) ? ~0ULL : 0ULL;
+            const unsigned int run_len = static_cast<unsigned int>((rlw >> 1) & 0xFFFFFFFFULL);
+            const unsigned int lit = static_cast<unsigned int>(rlw >> 33);
+            const int n_run = static_cast<int>(run_len < static_cast<unsigned int>(W64 - o) ? run_len : W64 - o);
+            for (int k = lane; k < n_run; k += BSI_WAVE) dst[o + k] = run_val;
+            o += n_run;
+            int n_lit = static_cast<int>(lit < static_cast<unsigned int>(W64 - o) ? lit : W64 - o);
+            if (n_lit > in_len - idx) n_lit = in_len - idx;
+            for (int k = lane; k < n_lit; k += BSI_WAVE) dst[o + k] = in[idx + k];
+            o += n_lit;
+            idx += n_lit;
+            if (static_cast<unsigned int>(n_lit) < lit) break;  // clipped: the reference loop stops here too
+        }
+        for (int k = o + lane; k < wpad; k += BSI_WAVE) dst[k] = 0ULL;
+    }
+    __syncthreads();
+
+    const bool chain = tid < 256;
+    const int ckey = tid & 15, cn = (tid >> 4) & 15;
+    const int64_t cr = tile * 16 + ckey;
+    const bool cvalid = chain && cn == 0 && cr < R;
+    const float down = __uint_as_float(static_cast<uint32_t>(127 - down_shift) << 23);
+    const int sstep = (qscale_stride == 1) ? 0 : 1;
+    float accf = 0.0f;
+
+    for (int p0 = 0; p0 < chunks; p0 += pass_chunks) {
+        const int pend = (p0 + pass_chunks < chunks) ? p0 + pass_chunks : chunks;
+        for (int c = p0 + wave; c < pend; c += nwaves) {
+            uint2 kc[6];
+#pragma unroll
+            for (int j = 0; j < 6; ++j) {
+                const unsigned long long w = ksrc[(static_cast<size_t>(c) * 6 + j) * 64];
+                kc[j] = make_uint2(static_cast<uint32_t>(w), static_cast<uint32_t>(w >> 32));
+            }
+            // the query operand of this chunk from the decoded planes (column 0 of the MFMA; the other 15 stay zero)
+            uint32_t qlo[8], qhi[8];
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const int j = t - (8 - Sa);
+                const unsigned long long w =
+                    (ln == 0 && j >= 0) ? planes[static_cast<size_t>(j) * wpad + c * 4 + lg] : 0ULL;
+                qlo[t] = static_cast<uint32_t>(w);
+                qhi[t] = static_cast<uint32_t>(w >> 32);
+            }
+            transpose8x8(qlo);
+            transpose8x8(qhi);
+            v4i qb[4];
+            qb[0] = (v4i){static_cast<int>(qlo[0]), static_cast<int>(qlo[1]), static_cast<int>(qlo[2]), static_cast<int>(qlo[3])};
+            qb[1] = (v4i){static_cast<int>(qlo[4]), static_cast<int>(qlo[5]), static_cast<int>(qlo[6]), static_cast<int>(qlo[7])};
+            qb[2] = (v4i){static_cast<int>(qhi[0]), static_cast<int>(qhi[1]), static_cast<int>(qhi[2]), static_cast<int>(qhi[3])};
+            qb[3] = (v4i){static_cast<int>(qhi[4]), static_cast<int>(qhi[5]), static_cast<int>(qhi[6]), static_cast<int>(qhi[7])};
+            uint32_t lo[8], hi[8];
+            transpose_6planes(kc[0].x, kc[1].x, kc[2].x, kc[3].x, kc[4].x, kc[5].x, lo);
+            transpose_6planes(kc[0].y, kc[1].y, kc[2].y, kc[3].y, kc[4].y, kc[5].y, hi);
+            v4i ka[4];
+            ka[0] = (v4i){static_cast<int>(lo[0]), static_cast<int>(lo[1]), static_cast<int>(lo[2]), static_cast<int>(lo[3])};
+            ka[1] = (v4i){static_cast<int>(lo[4]), static_cast<int>(lo[5]), static_cast<int>(lo[6]), static_cast<int>(lo[7])};
+            ka[2] = (v4i){static_cast<int>(hi[0]), static_cast<int>(hi[1]), static_cast<int>(hi[2]), static_cast<int>(hi[3])};
+            ka[3] = (v4i){static_cast<int>(hi[4]), static_cast<int>(hi[5]), static_cast<int>(hi[6]), static_cast<int>(hi[7])};
+            v4i acc = {0, 0, 0, 0};
+#pragma unroll
+            for (int m = 0; m < 4; ++m) acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(ka[m], qb[m], acc, 0, 0, 0);
+            *reinterpret_cast<v4i*>(&ints[(c - p0) * 256 + ln * 16 + lg * 4]) = acc;
+        }
+        __syncthreads();
+        if (cvalid) {
+            for (int cc = p0; cc < pend; ++cc) {
+                const int v = ints[(cc - p0) * 256 + ckey];  // query 0, key ckey
+                accf = fmaf(static_cast<float>(v), qscale[cc * sstep] * down, accf);
+                if (kInts) chunk_ints[cr * chunks + cc] = v >> down_shift;
+            }
+        }
+        if (pend < chunks) __syncthreads();
+    }
+    if (cvalid) out[cr] = (accf * Bw[cr * 6]) * scale_inv;
+}
+
 // ------------------------------------------------------------------ VALU popcount core (Sa = 7, Sb = 6 shape templated)
 
 constexpr int kValuBlock = 256;
@@ -1504,6 +1620,55 @@ extern "C" int bsi_hip_dot(const uint64_t* A, const int8_t* A_ints8, const float
                        reinterpret_cast<const unsigned long long*>(B), Bw, Sb, W64, chunks, R, Q, scale_inv, R_total,
                        out, chunk_ints);
     BSI_LAUNCH_CHECK("dot_valu_generic_kernel");
+    return BSI_OK;
+}
+
+extern "C" int bsi_hip_dot_ewah_query(const uint64_t* comp_words, const int64_t* comp_off, const int32_t* comp_len,
+                                      int Sa, int W64, const float* A_chunk_scales, int A_scale_stride,
+                                      const uint64_t* B_tiled, const float* Bw, int Sb, int64_t R, float scale_inv,
+                                      float* out, int32_t* chunk_ints, void* stream) {
+    BSI_REQUIRE(R >= 0 && W64 >= 1, "bad shape");
+    BSI_REQUIRE(Sa >= 2 && Sa <= 8, "Sa must be in [2, 8] (got %d)", Sa);
+    if (Sb != 6) return fail(BSI_ERR_UNSUPPORTED, "the inline-decode kernel reads 6-plane tiled keys (got Sb = %d)", Sb);
+    if (R == 0) return BSI_OK;
+    BSI_REQUIRE(comp_words && comp_off && comp_len && A_chunk_scales && B_tiled && Bw && out, "null pointer");
+    const int chunks = (W64 + 3) / 4;
+    BSI_REQUIRE(A_scale_stride == chunks || A_scale_stride == 1,
+                "chunk scale stride mismatch: got %d expected %d (or 1 for a row scale)", A_scale_stride, chunks);
+    const size_t plane_bytes = static_cast<size_t>(Sa) * chunks * 4 * 8;
+    if (plane_bytes > 96 * 1024)
+        return fail(BSI_ERR_UNSUPPORTED, "query of %d words per slice does not fit the LDS plane buffer", W64);
+    int pass_chunks = static_cast<int>((kStreamLdsInts * sizeof(int) < 150 * 1024 - plane_bytes
+                                            ? kStreamLdsInts * sizeof(int)
+                                            : 150 * 1024 - plane_bytes) / 1024);
+    if (pass_chunks > chunks) pass_chunks = chunks;
+    const size_t lds = plane_bytes + static_cast<size_t>(pass_chunks) * 1024;
+    int waves = chunks < 16 ? chunks : 16;
+    if (waves < 4) waves = 4;
+    hipStream_t st = as_stream(stream);
+    const dim3 grid(static_cast<unsigned>((R + 15) / 16));
+    static bool configured = false;
+    if (!configured) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dot_mfma_stream_ewah_kernel<true>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dot_mfma_stream_ewah_kernel<false>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        configured = true;
+    }
+    const int down_shift = 16 - Sa - Sb;
+    if (chunk_ints)
+        hipLaunchKernelGGL((dot_mfma_stream_ewah_kernel<true>), grid, dim3(waves * 64), lds, st,
+                           reinterpret_cast<const unsigned long long*>(comp_words),
+                           reinterpret_cast<const long long*>(comp_off), comp_len, Sa, W64, A_chunk_scales,
+                           A_scale_stride, reinterpret_cast<const unsigned long long*>(B_tiled), Bw, chunks,
+                           pass_chunks, R, down_shift, scale_inv, out, chunk_ints);
+    else
+        hipLaunchKernelGGL((dot_mfma_stream_ewah_kernel<false>), grid, dim3(waves * 64), lds, st,
+                           reinterpret_cast<const unsigned long long*>(comp_words),
+                           reinterpret_cast<const long long*>(comp_off), comp_len, Sa, W64, A_chunk_scales,
+                           A_scale_stride, reinterpret_cast<const unsigned long long*>(B_tiled), Bw, chunks,
+                           pass_chunks, R, down_shift, scale_inv, out, chunk_ints);
+    BSI_LAUNCH_CHECK("dot_mfma_stream_ewah_kernel");
     return BSI_OK;
 }
 

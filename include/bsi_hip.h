@@ -179,6 +179,18 @@ int bsi_hip_dot(const uint64_t* A, const int8_t* A_ints8, const float* A_chunk_s
                 float scale_inv, int64_t R_total, float* out, int32_t* chunk_ints, int core, void* workspace,
                 size_t workspace_bytes, void* stream);
 
+/* The same dot for ONE query whose slices are EWAH streams (the hybrid query form of
+ * build_bsi_query_cuda_hybrid, bsi_cuda.cpp:386-431): stream s at comp_words + comp_off[s], comp_len[s]
+ * words, decoded to W64 words per slice inside the kernel's load stage with the semantics of
+ * ewah_decompress_kernel (bsi_cuda_kernels_ewah.cuh:5-33).  The reference decodes on the host side of the
+ * dot (one <<<1,1>>> launch per slice, bsi_cuda.cpp:402-414) and feeds verbatim words to the kernel; this
+ * entry point removes that pass.  Keys: tiled16 planes with Sb = 6.  out: float [R]; chunk_ints: optional
+ * int32 [R, chunks]. */
+int bsi_hip_dot_ewah_query(const uint64_t* comp_words, const int64_t* comp_off, const int32_t* comp_len, int Sa,
+                           int W64, const float* A_chunk_scales, int A_scale_stride, const uint64_t* B_tiled,
+                           const float* Bw, int Sb, int64_t R, float scale_inv, float* out, int32_t* chunk_ints,
+                           void* stream);
+
 /* Runs fn-independent timing of `iters` back-to-back bsi_hip_dot launches between two HIP events
  * recorded on `stream`, synchronises, and returns the mean launch duration in microseconds.
  * Mirrors the reference's BSI_PROFILE event pair (bsi_cuda.cpp:713-722,798-806). */

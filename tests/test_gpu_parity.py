@@ -350,6 +350,58 @@ def test_dot_bit_exact(hip, oracle, Q, R, d, kind, core, tiled, ints8):
         np.testing.assert_array_equal(out2, want_out)
 
 
+@pytest.mark.parametrize("R,d,kind,force", [(75, 2048, "relu", False), (200, 4096, "randn", True), (40, 700, "relu", True),
+                                            (20, 16640, "relu", False), (33, 256, "ties", True)])
+def test_dot_ewah_query_inline(hip, oracle, R, d, kind, force):
+    """One query handed over as EWAH streams, decoded inside the dot: identical to the dot on verbatim planes."""
+    x, k, qb, kb, want_ints, want_out = _oracle_case(oracle, 1, R, d, seed=R + d, qkind=kind)
+    L = hip.lib
+    W = (d + 63) // 64
+    chunks = (W + 3) // 4
+    planes = qb["words"][0]
+    flags = np.ones(7, dtype=np.int32) if force else oracle.compress_flags(planes, 0.5)
+    stream, off, lens = oracle.ewah_encode(planes, flags)
+    if kind == "relu" and not force:
+        assert lens[6] == 1  # the all-zero sign plane is one run marker
+    comp, offd, lend = dev(stream), dev(off.astype(np.int64)), dev(lens.astype(np.int32))
+    scales = dev(qb["scales"])
+    stride = chunks if qb["chunk_scale"] else 1
+    B = dev(kb["words"])
+    Bt = torch.full((((R + 15) // 16) * chunks * 6 * 64,), -1, dtype=torch.int64, device="cuda")
+    hip.check(L.bsi_hip_tile_key_planes(B.data_ptr(), R, 6, W, Bt.data_ptr(), st()), "tile")
+    Bw = dev(kb["slice_weights"])
+    for with_ints in (True, False):
+        out = torch.full((R,), float("nan"), dtype=torch.float32, device="cuda")
+        ints = torch.full((R, chunks), -7, dtype=torch.int32, device="cuda") if with_ints else None
+        hip.check(L.bsi_hip_dot_ewah_query(comp.data_ptr(), offd.data_ptr(), lend.data_ptr(), 7, W, scales.data_ptr(),
+                                           stride, Bt.data_ptr(), Bw.data_ptr(), 6, R, float(np.float32(1e-4)),
+                                           out.data_ptr(), ints.data_ptr() if with_ints else None, st()), "ewah dot")
+        torch.cuda.synchronize()
+        if with_ints:
+            np.testing.assert_array_equal(ints.cpu().numpy(), want_ints[0])
+        np.testing.assert_array_equal(out.cpu().numpy(), want_out[0])
+    rc = L.bsi_hip_dot_ewah_query(comp.data_ptr(), offd.data_ptr(), lend.data_ptr(), 7, W, scales.data_ptr(), stride,
+                                  Bt.data_ptr(), Bw.data_ptr(), 5, R, 1.0, out.data_ptr(), None, st())
+    assert rc == 3  # only 6-plane keys
+
+
+def test_hybrid_query_dot_decodes_inline(ops, oracle, monkeypatch):
+    x = np.maximum(_inputs(1, 4096, 11), 0)[0]
+    rng = np.random.default_rng(5)
+    k = (rng.standard_normal((300, 4096)) * 0.02).astype(np.float32)
+    kcap, *_ = ops.build_bsi_keys_cuda(torch.from_numpy(k), 2, 0.5)
+    cap, *_ = ops.build_bsi_query_cuda_hybrid(torch.from_numpy(x).cuda(), 2, 0.5)
+    out, *_ = ops.batch_dot_product_multiquery_cuda_caps([cap], kcap)       # streams decoded in the kernel
+    monkeypatch.setenv("BSI_EWAH_INLINE", "0")
+    ops._reset_flag_cache()
+    ref, *_ = ops.batch_dot_product_multiquery_cuda_caps([cap], kcap)       # verbatim planes
+    assert out.shape == (1, 300) and torch.equal(out, ref)
+    qi, _, qscale = oracle.quantize_fixed(x[None], 2, 7, False)   # a single query vector carries one row scale
+    kb = oracle.build_keys(k)
+    _, want = oracle.dot_fixed(oracle.pack(qi, 7), qscale, kb["words"], kb["scales"], oracle.scale_inv(2, 2))
+    np.testing.assert_array_equal(out.cpu().numpy(), want)
+
+
 @pytest.mark.parametrize("Sa,Sb", [(8, 8), (5, 4), (2, 2), (7, 5), (3, 7)])
 @pytest.mark.parametrize("core,tiled", [(1, False), (2, True), (2, "int8-128"), (2, "int8-64")])
 def test_dot_other_bit_widths(hip, oracle, Sa, Sb, core, tiled):
