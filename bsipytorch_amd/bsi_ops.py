@@ -96,13 +96,25 @@ def _check(cond: bool, msg: str) -> None:
         raise RuntimeError(msg)
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_device_objects: dict = {}
+
+
 def _stream() -> int:
+    """Handle of torch's current stream on the current device (what every launch is enqueued on)."""
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
 def _device() -> torch.device:
-    _check(torch.cuda.is_available(), "bsi_ops: no GPU visible; the HIP path is the only path")
-    return torch.device("cuda", torch.cuda.current_device())
+    idx = torch.cuda.current_device() if _device_objects else -1
+    dev = _device_objects.get(idx)
+    if dev is None:
+        _check(torch.cuda.is_available(), "bsi_ops: no GPU visible; the HIP path is the only path")
+        idx = torch.cuda.current_device()
+        dev = _device_objects[idx] = torch.device("cuda", idx)
+    return dev
 
 
 def _dtype_code(t: torch.Tensor) -> int:
@@ -506,6 +518,10 @@ def _dot(words, ints8, scales, scale_stride, Sa, W, keys: PrebuiltBSIKeysCUDA, Q
     R = keys.num_keys
     out = torch.empty((Q, R), dtype=torch.float32, device=dev)
     core = f["core"] if core is None else core
+    # the reference's A/B switch between its tensor-core and popcount kernels is read on every call
+    # (bsi_cuda_kernels_dot.cuh:2642); 0 selects the popcount core here
+    if os.environ.get("BSI_TC_DOT", "1").strip() == "0" and words is not None:
+        core = _lib.CORE_VALU
     ws = None
     ws_bytes = 0
     if ints8 is None:
