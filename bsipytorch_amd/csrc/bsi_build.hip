@@ -195,17 +195,15 @@ __global__ void shift_pack_kernel(Src src, int64_t Q, int64_t d, int chunks, int
 
 // ---------------------------------------------------------------- fused builds
 
-// Chunk-scale build in one pass: one wave per (row, chunk) rounds, reduces, shifts, clamps, packs.
+// Chunk-scale build of one (row, chunk) item by one wave: round, reduce, shift, clamp, pack (64-bit
+// arithmetic throughout: any magnitude, any slice count, optional clipping).
 template <typename T>
-__global__ void build_fixed_chunk_kernel(const T* __restrict__ x, int64_t Q, int64_t d, int chunks, int slices,
-                                         int words_per_slice, double dec_scale, float clip_k,
-                                         unsigned long long* __restrict__ words, int* __restrict__ shifts,
-                                         float* __restrict__ scales, int8_t* __restrict__ ints8) {
-    const int lane = threadIdx.x & (BSI_WAVE - 1);
-    const int64_t wave = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
-    if (wave >= Q * chunks) return;
-    const int64_t row = wave / chunks;
-    const int c = static_cast<int>(wave - row * chunks);
+__device__ __forceinline__ void build_chunk_item(const T* __restrict__ x, int64_t item, int64_t d, int chunks, int slices,
+                                                 int words_per_slice, double dec_scale, float clip_k,
+                                                 unsigned long long* __restrict__ words, int* __restrict__ shifts,
+                                                 float* __restrict__ scales, int8_t* __restrict__ ints8, int lane) {
+    const int64_t row = item / chunks;
+    const int c = static_cast<int>(item - row * chunks);
     const int64_t start = static_cast<int64_t>(c) * BSI_CHUNK_ELEMS;
     int64_t valid = d - start;
     if (valid > BSI_CHUNK_ELEMS) valid = BSI_CHUNK_ELEMS;
@@ -229,8 +227,8 @@ __global__ void build_fixed_chunk_kernel(const T* __restrict__ x, int64_t Q, int
     if (clip_k > 0.0f) sum = wave_sum_f64(sum);
     const int shift = (valid > 0) ? compute_shift(mx, sum, static_cast<int>(valid), slices, clip_k) : 0;
     if (lane == 0) {
-        shifts[wave] = shift;
-        scales[wave] = static_cast<float>(1ULL << shift);
+        shifts[item] = shift;
+        scales[item] = static_cast<float>(1ULL << shift);
     }
     const long long qmax = (1LL << (slices - 1)) - 1LL;
     const long long qmin = -(1LL << (slices - 1));
@@ -242,12 +240,179 @@ __global__ void build_fixed_chunk_kernel(const T* __restrict__ x, int64_t Q, int
         const long long q = (e < valid) ? shift_clamp(r[k], shift, qmin, qmax) : 0;
         v[k] = static_cast<unsigned long long>(q) & mask;
         if (ints8 != nullptr)
-            ints8[(static_cast<size_t>(row) * chunks + c) * BSI_CHUNK_ELEMS + mfma_byte_pos(e)] =
+            ints8[static_cast<size_t>(item) * BSI_CHUNK_ELEMS + mfma_byte_pos(e)] =
                 static_cast<int8_t>(static_cast<int>(q) << (8 - slices));
     }
     ballot_pack_store(v, slices, lane, c, words_per_slice,
                       words + static_cast<size_t>(row) * slices * words_per_slice);
 }
+
+template <typename T>
+__global__ void build_fixed_chunk_kernel(const T* __restrict__ x, int64_t Q, int64_t d, int chunks, int slices,
+                                         int words_per_slice, double dec_scale, float clip_k,
+                                         unsigned long long* __restrict__ words, int* __restrict__ shifts,
+                                         float* __restrict__ scales, int8_t* __restrict__ ints8) {
+    const int lane = threadIdx.x & (BSI_WAVE - 1);
+    const int64_t wave = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6);
+    if (wave >= Q * chunks) return;
+    build_chunk_item<T>(x, wave, d, chunks, slices, words_per_slice, dec_scale, clip_k, words, shifts, scales, ints8, lane);
+}
+
+// The same build for the common case (at most 8 slices, no clipping, whole chunks of words), about
+// seven times fewer instructions per element.  One wave takes 8 consecutive (row, chunk) items:
+//   * rounding stays in fp64 (the product (double)(float)v * 10^dec must be exact), but everything
+//     after it is 32-bit integer work; an item holding a magnitude of 2^31 or more (or a NaN) is
+//     handed to the 64-bit routine above, so results never differ;
+//   * the quantised values go to LDS as the int8 image (value << (8 - slices), the MFMA core's
+//     in-chunk order); the image is the bit-transpose of the planes, 32 elements at a time, so
+//     lane (item j, unit w) reads its 8 dwords, transposes the 8x8 bit blocks in registers and
+//     has one 32-bit half-word of every slice: no ballots, and all 64 lanes busy.
+// kFastItems = items per wave (1, 2, 4 or 8): fewer for small inputs, where the length of one wave's
+// instruction stream, not the throughput, sets the kernel's duration.
+template <typename T, int kFastItems>
+__global__ __launch_bounds__(kBlock) void build_fixed_chunk_fast_kernel(
+    const T* __restrict__ x, int64_t Q, int64_t d, int chunks, int slices, int words_per_slice, double dec_scale,
+    unsigned long long* __restrict__ words, int* __restrict__ shifts, float* __restrict__ scales,
+    int8_t* __restrict__ ints8) {
+    __shared__ uint32_t image[kWavesPerBlock][kFastItems][BSI_CHUNK_ELEMS / 4];
+    const int lane = threadIdx.x & (BSI_WAVE - 1);
+    const int wib = threadIdx.x >> 6;
+    const int64_t total = Q * chunks;
+    const int64_t item0 = (static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + wib) * kFastItems;
+    // (row, chunk) of item0 + j without a 64-bit division per item
+    const int64_t row0 = item0 / chunks;
+    const unsigned c0 = static_cast<unsigned>(item0 - row0 * chunks);
+#define BSI_ITEM_ROW_CHUNK(j, row, c)                                  \
+    const unsigned cj_##row = c0 + static_cast<unsigned>(j);          \
+    const unsigned dr_##row = cj_##row / static_cast<unsigned>(chunks); \
+    const int64_t row = row0 + dr_##row;                               \
+    const int c = static_cast<int>(cj_##row - dr_##row * static_cast<unsigned>(chunks));
+    const int qmax = (1 << (slices - 1)) - 1, qmin = -(1 << (slices - 1));
+    unsigned slow = 0u;  // items that took the 64-bit routine (their outputs are already written)
+    // all loads of the wave's 8 items first: one memory latency, not eight
+    float raw[kFastItems][4];
+#pragma unroll
+    for (int j = 0; j < kFastItems; ++j) {
+        const int64_t item = item0 + j;
+        BSI_ITEM_ROW_CHUNK(j, row, c)
+        const int64_t start = static_cast<int64_t>(c) * BSI_CHUNK_ELEMS;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int64_t e = start + k * BSI_WAVE + lane;
+            raw[j][k] = (item < total && e < d) ? load_as_float<T>(x, row * d + e) : 0.0f;
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < kFastItems; ++j) {
+        const int64_t item = item0 + j;
+        if (item < total) {
+            BSI_ITEM_ROW_CHUNK(j, row, c)
+            (void)row;
+            const int64_t start = static_cast<int64_t>(c) * BSI_CHUNK_ELEMS;
+            const int valid = static_cast<int>((d - start) < BSI_CHUNK_ELEMS ? (d - start) : BSI_CHUNK_ELEMS);
+            double xs[4];
+            bool big = false;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                xs[k] = __dmul_rn(static_cast<double>(raw[j][k]), dec_scale);  // elements past the end were loaded as 0
+                big = big || !(fabs(xs[k]) < 2147483000.0);
+            }
+            if (__any(big)) {
+                slow |= 1u << j;  // done below by the 64-bit routine
+            } else {
+                int r[4];
+                unsigned mx = 0u;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const int mag = static_cast<int>(floor(__dadd_rn(fabs(xs[k]), 0.5)));  // round half away from zero
+                    r[k] = (xs[k] < 0.0) ? -mag : mag;
+                    mx = (static_cast<unsigned>(mag) > mx) ? static_cast<unsigned>(mag) : mx;
+                }
+#pragma unroll
+                for (int off = 32; off > 0; off >>= 1) {
+                    const unsigned o = __shfl_xor(mx, off, BSI_WAVE);
+                    mx = o > mx ? o : mx;
+                }
+                const int shift = compute_shift(static_cast<unsigned long long>(mx), 0.0, valid, slices, 0.0f);
+                if (lane == 0) {
+                    shifts[item] = shift;
+                    scales[item] = static_cast<float>(1ULL << shift);
+                }
+                const unsigned round_add = (shift > 0) ? (1u << (shift - 1)) : 0u;
+                unsigned char* img = reinterpret_cast<unsigned char*>(image[wib][j]);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const unsigned av = static_cast<unsigned>(r[k] < 0 ? -r[k] : r[k]);
+                    const int qa = static_cast<int>((av + round_add) >> shift);
+                    int q = (r[k] < 0) ? -qa : qa;
+                    q = q < qmin ? qmin : (q > qmax ? qmax : q);
+                    img[mfma_byte_pos(k * BSI_WAVE + lane)] = static_cast<unsigned char>(q << (8 - slices));
+                }
+            }
+        }
+    }
+    if (slow != 0u) {
+#pragma unroll 1
+        for (int j = 0; j < kFastItems; ++j)
+            if (slow & (1u << j))
+                build_chunk_item<T>(x, item0 + j, d, chunks, slices, words_per_slice, dec_scale, 0.0f, words, shifts,
+                                    scales, ints8, lane);
+    }
+    __syncthreads();
+    // the int8 image: 256 bytes per item, one dword per lane
+    if (ints8 != nullptr) {
+#pragma unroll 1
+        for (int j = 0; j < kFastItems; ++j) {
+            const int64_t item = item0 + j;
+            if (item >= total) break;
+            if (slow & (1u << j)) continue;
+            reinterpret_cast<uint32_t*>(ints8)[static_cast<size_t>(item) * (BSI_CHUNK_ELEMS / 4) + lane] = image[wib][j][lane];
+        }
+    }
+    // the planes: lane = (item j, 32-element unit w)
+    {
+        const int j = lane >> 3, w = lane & 7;
+        const int64_t item = item0 + j;
+        if (j < kFastItems && item < total && !(slow & (1u << j))) {
+            uint32_t y[8];
+            const uint4 lo = *reinterpret_cast<const uint4*>(&image[wib][j][w * 8]);
+            const uint4 hi = *reinterpret_cast<const uint4*>(&image[wib][j][w * 8 + 4]);
+            y[0] = lo.x; y[1] = lo.y; y[2] = lo.z; y[3] = lo.w;
+            y[4] = hi.x; y[5] = hi.y; y[6] = hi.z; y[7] = hi.w;
+            // bit b of image byte (element 8m + t) <-> bit (8m + t) of plane b's half-word: an 8x8 bit transpose
+            uint32_t a[8];
+#pragma unroll
+            for (int s2 = 0; s2 < 4; ++s2) {
+                const uint32_t l = y[s2], h = y[s2 + 4];
+                a[s2] = (l & 0x0F0F0F0Fu) | ((h << 4) & 0xF0F0F0F0u);
+                a[s2 + 4] = ((l >> 4) & 0x0F0F0F0Fu) | (h & 0xF0F0F0F0u);
+            }
+#pragma unroll
+            for (int b = 0; b < 8; b += 4)
+#pragma unroll
+                for (int s2 = b; s2 < b + 2; ++s2) {
+                    const uint32_t l = a[s2], h = a[s2 + 2];
+                    y[s2] = (l & 0x33333333u) | ((h << 2) & 0xCCCCCCCCu);
+                    y[s2 + 2] = ((l >> 2) & 0x33333333u) | (h & 0xCCCCCCCCu);
+                }
+#pragma unroll
+            for (int s2 = 0; s2 < 8; s2 += 2) {
+                const uint32_t l = y[s2], h = y[s2 + 1];
+                a[s2] = (l & 0x55555555u) | ((h << 1) & 0xAAAAAAAAu);
+                a[s2 + 1] = ((l >> 1) & 0x55555555u) | (h & 0xAAAAAAAAu);
+            }
+            BSI_ITEM_ROW_CHUNK(j, row, c)
+            uint32_t* out32 = reinterpret_cast<uint32_t*>(words) +
+                              (static_cast<size_t>(row) * slices * words_per_slice + static_cast<size_t>(c) * 4) * 2 + w;
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const int sl = t - (8 - slices);  // image bit t is slice t - (8 - slices)
+                if (sl >= 0) out32[static_cast<size_t>(sl) * words_per_slice * 2] = a[t];
+            }
+        }
+    }
+}
+#undef BSI_ITEM_ROW_CHUNK
 
 // Row-scale build: one block per row; pass 1 reduces the row maximum, pass 2 (row now in cache)
 // quantises and packs, one wave per group of 4 words.
@@ -496,7 +661,25 @@ extern "C" int bsi_hip_build_fixed(const void* x, int dtype, int64_t Q, int64_t 
     const int W = static_cast<int>((d + 63) / 64);
     const int chunks = static_cast<int>((d + 255) / 256);
     const double dec_scale = pow(10.0, static_cast<double>(decimal_places));
-    if (chunk_scale) {
+    if (chunk_scale && fixed_bits <= 8 && !(clip_k > 0.0f) && W % 4 == 0) {
+        const int64_t items = Q * chunks;
+#define BSI_LAUNCH_FAST(N)                                                                                          \
+    {                                                                                                               \
+        const int64_t waves = (items + (N) - 1) / (N);                                                              \
+        BSI_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((build_fixed_chunk_fast_kernel<T, N>), dim3(grid_for(waves)),   \
+                                                     dim3(kBlock), 0, as_stream(stream), static_cast<const T*>(x), Q, \
+                                                     d, chunks, fixed_bits, W, dec_scale,                            \
+                                                     reinterpret_cast<unsigned long long*>(words), shifts, scales,   \
+                                                     ints8));                                                        \
+    }
+        // a wave gets more items only once there are more than about 16 waves per SIMD (16384 in all)
+        if (items > 8 * 16384) BSI_LAUNCH_FAST(8)
+        else if (items > 4 * 16384) BSI_LAUNCH_FAST(4)
+        else if (items > 16384) BSI_LAUNCH_FAST(2)
+        else BSI_LAUNCH_FAST(1)
+#undef BSI_LAUNCH_FAST
+        BSI_LAUNCH_CHECK("build_fixed_chunk_fast_kernel");
+    } else if (chunk_scale) {
         BSI_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(build_fixed_chunk_kernel<T>, dim3(grid_for(Q * chunks)),
                                                      dim3(kBlock), 0, as_stream(stream), static_cast<const T*>(x), Q,
                                                      d, chunks, fixed_bits, W, dec_scale, clip_k,

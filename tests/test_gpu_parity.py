@@ -106,6 +106,33 @@ def test_build_fixed_matches_oracle(hip, oracle, Q, d, kind, bits, chunk):
     assert torch.equal(i8, i8b)
 
 
+def test_build_huge_magnitudes_take_the_wide_path(hip, oracle):
+    """Chunks holding |v * 10^dec| >= 2^31 leave the 32-bit fast path; their neighbours in the same wave do not."""
+    x = _inputs(6, 2048, 21)
+    x[0, 3] = 3.0e7          # 3e9 after scaling: beyond int32
+    x[2, 300] = -5.0e12
+    x[5, 2047] = 2.2e7       # 2.2e9: just beyond
+    x[4, 1000] = 2.1e7       # 2.1e9: just inside
+    ints, shifts, scales = oracle.quantize_fixed(x, 2, 7, True)
+    xd = dev(x)
+    words = torch.full((6, 7, 32), -1, dtype=torch.int64, device="cuda")
+    sh = torch.full(shifts.shape, -1, dtype=torch.int32, device="cuda")
+    sc = torch.zeros(scales.shape, dtype=torch.float32, device="cuda")
+    i8 = torch.full((6, 2048), 77, dtype=torch.int8, device="cuda")
+    hip.check(hip.lib.bsi_hip_build_fixed(xd.data_ptr(), 0, 6, 2048, 2, 7, 1, 0.0, words.data_ptr(), sh.data_ptr(),
+                                          sc.data_ptr(), i8.data_ptr(), st()), "build")
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(sh.cpu().numpy(), shifts)
+    np.testing.assert_array_equal(sc.cpu().numpy(), scales)
+    np.testing.assert_array_equal(host_u64(words), oracle.pack(ints, 7))
+    e = np.arange(2048)
+    pos = (e // 32) * 32 + ((e % 32) % 8) * 4 + (e % 32) // 8
+    want8 = np.zeros((6, 2048), dtype=np.int64)
+    want8[:, pos] = ints << 1
+    np.testing.assert_array_equal(i8.cpu().numpy().astype(np.int64), want8)
+    assert shifts.max() >= 30
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_build_half_inputs(hip, oracle, dtype):
     x = torch.from_numpy(_inputs(12, 1024, 5)).to(dtype)
