@@ -143,6 +143,37 @@ def main() -> int:
     if used_core == "valu":
         result["valu"] = valu
 
+    # peaks measured on this GPU by the library's probes (a pure v_mfma_i32_16x16x64_i8 loop, a pure
+    # v_and/v_bcnt loop, a streaming read of 1 GiB), next to the published figures the roofline uses
+    peaks = {"published": {"int8_mfma_TOPS": MFMA_I8_PEAK_TOPS, "hbm_GBs": HBM_PEAK_GBS}}
+    v = ctypes.c_double(0.0)
+    _lib.check(_lib.lib.bsi_hip_probe_mfma_i8(ctypes.byref(v), stream), "probe_mfma")
+    peaks["int8_mfma_TOPS"] = v.value / 1e12
+    _lib.check(_lib.lib.bsi_hip_probe_valu_popcount(ctypes.byref(v), stream), "probe_valu")
+    peaks["valu_and_bcnt_Tbitmac_s"] = v.value * 32 / 2 / 1e12   # one v_and + one v_bcnt per 32 bit-MACs
+    buf = torch.ones(1 << 30, dtype=torch.uint8, device="cuda")
+    _lib.check(_lib.lib.bsi_hip_probe_stream_read(buf.data_ptr(), buf.numel(), ctypes.byref(v), stream), "probe_read")
+    peaks["stream_read_GBs"] = v.value / 1e9
+    del buf
+    result["measured_peaks"] = peaks
+    result["roofline"]["frac_of_measured_mfma_peak"] = (int8_ops / (kern_us * 1e-6) / 1e12) / peaks["int8_mfma_TOPS"]
+
+    # dense baselines of the same shape on the same GPU (resident operands, same event timing)
+    Xd, Kd = X.cuda(), K.cuda()
+    dense = {}
+    for name, dt in (("fp32", torch.float32), ("bf16", torch.bfloat16)):
+        a, b = Xd.to(dt), Kd.to(dt)
+        for _ in range(5):
+            torch.matmul(a, b.T)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(20):
+            torch.matmul(a, b.T)
+        e1.record()
+        torch.cuda.synchronize()
+        dense[f"torch_matmul_{name}_us"] = e0.elapsed_time(e1) / 20 * 1e3
+    result["dense_baseline"] = dense
+
     if not args.no_cpu:
         from oracle import bsi_oracle
 
