@@ -496,6 +496,54 @@ def test_dot_row_stride_and_untouched_columns(hip, oracle):
         assert np.isnan(out[:, R:]).all()  # columns past R are not written
 
 
+def test_dot_row_stride_int8_image_and_few_rows(hip, oracle):
+    x, k, qb, kb, want_ints, want_out = _oracle_case(oracle, 70, 150, 1024, seed=8)
+    for tiled in ("int8-128", "int8-64"):
+        _, out = _run_dot(hip, qb, kb, 70, 150, 16, 7, 6, 2, tiled=tiled, with_ints8=True, want_ints=False, R_total=163)
+        np.testing.assert_array_equal(out[:, :150], want_out)
+        assert np.isnan(out[:, 150:]).all()
+    x, k, qb, kb, want_ints, want_out = _oracle_case(oracle, 9, 150, 1024, seed=9)
+    _, out = _run_dot(hip, qb, kb, 9, 150, 16, 7, 6, 2, tiled=True, with_ints8=True, want_ints=False, R_total=163)
+    np.testing.assert_array_equal(out[:, :150], want_out)
+    assert np.isnan(out[:, 150:]).all()
+
+
+def test_build_and_dot_replay_from_a_hip_graph(ops):
+    """Query build + dot launched on a side stream are captured once and replayed; every replay, with
+    eager work and synchronisations between them, gives the eager result for the input then in place."""
+    torch.manual_seed(3)
+    K = torch.randn(300, 1024) * 0.02
+    kcap, *_ = ops.build_bsi_keys_cuda(K, 2, 0.5)
+    xs = [torch.randn(40, 1024, device="cuda") for _ in range(3)]
+    xs_few = [torch.randn(5, 1024, device="cuda") for _ in range(3)]
+    for inputs in (xs, xs_few):   # the int8-image kernel, then the few-rows kernel
+        eager = []
+        for xi in inputs:
+            qc = ops.build_bsi_queries_cuda_batch_packed(xi, 2, 0.5)
+            eager.append(ops.batch_dot_product_multiquery_cuda_batch_caps(qc, kcap)[0].clone())
+        static_x = inputs[0].clone()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            qc = ops.build_bsi_queries_cuda_batch_packed(static_x, 2, 0.5)
+            ops.batch_dot_product_multiquery_cuda_batch_caps(qc, kcap)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            qc = ops.build_bsi_queries_cuda_batch_packed(static_x, 2, 0.5)
+            static_out = ops.batch_dot_product_multiquery_cuda_batch_caps(qc, kcap)[0]
+        for rep in range(2):
+            for xi, want in zip(inputs, eager):
+                static_x.copy_(xi)
+                g.replay()
+                torch.cuda.synchronize()
+                assert torch.equal(static_out, want)
+                other = ops.build_bsi_queries_cuda_batch_packed(inputs[(rep + 1) % 3], 2, 0.5)   # eager work in between
+                ops.batch_dot_product_multiquery_cuda_batch_caps(other, kcap)
+                torch.cuda.synchronize()
+
+
 # ------------------------------------------------------------------ through the bsi_ops mirror
 
 
