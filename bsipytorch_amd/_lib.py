@@ -49,6 +49,7 @@ PROTOTYPES = {
     "bsi_hip_set_option": [_i, _i],
     "bsi_hip_dot_workspace_bytes": [_i64, _i, _i],
     "bsi_hip_dot": [_vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _i, _i64, _i64, _f, _i64, _vp, _vp, _i, _vp, _sz, _vp],
+    "bsi_hip_dot_bias": [_vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _i, _i64, _i64, _f, _i64, _vp, _vp, _i, _vp, _sz, _vp],
     "bsi_hip_dot_ewah_query": [_vp, _vp, _vp, _i, _i, _vp, _i, _vp, _vp, _i, _i64, _f, _vp, _vp, _vp],
     "bsi_hip_dot_timed": [_vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _i, _i64, _i64, _f, _i64, _vp, _i, _vp, _sz, _i,
                           ctypes.POINTER(_f), _vp],

@@ -512,7 +512,8 @@ def key_operand(keys: "PrebuiltBSIKeysCUDA", Q: int, Sa: int, core: int):
     return keys.words.data_ptr(), keys.layout
 
 
-def _dot(words, ints8, scales, scale_stride, Sa, W, keys: PrebuiltBSIKeysCUDA, Q, decimals_q, chunk_ints=None, core=None):
+def _dot(words, ints8, scales, scale_stride, Sa, W, keys: PrebuiltBSIKeysCUDA, Q, decimals_q, chunk_ints=None, core=None,
+         bias=None):
     f = _flags()
     dev = words.device
     R = keys.num_keys
@@ -532,10 +533,18 @@ def _dot(words, ints8, scales, scale_stride, Sa, W, keys: PrebuiltBSIKeysCUDA, Q
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
     kptr, klayout = key_operand(keys, Q, Sa, core)
-    check(lib.bsi_hip_dot(words.data_ptr(), _ptr(ints8), scales.data_ptr(), scale_stride, Sa, W,
-                          kptr, klayout, keys.slice_weights.data_ptr(), keys.Sb, R, Q,
-                          _scale_inv(decimals_q, keys.decimals), R, out.data_ptr(), _ptr(chunk_ints), core,
-                          _ptr(ws), ws_bytes, _stream()), "bsi_hip_dot")
+    if bias is not None and chunk_ints is None:
+        check(lib.bsi_hip_dot_bias(words.data_ptr(), _ptr(ints8), scales.data_ptr(), scale_stride, Sa, W,
+                                   kptr, klayout, keys.slice_weights.data_ptr(), keys.Sb, R, Q,
+                                   _scale_inv(decimals_q, keys.decimals), R, bias.data_ptr(), out.data_ptr(), core,
+                                   _ptr(ws), ws_bytes, _stream()), "bsi_hip_dot_bias")
+    else:
+        check(lib.bsi_hip_dot(words.data_ptr(), _ptr(ints8), scales.data_ptr(), scale_stride, Sa, W,
+                              kptr, klayout, keys.slice_weights.data_ptr(), keys.Sb, R, Q,
+                              _scale_inv(decimals_q, keys.decimals), R, out.data_ptr(), _ptr(chunk_ints), core,
+                              _ptr(ws), ws_bytes, _stream()), "bsi_hip_dot")
+        if bias is not None:
+            out += bias
     ns = 0
     if prof:
         e1.record()
@@ -554,9 +563,11 @@ def _dot_result(out, ns, Q, R):
     return out, int(ns), per_q, per_s
 
 
-def batch_dot_product_multiquery_cuda_batch_caps(query_batch_cap, keyset_cuda_cap):
+def batch_dot_product_multiquery_cuda_batch_caps(query_batch_cap, keyset_cuda_cap, bias=None):
     """bsi_cuda.cpp:658-815 -> (out[Q, R] float32 on the device, dot_ns_total, ns_per_query, ns_per_scalar).
-    The times are zero unless BSI_PROFILE=1 (which synchronises), as in the reference."""
+    The times are zero unless BSI_PROFILE=1 (which synchronises), as in the reference.
+    ``bias`` (not in the reference's signature): an optional float32 [R] device tensor added to every output
+    row in the same launch, rounded as ``out + bias`` would be."""
     keys = _capsule(keyset_cuda_cap, PrebuiltBSIKeysCUDA, "Invalid CUDA keys capsule")
     qb = _capsule(query_batch_cap, PrebuiltBSIQueryBatchCUDA, "Invalid CUDA query-batch capsule")
     _check(qb.words is not None and qb.slice_weights is not None, "Query batch tensors are not defined")
@@ -582,7 +593,10 @@ def batch_dot_product_multiquery_cuda_batch_caps(query_batch_cap, keyset_cuda_ca
         scales, stride = qb.row_scales, 1
     _check(qb.decimals == keys.decimals,
            f"Decimal mismatch between queries and keys: q={qb.decimals} k={keys.decimals}")
-    out, ns = _dot(qb.words, qb.ints8, scales, stride, int(Sa), int(W), keys, int(Q), qb.decimals)
+    if bias is not None:
+        _check(bias.is_cuda and bias.dtype == torch.float32 and bias.dim() == 1 and bias.numel() == R and bias.is_contiguous(),
+               "bias must be a contiguous float32 CUDA tensor of [R]")
+    out, ns = _dot(qb.words, qb.ints8, scales, stride, int(Sa), int(W), keys, int(Q), qb.decimals, bias=bias)
     return _dot_result(out, ns, Q, R)
 
 

@@ -761,7 +761,7 @@ __global__ __launch_bounds__(I8Cfg<T>::kBlock) void dot_mfma_i8_kernel(
     const int8_t* __restrict__ A8, const float* __restrict__ qscale, int qscale_stride,
     const int8_t* __restrict__ K8,  // int8 key image [R, chunks * 256]
     const float* __restrict__ Bw, int Sb, int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv,
-    int64_t R_total, float* __restrict__ out, int* __restrict__ chunk_ints) {
+    int64_t R_total, float* __restrict__ out, int* __restrict__ chunk_ints, const float* __restrict__ bias) {
     using C = I8Cfg<T>;
     constexpr int WM = C::kWM, WN = C::kWN;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];  // C::kLds
@@ -919,26 +919,32 @@ __global__ __launch_bounds__(I8Cfg<T>::kBlock) void dot_mfma_i8_kernel(
 #pragma unroll
     for (int a = 0; a < WM; ++a) {
         const int64_t rb = r0 + wr * (WM * 16) + a * 16 + lg * 4;
-        float bs[4];
+        float bs[4], bi[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) bs[e] = (rb + e < R) ? Bw[(rb + e) * Sb] : 0.0f;
+        for (int e = 0; e < 4; ++e) {
+            bs[e] = (rb + e < R) ? Bw[(rb + e) * Sb] : 0.0f;
+            bi[e] = (bias != nullptr && rb + e < R) ? bias[rb + e] : 0.0f;
+        }
 #pragma unroll
         for (int b = 0; b < WN; ++b)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) accf[a][b][e] *= down;
+            for (int e = 0; e < 4; ++e) {
+                // (acc * key scale) * scale_inv, then + bias: each step rounded on its own, as separate kernels would
+                float v = ((accf[a][b][e] * down) * bs[e]) * scale_inv;
+                if (bias != nullptr) v = v + bi[e];
+                accf[a][b][e] = v;
+            }
 #pragma unroll
         for (int b = 0; b < WN; ++b) {
             const int64_t q = q0 + wq * (WN * 16) + b * 16 + ln;
             if (q >= Q) continue;
             float* dst = out + static_cast<size_t>(q) * R_total + rb;
             if (rb + 3 < R && ((reinterpret_cast<uintptr_t>(dst) & 15) == 0)) {
-                *reinterpret_cast<float4*>(dst) =
-                    make_float4((accf[a][b][0] * bs[0]) * scale_inv, (accf[a][b][1] * bs[1]) * scale_inv,
-                                (accf[a][b][2] * bs[2]) * scale_inv, (accf[a][b][3] * bs[3]) * scale_inv);
+                *reinterpret_cast<float4*>(dst) = make_float4(accf[a][b][0], accf[a][b][1], accf[a][b][2], accf[a][b][3]);
             } else {
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
-                    if (rb + e < R) dst[e] = (accf[a][b][e] * bs[e]) * scale_inv;
+                    if (rb + e < R) dst[e] = accf[a][b][e];
             }
         }
     }
@@ -964,7 +970,7 @@ __global__ __launch_bounds__(1024) void dot_mfma_stream_kernel(
     const int8_t* __restrict__ A8, const float* __restrict__ qscale, int qscale_stride,
     const unsigned long long* __restrict__ B64,  // tiled key planes, Sb = 6
     const float* __restrict__ Bw, int chunks, int pass_chunks, int64_t R, int64_t Q, int down_shift, float scale_inv,
-    int64_t R_total, float* __restrict__ out, int* __restrict__ chunk_ints) {
+    int64_t R_total, float* __restrict__ out, int* __restrict__ chunk_ints, const float* __restrict__ bias) {
     extern __shared__ __attribute__((aligned(16))) int ints[];  // [pass_chunks][KT][NT][16 queries][16 keys]
     constexpr int kSlot = KT * NT * 256;
 
@@ -1070,7 +1076,11 @@ __global__ __launch_bounds__(1024) void dot_mfma_stream_kernel(
         }
         if (pend < chunks) __syncthreads();
     }
-    if (cvalid) out[static_cast<size_t>(cq) * R_total + cr] = (accf * Bw[cr * 6]) * scale_inv;
+    if (cvalid) {
+        float v = (accf * Bw[cr * 6]) * scale_inv;
+        if (bias != nullptr) v = v + bias[cr];
+        out[static_cast<size_t>(cq) * R_total + cr] = v;
+    }
 }
 
 // ------------------------------------------------------------------ one EWAH-compressed query, decode inline
@@ -1356,6 +1366,15 @@ __global__ void dot_valu_generic_kernel(const unsigned long long* __restrict__ A
     out[static_cast<size_t>(q) * R_total + r] = (acc * Bw[r * Sb]) * scale_inv;
 }
 
+// out[q, r] += bias[r] for the kernels that do not add the bias in their own epilogue
+__global__ void add_bias_kernel(float* __restrict__ out, const float* __restrict__ bias, int64_t Q, int64_t R,
+                                int64_t R_total) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= Q * R) return;
+    const int64_t q = i / R, r = i - q * R;
+    out[q * R_total + r] = out[q * R_total + r] + bias[r];
+}
+
 static int launch_planes_to_int8(const uint64_t* words, int64_t rows, int S, int W64, int8_t* out, hipStream_t st) {
     const int chunks = (W64 + 3) / 4;
     const int64_t total = rows * chunks * 8;
@@ -1418,7 +1437,7 @@ static void launch_mfma_ws(const int8_t* A8, const float* qscale, int stride, co
 template <int T>
 static void launch_mfma_i8_t(const int8_t* A8, const float* qscale, int stride, const int8_t* K8, const float* Bw,
                              int Sb, int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv,
-                             int64_t R_total, float* out, int32_t* chunk_ints, hipStream_t st) {
+                             int64_t R_total, float* out, int32_t* chunk_ints, const float* bias, hipStream_t st) {
     using C = I8Cfg<T>;
     const dim3 grid(static_cast<unsigned>((R + T - 1) / T), static_cast<unsigned>((Q + T - 1) / T));
     static bool configured = false;
@@ -1431,29 +1450,29 @@ static void launch_mfma_i8_t(const int8_t* A8, const float* qscale, int stride, 
     }
     if (chunk_ints)
         hipLaunchKernelGGL((dot_mfma_i8_kernel<T, true>), grid, dim3(C::kBlock), C::kLds, st, A8, qscale, stride, K8,
-                           Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints);
+                           Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias);
     else
         hipLaunchKernelGGL((dot_mfma_i8_kernel<T, false>), grid, dim3(C::kBlock), C::kLds, st, A8, qscale, stride, K8,
-                           Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints);
+                           Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias);
 }
 
 static void launch_mfma_i8(const int8_t* A8, const float* qscale, int stride, const int8_t* K8, const float* Bw, int Sb,
                            int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv, int64_t R_total,
-                           float* out, int32_t* chunk_ints, hipStream_t st) {
+                           float* out, int32_t* chunk_ints, const float* bias, hipStream_t st) {
     // 128 x 128 tiles unless they would leave most of the 256 CUs without a workgroup
     const int64_t big = ((R + 127) / 128) * ((Q + 127) / 128);
     if (big >= g_i8_small_tile_below)
         launch_mfma_i8_t<128>(A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out,
-                              chunk_ints, st);
+                              chunk_ints, bias, st);
     else
         launch_mfma_i8_t<64>(A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out,
-                             chunk_ints, st);
+                             chunk_ints, bias, st);
 }
 
 template <int NT, int KT>
 static void launch_mfma_stream(const int8_t* A8, const float* qscale, int stride, const uint64_t* B, const float* Bw,
                                int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv, int64_t R_total,
-                               float* out, int32_t* chunk_ints, hipStream_t st) {
+                               float* out, int32_t* chunk_ints, const float* bias, hipStream_t st) {
     constexpr int kSlot = KT * NT * 256;
     const int64_t ntiles = (R + 15) / 16;
     const dim3 grid(static_cast<unsigned>((ntiles + KT - 1) / KT), static_cast<unsigned>((Q + 16 * NT - 1) / (16 * NT)));
@@ -1468,11 +1487,11 @@ static void launch_mfma_stream(const int8_t* A8, const float* qscale, int stride
     if (chunk_ints)
         hipLaunchKernelGGL((dot_mfma_stream_kernel<NT, KT, true>), grid, dim3(waves * 64), lds, st, A8, qscale, stride,
                            reinterpret_cast<const unsigned long long*>(B), Bw, chunks, pass_chunks, R, Q, down_shift,
-                           scale_inv, R_total, out, chunk_ints);
+                           scale_inv, R_total, out, chunk_ints, bias);
     else
         hipLaunchKernelGGL((dot_mfma_stream_kernel<NT, KT, false>), grid, dim3(waves * 64), lds, st, A8, qscale, stride,
                            reinterpret_cast<const unsigned long long*>(B), Bw, chunks, pass_chunks, R, Q, down_shift,
-                           scale_inv, R_total, out, chunk_ints);
+                           scale_inv, R_total, out, chunk_ints, bias);
 }
 
 template <bool kTiled>
@@ -1532,10 +1551,13 @@ extern "C" size_t bsi_hip_dot_workspace_bytes(int64_t Q, int W64, int core) {
     return static_cast<size_t>(Q) * static_cast<size_t>((W64 + 3) / 4) * 256;
 }
 
-extern "C" int bsi_hip_dot(const uint64_t* A, const int8_t* A_ints8, const float* A_chunk_scales, int A_scale_stride,
-                           int Sa, int W64, const uint64_t* B, int b_layout, const float* Bw, int Sb, int64_t R,
-                           int64_t Q, float scale_inv, int64_t R_total, float* out, int32_t* chunk_ints, int core,
-                           void* workspace, size_t workspace_bytes, void* stream) {
+// Validation, kernel selection and launch.  `bias` (optional) is added to every output; *bias_fused tells
+// the caller whether the selected kernel did that in its own epilogue.
+static int dot_launch(const uint64_t* A, const int8_t* A_ints8, const float* A_chunk_scales, int A_scale_stride,
+                      int Sa, int W64, const uint64_t* B, int b_layout, const float* Bw, int Sb, int64_t R, int64_t Q,
+                      float scale_inv, int64_t R_total, float* out, int32_t* chunk_ints, int core, void* workspace,
+                      size_t workspace_bytes, void* stream, const float* bias, bool* bias_fused) {
+    *bias_fused = false;
     BSI_REQUIRE(Q >= 0 && R >= 0, "negative Q or R");
     BSI_REQUIRE(W64 >= 1, "W64 must be >= 1");
     BSI_REQUIRE(Sa >= 1 && Sa <= 16 && Sb >= 1 && Sb <= 16, "Sa and Sb must be in [1, 16]");
@@ -1570,19 +1592,21 @@ extern "C" int bsi_hip_dot(const uint64_t* A, const int8_t* A_ints8, const float
         if (b_layout == BSI_LAYOUT_INT8) {
             BSI_REQUIRE((reinterpret_cast<uintptr_t>(B) & 15) == 0, "int8 key image must be 16-byte aligned");
             launch_mfma_i8(A8, A_chunk_scales, A_scale_stride, reinterpret_cast<const int8_t*>(B), Bw, Sb, chunks, R, Q,
-                           down_shift, scale_inv, R_total, out, chunk_ints, st);
+                           down_shift, scale_inv, R_total, out, chunk_ints, bias, st);
             BSI_LAUNCH_CHECK("dot_mfma_i8_kernel");
+            *bias_fused = true;
             return BSI_OK;
         }
         const bool tiled = (b_layout == BSI_LAYOUT_TILED16);
         if (Sb == 6 && tiled && Q <= kStreamMaxQ) {
             // two key tiles per workgroup halve the query re-reads once there are enough tiles to fill the GPU
             const bool two = (R + 15) / 16 >= 1024;
-#define BSI_STREAM_ARGS A8, A_chunk_scales, A_scale_stride, B, Bw, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, st
+#define BSI_STREAM_ARGS A8, A_chunk_scales, A_scale_stride, B, Bw, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias, st
             if (Q <= 16) { if (two) launch_mfma_stream<1, 2>(BSI_STREAM_ARGS); else launch_mfma_stream<1, 1>(BSI_STREAM_ARGS); }
             else { if (two) launch_mfma_stream<2, 2>(BSI_STREAM_ARGS); else launch_mfma_stream<2, 1>(BSI_STREAM_ARGS); }
 #undef BSI_STREAM_ARGS
             BSI_LAUNCH_CHECK("dot_mfma_stream_kernel");
+            *bias_fused = true;
             return BSI_OK;
         }
         if (Sb == 6 && tiled) {
@@ -1621,6 +1645,37 @@ extern "C" int bsi_hip_dot(const uint64_t* A, const int8_t* A_ints8, const float
                        out, chunk_ints);
     BSI_LAUNCH_CHECK("dot_valu_generic_kernel");
     return BSI_OK;
+}
+
+static int dot_with_bias(const uint64_t* A, const int8_t* A_ints8, const float* A_chunk_scales, int A_scale_stride,
+                         int Sa, int W64, const uint64_t* B, int b_layout, const float* Bw, int Sb, int64_t R, int64_t Q,
+                         float scale_inv, int64_t R_total, float* out, int32_t* chunk_ints, int core, void* workspace,
+                         size_t workspace_bytes, void* stream, const float* bias) {
+    bool fused = false;
+    const int rc = dot_launch(A, A_ints8, A_chunk_scales, A_scale_stride, Sa, W64, B, b_layout, Bw, Sb, R, Q, scale_inv,
+                              R_total, out, chunk_ints, core, workspace, workspace_bytes, stream, bias, &fused);
+    if (rc != BSI_OK || bias == nullptr || fused || Q == 0 || R == 0) return rc;
+    const int64_t total = Q * R;
+    hipLaunchKernelGGL(add_bias_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, as_stream(stream),
+                       out, bias, Q, R, R_total);
+    BSI_LAUNCH_CHECK("add_bias_kernel");
+    return BSI_OK;
+}
+
+extern "C" int bsi_hip_dot(const uint64_t* A, const int8_t* A_ints8, const float* A_chunk_scales, int A_scale_stride,
+                           int Sa, int W64, const uint64_t* B, int b_layout, const float* Bw, int Sb, int64_t R,
+                           int64_t Q, float scale_inv, int64_t R_total, float* out, int32_t* chunk_ints, int core,
+                           void* workspace, size_t workspace_bytes, void* stream) {
+    return dot_with_bias(A, A_ints8, A_chunk_scales, A_scale_stride, Sa, W64, B, b_layout, Bw, Sb, R, Q, scale_inv,
+                         R_total, out, chunk_ints, core, workspace, workspace_bytes, stream, nullptr);
+}
+
+extern "C" int bsi_hip_dot_bias(const uint64_t* A, const int8_t* A_ints8, const float* A_chunk_scales,
+                                int A_scale_stride, int Sa, int W64, const uint64_t* B, int b_layout, const float* Bw,
+                                int Sb, int64_t R, int64_t Q, float scale_inv, int64_t R_total, const float* bias,
+                                float* out, int core, void* workspace, size_t workspace_bytes, void* stream) {
+    return dot_with_bias(A, A_ints8, A_chunk_scales, A_scale_stride, Sa, W64, B, b_layout, Bw, Sb, R, Q, scale_inv,
+                         R_total, out, nullptr, core, workspace, workspace_bytes, stream, bias);
 }
 
 extern "C" int bsi_hip_dot_ewah_query(const uint64_t* comp_words, const int64_t* comp_off, const int32_t* comp_len,

@@ -120,8 +120,14 @@ class BSIQuantizedLinear(nn.Module):
             c["build_kernel_ns_total"] += int(t_ns)
             c["build_calls"] += 1
 
+        bias = self.bias
+        # fp32 activations: the bias goes into the dot's epilogue (same rounding as scores + bias); in half
+        # precision the reference adds it after the cast, so it stays a separate addition there
+        fuse_bias = (use_packed and bias is not None and original_dtype == torch.float32 and bias.is_cuda
+                     and bias.dtype == torch.float32 and bias.is_contiguous())
         if use_packed:
-            scores, ns_total, ns_q, ns_s = bsi_ops.batch_dot_product_multiquery_cuda_batch_caps(qcap, self._bsi_keys_cuda)
+            scores, ns_total, ns_q, ns_s = bsi_ops.batch_dot_product_multiquery_cuda_batch_caps(
+                qcap, self._bsi_keys_cuda, bias if fuse_bias else None)
         else:
             scores, ns_total, ns_q, ns_s = bsi_ops.batch_dot_product_multiquery_cuda_caps(qcap, self._bsi_keys_cuda)
         c["dot_kernel_ns_per_query_last"] = float(ns_q)
@@ -133,8 +139,7 @@ class BSIQuantizedLinear(nn.Module):
 
         if scores.dtype != original_dtype:
             scores = scores.to(dtype=original_dtype)
-        bias = self.bias
-        if bias is not None:
+        if bias is not None and not fuse_bias:
             if bias.dtype != original_dtype or bias.device != scores.device:
                 bias = bias.to(device=scores.device, dtype=original_dtype)
             scores = scores + bias

@@ -179,6 +179,15 @@ int bsi_hip_dot(const uint64_t* A, const int8_t* A_ints8, const float* A_chunk_s
                 float scale_inv, int64_t R_total, float* out, int32_t* chunk_ints, int core, void* workspace,
                 size_t workspace_bytes, void* stream);
 
+/* bsi_hip_dot followed by out[q, r] += bias[r] (bias: float [R], may be NULL), the two steps of a BSI-linear
+ * forward (scores = dot(...); scores + bias, verify_accuracy_bsi.py:185-209) in one call.  The sum is rounded as
+ * the separate addition would round it; the matrix-core kernels add the bias in their epilogue, the others
+ * are followed by a small addition kernel. */
+int bsi_hip_dot_bias(const uint64_t* A, const int8_t* A_ints8, const float* A_chunk_scales, int A_scale_stride, int Sa,
+                     int W64, const uint64_t* B, int b_layout, const float* Bw, int Sb, int64_t R, int64_t Q,
+                     float scale_inv, int64_t R_total, const float* bias, float* out, int core, void* workspace,
+                     size_t workspace_bytes, void* stream);
+
 /* The same dot for ONE query whose slices are EWAH streams (the hybrid query form of
  * build_bsi_query_cuda_hybrid, bsi_cuda.cpp:386-431): stream s at comp_words + comp_off[s], comp_len[s]
  * words, decoded to W64 words per slice inside the kernel's load stage with the semantics of

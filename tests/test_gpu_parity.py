@@ -508,6 +508,41 @@ def test_dot_row_stride_int8_image_and_few_rows(hip, oracle):
     assert np.isnan(out[:, 150:]).all()
 
 
+@pytest.mark.parametrize("Q,tiled", [(70, "int8-128"), (70, "int8-64"), (9, True), (70, True), (70, False)])
+def test_dot_bias_entry_point(hip, oracle, Q, tiled):
+    """bsi_hip_dot_bias == bsi_hip_dot followed by a float addition of the bias row, bit for bit, whether the
+    kernel adds it in its epilogue (int8 image, few rows) or the library appends an addition kernel."""
+    R, d, W = 150, 1024, 16
+    x, k, qb, kb, want_ints, want_out = _oracle_case(oracle, Q, R, d, seed=Q)
+    rng = np.random.default_rng(1)
+    bias = rng.standard_normal(R).astype(np.float32)
+    L = hip.lib
+    A, scales, Bc, Bw = dev(qb["words"]), dev(qb["scales"]), dev(kb["words"]), dev(kb["slice_weights"])
+    a8 = torch.zeros((Q, 4 * 256), dtype=torch.int8, device="cuda")
+    hip.check(L.bsi_hip_planes_to_int8(A.data_ptr(), Q, 7, W, a8.data_ptr(), st()), "p2i8")
+    if tiled in ("int8-128", "int8-64"):
+        hip.check(L.bsi_hip_set_option(hip.OPT_I8_SMALL_TILE_BELOW, 0 if tiled == "int8-128" else 1 << 30), "opt")
+        B = torch.zeros((R, 4 * 256), dtype=torch.int8, device="cuda")
+        hip.check(L.bsi_hip_planes_to_int8(Bc.data_ptr(), R, 6, W, B.data_ptr(), st()), "image")
+        layout = 2
+    elif tiled:
+        B = torch.zeros((((R + 15) // 16) * 4 * 6 * 64,), dtype=torch.int64, device="cuda")
+        hip.check(L.bsi_hip_tile_key_planes(Bc.data_ptr(), R, 6, W, B.data_ptr(), st()), "tile")
+        layout = 1
+    else:
+        B, layout = Bc, 0
+    bd = dev(bias)
+    out = torch.full((Q, R + 5), float("nan"), dtype=torch.float32, device="cuda")
+    hip.check(L.bsi_hip_dot_bias(A.data_ptr(), a8.data_ptr(), scales.data_ptr(), 4, 7, W, B.data_ptr(), layout,
+                                 Bw.data_ptr(), 6, R, Q, float(np.float32(1e-4)), R + 5, bd.data_ptr(), out.data_ptr(),
+                                 2, None, 0, st()), "dot_bias")
+    torch.cuda.synchronize()
+    hip.check(L.bsi_hip_set_option(hip.OPT_I8_SMALL_TILE_BELOW, 100), "opt")
+    got = out.cpu().numpy()
+    np.testing.assert_array_equal(got[:, :R], want_out + bias[None, :])
+    assert np.isnan(got[:, R:]).all()
+
+
 def test_build_and_dot_replay_from_a_hip_graph(ops):
     """Query build + dot launched on a side stream are captured once and replayed; every replay, with
     eager work and synchronisations between them, gives the eager result for the input then in place."""
