@@ -10,6 +10,13 @@
 //         v_mfma_i32_16x16x64_i8 accumulates 2^(16-Sa-Sb) * I per chunk.  Keys are the M operand,
 //         queries the N operand, so a lane owns one query column: its chunk scale is one value.
 //
+//         Kernels of this core, chosen by bsi_hip_dot from the key layout and the number of query rows:
+//           dot_mfma_i8_kernel       compute-bound calls on the cached int8 image of the keys
+//           dot_mfma_stream_kernel   a few query rows: streams the packed planes once (bandwidth-bound)
+//           dot_mfma_stream_ewah_kernel   the same for one query handed over as EWAH streams
+//           dot_mfma_ws_kernel       many rows on tiled planes (producer waves recombine the planes)
+//           dot_mfma_kernel          canonical planes or slice counts other than 6
+//
 // Both feed the same fp32 epilogue, in chunk order:  acc = fmaf((float)I, qscale[q,c], acc), then
 // out = (acc * bscale[r]) * scale_inv.  bscale is a power of two, so hoisting it out of the chain is
 // exact and the result is bit-identical to fmaf((float)I, qscale*bscale, acc) of the reference
