@@ -147,3 +147,44 @@ def test_dot_error_paths_on_host():
         bsi_ops.build_bsi_keys_cuda(torch.zeros(4), 2)
     with pytest.raises(RuntimeError, match="1D"):
         bsi_ops.build_bsi_query_cuda(torch.zeros(4, 4), 2)
+
+
+def test_key_operand_selection_and_new_flags(monkeypatch):
+    """Which key representation a dot reads: packed planes for a few query rows or the popcount core, the cached
+    int8 image otherwise (host logic only: the tensors are never touched)."""
+    from bsipytorch_amd import _lib, bsi_ops
+
+    for k in list(os.environ):
+        if k.startswith("BSI_"):
+            monkeypatch.delenv(k)
+    bsi_ops._reset_flag_cache()
+    f = bsi_ops._flags()
+    assert f["key_image"] and f["ewah_inline"]
+    keys = bsi_ops.PrebuiltBSIKeysCUDA()
+    keys.words = torch.zeros(4, dtype=torch.int64)
+    keys.layout = _lib.LAYOUT_TILED16
+    keys.ints8 = torch.zeros(16, dtype=torch.int8)
+    planes = (keys.words.data_ptr(), _lib.LAYOUT_TILED16)
+    image = (keys.ints8.data_ptr(), _lib.LAYOUT_INT8)
+    assert bsi_ops.key_operand(keys, 1, 7, _lib.CORE_AUTO) == planes
+    assert bsi_ops.key_operand(keys, 32, 7, _lib.CORE_MFMA) == planes
+    assert bsi_ops.key_operand(keys, 33, 7, _lib.CORE_AUTO) == image
+    assert bsi_ops.key_operand(keys, 512, 7, _lib.CORE_VALU) == planes      # the popcount core reads planes
+    assert bsi_ops.key_operand(keys, 512, 12, _lib.CORE_AUTO) == planes     # values wider than int8
+    keys.ints8 = None
+    assert bsi_ops.key_operand(keys, 512, 7, _lib.CORE_AUTO) == planes
+    monkeypatch.setenv("BSI_KEY_INT8_IMAGE", "0")
+    monkeypatch.setenv("BSI_EWAH_INLINE", "0")
+    bsi_ops._reset_flag_cache()
+    f = bsi_ops._flags()
+    assert not f["key_image"] and not f["ewah_inline"]
+    bsi_ops._reset_flag_cache()
+
+
+def test_set_option_validates_on_host():
+    from bsipytorch_amd import _lib
+
+    assert _lib.lib.bsi_hip_set_option(_lib.OPT_I8_SMALL_TILE_BELOW, 100) == 0
+    assert _lib.lib.bsi_hip_set_option(_lib.OPT_I8_SMALL_TILE_BELOW, -1) == 1
+    assert _lib.lib.bsi_hip_set_option(999, 1) == 1
+    assert b"unknown option" in _lib.lib.bsi_hip_last_error()
