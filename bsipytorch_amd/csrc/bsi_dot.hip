@@ -702,21 +702,21 @@ __device__ __forceinline__ void load16_to_lds(bsi_rsrc r, uint32_t lane_off, uin
                                              static_cast<int>(wave_off), 0, 0);
 }
 
-// Tile configuration: T keys x T queries per workgroup (T = 128, or 64 for grids that would leave
-// most CUs without a workgroup), MFMA waves arranged 2 (keys) x kWavesN (queries), each WM x WN
-// tiles of 16 x 16; one loader wave per 32 rows.
-static int g_i8_small_tile_below = 100;  // workgroups of 128 x 128 below which 64 x 64 tiles are used (tunable)
+// Tile configuration: TM keys x TN queries per workgroup (128 x 128, 128 x 64 or 64 x 64; the smaller ones
+// for grids that would leave CUs without a workgroup), MFMA waves arranged 2 (keys) x kWavesN (queries),
+// each WM x WN tiles of 16 x 16; one loader wave per 64 operand rows.
+static int g_i8_tile = 0;  // 0 = by grid size; 128, 12864 (128 keys x 64 queries) or 64 force a tile
 
-template <int T>
+template <int TM, int TN>
 struct I8Cfg {
-    static constexpr int kWM = T / 32;                 // 16-key tiles per wave (2 waves along the keys)
+    static constexpr int kWM = TM / 32;                // 16-key tiles per wave (2 waves along the keys)
     static constexpr int kWN = 2;                      // 16-query tiles per wave
-    static constexpr int kWavesN = T / 32;             // waves along the queries
+    static constexpr int kWavesN = TN / 32;            // waves along the queries
     static constexpr int kConsumers = 2 * kWavesN;
-    static constexpr int kLoaders = T / 32;
+    static constexpr int kLoaders = (TM + TN) / 64;    // a loader wave moves 64 of the TM + TN operand rows
     static constexpr int kBlock = (kConsumers + kLoaders) * 64;
-    static constexpr int kOperand = T * 128;           // bytes of one operand tile of one half-chunk
-    static constexpr int kStage = 2 * kOperand;        // keys then queries
+    static constexpr int kOperandK = TM * 128;         // bytes of the key tile of one half-chunk
+    static constexpr int kStage = (TM + TN) * 128;     // keys then queries
     static constexpr int kScaleBytes = 4 * kLoaders * 256;  // chunk scales: ring of 4 chunks x loader regions x 64 floats
     static constexpr int kLds = 4 * kStage + kScaleBytes;
 };
@@ -763,56 +763,57 @@ __device__ __forceinline__ void i8_consume_half(const unsigned char* __restrict_
     }
 }
 
-template <int T, bool kInts>
-__global__ __launch_bounds__(I8Cfg<T>::kBlock) void dot_mfma_i8_kernel(
+template <int TM, int TN, bool kInts>
+__global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
     const int8_t* __restrict__ A8, const float* __restrict__ qscale, int qscale_stride,
     const int8_t* __restrict__ K8,  // int8 key image [R, chunks * 256]
     const float* __restrict__ Bw, int Sb, int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv,
     int64_t R_total, float* __restrict__ out, int* __restrict__ chunk_ints, const float* __restrict__ bias) {
-    using C = I8Cfg<T>;
+    using C = I8Cfg<TM, TN>;
     constexpr int WM = C::kWM, WN = C::kWN;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];  // C::kLds
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int64_t r0 = static_cast<int64_t>(blockIdx.x) * T;
-    const int64_t q0 = static_cast<int64_t>(blockIdx.y) * T;
+    const int64_t r0 = static_cast<int64_t>(blockIdx.x) * TM;
+    const int64_t q0 = static_cast<int64_t>(blockIdx.y) * TN;
     const size_t rowbytes = static_cast<size_t>(chunks) * 256;
     const int halves = chunks * 2;
     unsigned char* const scale_lds = lds + 4 * C::kStage;  // [chunk & 3][loader][64] floats
 
     if (wave >= C::kConsumers) {
-        // ---- loader wave lw: rows 32 lw .. 32 lw + 31 of both operand tiles of every stage (4 + 4 loads of
-        // 1 KiB), plus the chunk scales of 64 queries once per chunk.
+        // ---- loader wave lw: 8 of the stage's groups of 8 rows (the TM key rows, then the TN query rows: a
+        // load moves 1 KiB = 8 rows x 128 bytes), plus the chunk scales of 64 queries once per chunk.
         const int lw = wave - C::kConsumers;
         const bsi_rsrc rk = make_rsrc(K8 + static_cast<size_t>(r0) * rowbytes, static_cast<size_t>(R - r0) * rowbytes);
         const bsi_rsrc rq = make_rsrc(A8 + static_cast<size_t>(q0) * rowbytes, static_cast<size_t>(Q - q0) * rowbytes);
         const bsi_rsrc rs = make_rsrc(qscale + q0 * qscale_stride, static_cast<size_t>(Q - q0) * qscale_stride * 4);
-        uint32_t koff[4], qoff[4];
+        // the stage has (TM + TN) / 8 groups of 8 rows, keys first; loader lw moves groups lw, lw + kLoaders, ...
+        uint32_t off[8];
+        bool is_key[8];  // wave-uniform
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int rowl = (4 * lw + i) * 8 + (lane >> 3);                                 // tile row this lane fetches
+        for (int i = 0; i < 8; ++i) {
+            const int g = lw + C::kLoaders * i;
+            is_key[i] = g < TM / 8;
+            const int rowl = (is_key[i] ? g : g - TM / 8) * 8 + (lane >> 3);  // row of its operand tile
             const uint32_t col = static_cast<uint32_t>((lane & 7) ^ ((rowl >> 1) & 7)) * 16;  // logical column landing here
-            const int64_t kr = (r0 + rowl < R) ? rowl : (R - 1 - r0);                         // past the end: clamp (never stored)
-            const int64_t qr = (q0 + rowl < Q) ? rowl : (Q - 1 - q0);
-            koff[i] = static_cast<uint32_t>(kr * rowbytes) + col;
-            qoff[i] = static_cast<uint32_t>(qr * rowbytes) + col;
+            const int64_t lim = is_key[i] ? (R - r0) : (Q - q0);              // past the end: clamp (never stored)
+            const int64_t rr = (rowl < lim) ? rowl : (lim - 1);
+            off[i] = static_cast<uint32_t>(rr * rowbytes) + col;
         }
-        // scales: loader wave lw fetches the 64 queries of group lw % (T / 64) (with T = 128 two pairs of
-        // waves fetch the same data into their own regions, so that every loader wave has the same number
-        // of loads in flight)
-        const int sq = (lw % (T / 64)) * 64 + lane;
+        // scales: loader wave lw fetches the 64 queries of group lw % (TN / 64) (waves fetching the same group
+        // write their own regions, so that every loader wave has the same number of loads in flight)
+        const int sq = (lw % (TN / 64)) * 64 + lane;
         const uint32_t soff = static_cast<uint32_t>(((q0 + sq < Q) ? sq : (Q - 1 - q0)) * qscale_stride * 4);
         const int sstep = (qscale_stride == 1) ? 0 : 4;
         auto issue = [&](int h) {  // stage of half-chunk h (clamped to the last) into its ring slot
             const int hc = h < halves ? h : halves - 1;
-            unsigned char* slot = lds + (h & 3) * C::kStage + (4 * lw) * 1024;
+            unsigned char* slot = lds + (h & 3) * C::kStage + lw * 1024;
             const uint32_t so = static_cast<uint32_t>(hc) * 128;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) load16_to_lds(rk, koff[i], so, slot + i * 1024);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) load16_to_lds(rq, qoff[i], so, slot + C::kOperand + i * 1024);
+            for (int i = 0; i < 8; ++i)
+                load16_to_lds(is_key[i] ? rk : rq, off[i], so, slot + i * (C::kLoaders * 1024));
             if (h & 1) {  // with the second half of chunk c = h / 2: its scales
                 const int c = hc >> 1;
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(
@@ -840,7 +841,7 @@ __global__ __launch_bounds__(I8Cfg<T>::kBlock) void dot_mfma_i8_kernel(
     const int wr = wave & 1, wq = wave >> 1;  // half of the keys, group of 32 queries
     const int ln = lane & 15, lg = lane >> 4;
     const int krow_off = (wr * (WM * 16) + ln) * 128;
-    const int qrow_off = C::kOperand + (wq * (WN * 16) + ln) * 128;
+    const int qrow_off = C::kOperandK + (wq * (WN * 16) + ln) * 128;
     int pcol[2];
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) pcol[kk] = ((kk * 4 + lg) ^ (ln >> 1)) * 16;
@@ -1441,39 +1442,55 @@ static void launch_mfma_ws(const int8_t* A8, const float* qscale, int stride, co
                            R_total, out, chunk_ints);
 }
 
-template <int T>
+template <int TM, int TN>
 static void launch_mfma_i8_t(const int8_t* A8, const float* qscale, int stride, const int8_t* K8, const float* Bw,
                              int Sb, int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv,
                              int64_t R_total, float* out, int32_t* chunk_ints, const float* bias, hipStream_t st) {
-    using C = I8Cfg<T>;
-    const dim3 grid(static_cast<unsigned>((R + T - 1) / T), static_cast<unsigned>((Q + T - 1) / T));
+    using C = I8Cfg<TM, TN>;
+    const dim3 grid(static_cast<unsigned>((R + TM - 1) / TM), static_cast<unsigned>((Q + TN - 1) / TN));
     static bool configured = false;
     if (!configured) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dot_mfma_i8_kernel<T, true>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dot_mfma_i8_kernel<TM, TN, true>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, C::kLds);
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dot_mfma_i8_kernel<T, false>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dot_mfma_i8_kernel<TM, TN, false>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, C::kLds);
         configured = true;
     }
     if (chunk_ints)
-        hipLaunchKernelGGL((dot_mfma_i8_kernel<T, true>), grid, dim3(C::kBlock), C::kLds, st, A8, qscale, stride, K8,
-                           Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias);
+        hipLaunchKernelGGL((dot_mfma_i8_kernel<TM, TN, true>), grid, dim3(C::kBlock), C::kLds, st, A8, qscale, stride,
+                           K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias);
     else
-        hipLaunchKernelGGL((dot_mfma_i8_kernel<T, false>), grid, dim3(C::kBlock), C::kLds, st, A8, qscale, stride, K8,
-                           Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias);
+        hipLaunchKernelGGL((dot_mfma_i8_kernel<TM, TN, false>), grid, dim3(C::kBlock), C::kLds, st, A8, qscale, stride,
+                           K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias);
+}
+
+// Tile choice.  The 128 x 128 tile moves the fewest operand bytes per MAC and is the fastest whenever its grid
+// covers the 256 CUs (one workgroup per CU at a time) -- measured up to several rounds of 256.  A smaller grid
+// leaves CUs idle that smaller tiles would use: a workgroup's time per half-chunk is about 1 : 0.63 : 0.35 for
+// 128 x 128 : 128 x 64 : 64 x 64, so take the least (rounds of 256 workgroups x time), the larger tile on a tie.
+// g_i8_tile forces a tile (tuning and tests).
+static int choose_i8_tile(int64_t R, int64_t Q) {
+    if (g_i8_tile != 0) return g_i8_tile;
+    const int64_t n128 = ((R + 127) / 128) * ((Q + 127) / 128);
+    if (n128 > 256) return 128;
+    const int64_t n12864 = ((R + 127) / 128) * ((Q + 63) / 64);
+    const int64_t n64 = ((R + 63) / 64) * ((Q + 63) / 64);
+    const int64_t cost128 = 100;
+    const int64_t cost12864 = ((n12864 + 255) / 256) * 63;
+    const int64_t cost64 = ((n64 + 255) / 256) * 35;
+    if (cost128 <= cost12864 && cost128 <= cost64) return 128;
+    return cost12864 <= cost64 ? 12864 : 64;
 }
 
 static void launch_mfma_i8(const int8_t* A8, const float* qscale, int stride, const int8_t* K8, const float* Bw, int Sb,
                            int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv, int64_t R_total,
                            float* out, int32_t* chunk_ints, const float* bias, hipStream_t st) {
-    // 128 x 128 tiles unless they would leave most of the 256 CUs without a workgroup
-    const int64_t big = ((R + 127) / 128) * ((Q + 127) / 128);
-    if (big >= g_i8_small_tile_below)
-        launch_mfma_i8_t<128>(A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out,
-                              chunk_ints, bias, st);
-    else
-        launch_mfma_i8_t<64>(A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out,
-                             chunk_ints, bias, st);
+    const int tile = choose_i8_tile(R, Q);
+#define BSI_I8_ARGS A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias, st
+    if (tile == 128) launch_mfma_i8_t<128, 128>(BSI_I8_ARGS);
+    else if (tile == 12864) launch_mfma_i8_t<128, 64>(BSI_I8_ARGS);
+    else launch_mfma_i8_t<64, 64>(BSI_I8_ARGS);
+#undef BSI_I8_ARGS
 }
 
 template <int NT, int KT>
@@ -1544,9 +1561,9 @@ extern "C" int bsi_hip_planes_to_int8(const uint64_t* words, int64_t rows, int S
 
 extern "C" int bsi_hip_set_option(int option, int value) {
     switch (option) {
-        case BSI_OPT_I8_SMALL_TILE_BELOW:
-            BSI_REQUIRE(value >= 0, "threshold must be >= 0");
-            g_i8_small_tile_below = value;
+        case BSI_OPT_I8_TILE:
+            BSI_REQUIRE(value == 0 || value == 128 || value == 12864 || value == 64, "tile must be 0, 128, 12864 or 64");
+            g_i8_tile = value;
             return BSI_OK;
         default:
             return fail(BSI_ERR_INVALID, "unknown option %d", option);

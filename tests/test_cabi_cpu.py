@@ -184,7 +184,8 @@ def test_key_operand_selection_and_new_flags(monkeypatch):
 def test_set_option_validates_on_host():
     from bsipytorch_amd import _lib
 
-    assert _lib.lib.bsi_hip_set_option(_lib.OPT_I8_SMALL_TILE_BELOW, 100) == 0
-    assert _lib.lib.bsi_hip_set_option(_lib.OPT_I8_SMALL_TILE_BELOW, -1) == 1
+    assert _lib.lib.bsi_hip_set_option(_lib.OPT_I8_TILE, 12864) == 0
+    assert _lib.lib.bsi_hip_set_option(_lib.OPT_I8_TILE, 96) == 1
+    assert _lib.lib.bsi_hip_set_option(_lib.OPT_I8_TILE, 0) == 0
     assert _lib.lib.bsi_hip_set_option(999, 1) == 1
     assert b"unknown option" in _lib.lib.bsi_hip_last_error()

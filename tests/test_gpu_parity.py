@@ -306,6 +306,10 @@ def _oracle_case(oracle, Q, R, d, seed, qkind="randn", ksigma=0.02, bits_q=7, bi
     return x, k, qb, kb, ints, out
 
 
+# forms of the `tiled` argument that select the cached int8 key image, and the tile each one forces (0: automatic)
+_I8_TILES = {"int8": 0, "int8-128": 128, "int8-12864": 12864, "int8-64": 64}
+
+
 def _run_dot(hip, qb, kb, Q, R, W, Sa, Sb, core, tiled, with_ints8, want_ints=True, R_total=None):
     L = hip.lib
     chunks = (W + 3) // 4
@@ -314,9 +318,8 @@ def _run_dot(hip, qb, kb, Q, R, W, Sa, Sb, core, tiled, with_ints8, want_ints=Tr
     stride = chunks if qb["chunk_scale"] else 1
     B = dev(kb["words"])
     layout = 0
-    if tiled in ("int8", "int8-128", "int8-64"):   # the cached int8 image of the key integers; tile size forced or automatic
-        hip.check(L.bsi_hip_set_option(hip.OPT_I8_SMALL_TILE_BELOW, {"int8": 100, "int8-128": 0, "int8-64": 1 << 30}[tiled]),
-                  "set_option")
+    if tiled in _I8_TILES:   # the cached int8 image of the key integers; tile forced or automatic
+        hip.check(L.bsi_hip_set_option(hip.OPT_I8_TILE, _I8_TILES[tiled]), "set_option")
         Bi = torch.full((R, chunks * 256), 77, dtype=torch.int8, device="cuda")
         hip.check(L.bsi_hip_planes_to_int8(B.data_ptr(), R, Sb, W, Bi.data_ptr(), st()), "key image")
         B, layout = Bi, 2
@@ -339,7 +342,7 @@ def _run_dot(hip, qb, kb, Q, R, W, Sa, Sb, core, tiled, with_ints8, want_ints=Tr
                             out.data_ptr(), ints.data_ptr() if ints is not None else None, core, ws.data_ptr(),
                             ws_bytes, st()), "dot")
     torch.cuda.synchronize()
-    hip.check(L.bsi_hip_set_option(hip.OPT_I8_SMALL_TILE_BELOW, 100), "set_option")
+    hip.check(L.bsi_hip_set_option(hip.OPT_I8_TILE, 0), "set_option")
     return (ints.cpu().numpy() if ints is not None else None), out.cpu().numpy()
 
 
@@ -360,7 +363,8 @@ DOT_SHAPES = [
 
 @pytest.mark.parametrize("Q,R,d,kind", DOT_SHAPES)
 @pytest.mark.parametrize("core,tiled,ints8", [(1, False, False), (1, True, False), (2, False, True), (2, True, False),
-                                              (0, True, True), (2, "int8-128", True), (0, "int8-64", False)])
+                                              (0, True, True), (2, "int8-128", True), (0, "int8-64", False),
+                                              (2, "int8-12864", True), (0, "int8-12864", False)])
 def test_dot_bit_exact(hip, oracle, Q, R, d, kind, core, tiled, ints8):
     x, k, qb, kb, want_ints, want_out = _oracle_case(oracle, Q, R, d, seed=Q + R + d, qkind=kind)
     W = (d + 63) // 64
@@ -430,7 +434,7 @@ def test_hybrid_query_dot_decodes_inline(ops, oracle, monkeypatch):
 
 
 @pytest.mark.parametrize("Sa,Sb", [(8, 8), (5, 4), (2, 2), (7, 5), (3, 7)])
-@pytest.mark.parametrize("core,tiled", [(1, False), (2, True), (2, "int8-128"), (2, "int8-64")])
+@pytest.mark.parametrize("core,tiled", [(1, False), (2, True), (2, "int8-128"), (2, "int8-12864"), (2, "int8-64")])
 def test_dot_other_bit_widths(hip, oracle, Sa, Sb, core, tiled):
     Q, R, d = 19, 35, 1024
     x, k, qb, kb, want_ints, want_out = _oracle_case(oracle, Q, R, d, seed=Sa * 10 + Sb, ksigma=0.05, bits_q=Sa, bits_k=Sb)
@@ -498,7 +502,7 @@ def test_dot_row_stride_and_untouched_columns(hip, oracle):
 
 def test_dot_row_stride_int8_image_and_few_rows(hip, oracle):
     x, k, qb, kb, want_ints, want_out = _oracle_case(oracle, 70, 150, 1024, seed=8)
-    for tiled in ("int8-128", "int8-64"):
+    for tiled in ("int8-128", "int8-12864", "int8-64"):
         _, out = _run_dot(hip, qb, kb, 70, 150, 16, 7, 6, 2, tiled=tiled, with_ints8=True, want_ints=False, R_total=163)
         np.testing.assert_array_equal(out[:, :150], want_out)
         assert np.isnan(out[:, 150:]).all()
@@ -508,7 +512,7 @@ def test_dot_row_stride_int8_image_and_few_rows(hip, oracle):
     assert np.isnan(out[:, 150:]).all()
 
 
-@pytest.mark.parametrize("Q,tiled", [(70, "int8-128"), (70, "int8-64"), (9, True), (70, True), (70, False)])
+@pytest.mark.parametrize("Q,tiled", [(70, "int8-128"), (70, "int8-12864"), (70, "int8-64"), (9, True), (70, True), (70, False)])
 def test_dot_bias_entry_point(hip, oracle, Q, tiled):
     """bsi_hip_dot_bias == bsi_hip_dot followed by a float addition of the bias row, bit for bit, whether the
     kernel adds it in its epilogue (int8 image, few rows) or the library appends an addition kernel."""
@@ -520,8 +524,8 @@ def test_dot_bias_entry_point(hip, oracle, Q, tiled):
     A, scales, Bc, Bw = dev(qb["words"]), dev(qb["scales"]), dev(kb["words"]), dev(kb["slice_weights"])
     a8 = torch.zeros((Q, 4 * 256), dtype=torch.int8, device="cuda")
     hip.check(L.bsi_hip_planes_to_int8(A.data_ptr(), Q, 7, W, a8.data_ptr(), st()), "p2i8")
-    if tiled in ("int8-128", "int8-64"):
-        hip.check(L.bsi_hip_set_option(hip.OPT_I8_SMALL_TILE_BELOW, 0 if tiled == "int8-128" else 1 << 30), "opt")
+    if tiled in _I8_TILES:
+        hip.check(L.bsi_hip_set_option(hip.OPT_I8_TILE, _I8_TILES[tiled]), "opt")
         B = torch.zeros((R, 4 * 256), dtype=torch.int8, device="cuda")
         hip.check(L.bsi_hip_planes_to_int8(Bc.data_ptr(), R, 6, W, B.data_ptr(), st()), "image")
         layout = 2
@@ -537,7 +541,7 @@ def test_dot_bias_entry_point(hip, oracle, Q, tiled):
                                  Bw.data_ptr(), 6, R, Q, float(np.float32(1e-4)), R + 5, bd.data_ptr(), out.data_ptr(),
                                  2, None, 0, st()), "dot_bias")
     torch.cuda.synchronize()
-    hip.check(L.bsi_hip_set_option(hip.OPT_I8_SMALL_TILE_BELOW, 100), "opt")
+    hip.check(L.bsi_hip_set_option(hip.OPT_I8_TILE, 0), "opt")
     got = out.cpu().numpy()
     np.testing.assert_array_equal(got[:, :R], want_out + bias[None, :])
     assert np.isnan(got[:, R:]).all()
