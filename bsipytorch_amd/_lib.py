@@ -37,6 +37,7 @@ PROTOTYPES = {
     "bsi_hip_quantize_shift_pack_row_batch": [_vp, _i, _i64, _i64, _i, _i, _d, _i, _vp, _vp, _vp],
     "bsi_hip_quantize_shift_pack_chunk_batch": [_vp, _i, _i64, _i64, _i, _i, _i, _d, _i, _vp, _vp, _vp],
     "bsi_hip_pack_bits_batch": [_vp, _i64, _i64, _i, _i, _vp, _vp],
+    "bsi_hip_decimal_stats": [_vp, _i64, _i64, _vp, _vp, _vp],
     "bsi_hip_build_fixed": [_vp, _i, _i64, _i64, _i, _i, _i, _f, _vp, _vp, _vp, _vp, _vp],
     "bsi_hip_slice_popcount_sum": [_vp, _i, _i, _vp, _vp],
     "bsi_hip_compress_flags_from_density": [_vp, _i, _i, _d, _vp, _vp],
@@ -51,6 +52,7 @@ PROTOTYPES = {
     "bsi_hip_dot": [_vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _i, _i64, _i64, _f, _i64, _vp, _vp, _i, _vp, _sz, _vp],
     "bsi_hip_dot_bias": [_vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _i, _i64, _i64, _f, _i64, _vp, _vp, _i, _vp, _sz, _vp],
     "bsi_hip_dot_ewah_query": [_vp, _vp, _vp, _i, _i, _vp, _i, _vp, _vp, _i, _i64, _f, _vp, _vp, _vp],
+    "bsi_hip_dot_weighted": [_vp, _vp, _i, _i, _vp, _i, _vp, _i, _i64, _i64, _vp, _f, _i64, _vp, _vp],
     "bsi_hip_dot_timed": [_vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _i, _i64, _i64, _f, _i64, _vp, _i, _vp, _sz, _i,
                           ctypes.POINTER(_f), _vp],
     "bsi_hip_probe_valu_popcount": [ctypes.POINTER(_d), _vp],

@@ -31,6 +31,8 @@ def run(Q, R, D, decimal_places=2, compress_threshold=0.5, warmup=10, iters=50, 
     if report_stats:
         print("[Keys]", bsi_ops.bsi_keys_cuda_stats(kcap))
     chunks = (W + 3) // 4
+    if not (qcap.fixed and kcap.fixed):
+        return _run_weighted(qcap, kcap, Q, R, D, W, key_bytes, warmup, iters)
     if qcap.chunk_scales is not None:
         scales, stride = qcap.chunk_scales, chunks
     else:
@@ -54,6 +56,25 @@ def run(Q, R, D, decimal_places=2, compress_threshold=0.5, warmup=10, iters=50, 
     return {"Q": Q, "R": R, "D": D, "core": core, "layout": {0: "canonical", 1: "tiled16", 2: "int8 image"}[klayout],
             "avg_dot_us": t * 1e6, "dot_q_us": t * 1e6 / Q, "dot_s_ns": t * 1e9 / (Q * R),
             "effective_bitop_TOPS": bit_ops / t / 1e12, "int8_TOPS": 2.0 * Q * R * D / t / 1e12,
+            "algorithmic_GBps": alg_bytes / t / 1e9, "key_plane_GBps": key_bytes / t / 1e9, "iters": iters}
+
+
+def _run_weighted(qcap, kcap, Q, R, D, W, key_bytes, warmup, iters):
+    """Decimal-mode operands (BSI_FIXED_BITS*=0): the weighted-slice dot, timed by device events over `iters` calls."""
+    for _ in range(max(warmup, 1)):
+        bsi_ops.batch_dot_product_multiquery_cuda_batch_caps(qcap, kcap)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        bsi_ops.batch_dot_product_multiquery_cuda_batch_caps(qcap, kcap)
+    e1.record()
+    e1.synchronize()
+    t = e0.elapsed_time(e1) * 1e-3 / iters
+    bit_ops = 2.0 * qcap.Sa * kcap.Sb * Q * R * D
+    alg_bytes = Q * qcap.Sa * W * 8 + R * kcap.Sb * W * 8 + (Q * qcap.Sa + R * kcap.Sb) * 4 + Q * R * 4
+    return {"Q": Q, "R": R, "D": D, "core": "weighted", "layout": "canonical" if kcap.layout == 0 else "tiled16",
+            "Sa": qcap.Sa, "Sb": kcap.Sb, "avg_dot_us": t * 1e6, "dot_q_us": t * 1e6 / Q, "dot_s_ns": t * 1e9 / (Q * R),
+            "effective_bitop_TOPS": bit_ops / t / 1e12, "popcount_word_ops_per_s": qcap.Sa * kcap.Sb * Q * R * W / t,
             "algorithmic_GBps": alg_bytes / t / 1e9, "key_plane_GBps": key_bytes / t / 1e9, "iters": iters}
 
 

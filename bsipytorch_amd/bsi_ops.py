@@ -58,7 +58,7 @@ def _flags() -> dict:
     base = _env_int("BSI_FIXED_BITS", None)
     q = _env_int("BSI_FIXED_BITS_QUERIES", None)
     k = _env_int("BSI_FIXED_BITS_KEYS", None)
-    # default (nothing set): fixed76 chunk-scale
+    # default (nothing set): fixed76 chunk-scale; an explicit 0 selects the decimal builder
     bits_q = _clamp_bits(q if q is not None else (base if base is not None else 7))
     bits_k = _clamp_bits(k if k is not None else (base if base is not None else 6))
     clip = 0.0
@@ -147,7 +147,8 @@ class PrebuiltBSIKeysCUDA(_Capsule):
         self.layout = _lib.LAYOUT_CANONICAL
         self.ints8: Optional[torch.Tensor] = None  # cached int8 image [R, chunks*256] of the same integers, or None
         self.slice_weights: torch.Tensor = None  # [R, Sb] float32
-        self.shifts: torch.Tensor = None         # [R] int32
+        self.shifts: torch.Tensor = None         # [R] int32 (fixed-bit keys only)
+        self.fixed = True                        # False: decimal-mode keys (slice count from the data, canonical planes)
         self.Sb = 0
         self.W = 0
         self.d = 0
@@ -167,6 +168,7 @@ class PrebuiltBSIQueryBatchCUDA(_Capsule):
         self.chunk_scales: Optional[torch.Tensor] = None  # [Q, chunks] float32 or None
         self.row_scales: Optional[torch.Tensor] = None    # [Q] float32 when there are no chunk scales
         self.ints8: Optional[torch.Tensor] = None         # [Q, chunks*256] int8 (MFMA operand) or None
+        self.fixed = True                                 # False: decimal-mode batch (no scales; weighted-slice dot)
         self.Sa = 0
         self.W = 0
         self.decimals = 0
@@ -185,6 +187,7 @@ class PrebuiltBSIQueryCUDA(_Capsule):
         self.chunk_scales: Optional[torch.Tensor] = None  # [chunks]
         self.row_scale: Optional[torch.Tensor] = None     # [] when no chunk scales
         self.ints8: Optional[torch.Tensor] = None         # [chunks*256]
+        self.fixed = True                                 # False: decimal-mode row (no scale)
         self.S = 0
         self.W = 0
         self.rows = 0
@@ -278,9 +281,32 @@ def _build_fixed(x2d: torch.Tensor, decimal_places: int, fixed_bits: int, chunk_
     return words, shifts, scales, ints8
 
 
-def _require_fixed(bits: int, what: str) -> None:
-    _check(bits > 0, f"{what}: BSI_FIXED_BITS*=0 selects the decimal (data-dependent slice count) builder, "
-                     "which this build does not implement; unset it to use the fixed-bit path")
+def _build_decimal(x2d: torch.Tensor, decimal_places: int):
+    """Decimal mode (``BSI_FIXED_BITS*=0``), bsi_vector_cuda.cpp:565-577 + :1088-1166: round ``x * 10^dec`` half
+    away from zero, one slice count for the batch from its largest magnitude (:746-754), low ``S`` bits of the
+    two's-complement values packed, and per row the two's-complement weights iff the row holds a negative value.
+    -> (words [Q,S,W] int64, slice_weights [Q,S] float32, S, row_negative [Q] int32).
+    Reads one scalar back from the device to size the planes, as the reference does (``.item()``, :1092-1096)."""
+    dev = x2d.device
+    Q, d = x2d.shape
+    W = (d + 63) // 64 if d > 0 else 1
+    st = _stream()
+    ints = torch.empty((Q, d), dtype=torch.int64, device=dev)
+    if Q > 0 and d > 0:
+        check(lib.bsi_hip_quantize_round_to_int64(x2d.data_ptr(), _dtype_code(x2d), Q * d, 10.0 ** int(decimal_places),
+                                                  ints.data_ptr(), st), "bsi_hip_quantize_round_to_int64")
+    max_abs = torch.empty((1,), dtype=torch.int64, device=dev)
+    negative = torch.zeros((Q,), dtype=torch.int32, device=dev)
+    check(lib.bsi_hip_decimal_stats(ints.data_ptr() if Q > 0 and d > 0 else None, Q, d, max_abs.data_ptr(),
+                                    negative.data_ptr() if Q > 0 else None, st), "bsi_hip_decimal_stats")
+    m = int(max_abs.item()) & 0xFFFFFFFFFFFFFFFF  # |INT64_MIN| comes back as an unsigned 2^63
+    S = 2 if m == 0 else min(64, m.bit_length() + 2)
+    words = torch.zeros((Q, S, W), dtype=torch.int64, device=dev)
+    if Q > 0 and d > 0:
+        check(lib.bsi_hip_pack_bits_batch(ints.data_ptr(), Q, d, S, W, words.data_ptr(), st), "bsi_hip_pack_bits_batch")
+    w_twos, w_unsigned = _slice_weights(S, 0, True, dev), _slice_weights(S, 0, False, dev)
+    weights = torch.where(negative.bool().unsqueeze(1), w_twos.unsqueeze(0), w_unsigned.unsqueeze(0)).contiguous()
+    return words, weights, S, negative
 
 
 _expanded_cache: dict = {}
@@ -302,7 +328,6 @@ def _expanded_slice_weights(base: torch.Tensor, Q: int, bits: int, dev) -> torch
 def _build_query_batch(q2d: torch.Tensor, decimal_places: int) -> PrebuiltBSIQueryBatchCUDA:
     """bsi_vector_cuda.cpp:971-1064 (queries): chunk scales iff the flag is on and W64 % 4 == 0."""
     f = _flags()
-    _require_fixed(f["bits_q"], "build_bsi_queries")
     dev = _device()
     x = _as_build_input(q2d, dev)
     Q, d = x.shape
@@ -312,6 +337,22 @@ def _build_query_batch(q2d: torch.Tensor, decimal_places: int) -> PrebuiltBSIQue
     if prof:
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
+    if f["bits_q"] == 0:  # decimal mode: the slice count follows the data; no scales
+        words, weights, S, _neg = _build_decimal(x, decimal_places)
+        if prof:
+            e1.record()
+            e1.synchronize()
+            ns = int(e0.elapsed_time(e1) * 1.0e6)
+            _last_build_profile[:] = [0, ns, ns]
+        else:
+            _last_build_profile[:] = [0, 0, 0]
+        h = PrebuiltBSIQueryBatchCUDA()
+        h.words, h.slice_weights, h.fixed = words, weights, False
+        h.Sa, h.W, h.decimals, h.Q = S, W, int(decimal_places), Q
+        h.mem_bytes = words.numel() * 8 + weights.numel() * 4
+        if f["debug"]:
+            print(f"[BSI_HIP] build_bsi_queries_cuda_batch_data: Q={Q} slices={S} words_per_slice={W}")
+        return h
     words, _shifts, scales, ints8 = _build_fixed(x, decimal_places, f["bits_q"], chunk_scale, want_ints8=True)
     if prof:
         e1.record()
@@ -358,9 +399,10 @@ def build_bsi_queries_cuda_batch(q2d: torch.Tensor, decimal_places: int, compres
         h.S, h.W = b.Sa, b.W
         h.dev_words = b.words[qi]
         h.slice_weights = b.slice_weights[qi]
+        h.fixed = b.fixed
         if b.chunk_scales is not None and b.chunk_scales.numel() > 0:
             h.chunk_scales = b.chunk_scales[qi]
-        else:
+        elif b.row_scales is not None:
             h.row_scale = b.row_scales[qi]
         h.ints8 = b.ints8[qi] if b.ints8 is not None else None
         h.mem_bytes = h.dev_words.numel() * 8
@@ -374,9 +416,16 @@ def build_bsi_queries_cuda_batch(q2d: torch.Tensor, decimal_places: int, compres
 def _build_query_1d(q: torch.Tensor, decimal_places: int) -> PrebuiltBSIQueryCUDA:
     """bsi_vector_cuda.cpp:778-852 with fixed bits: one scale for the whole vector."""
     f = _flags()
-    _require_fixed(f["bits_q"], "build_bsi_query_cuda")
     dev = _device()
     x = _as_build_input(q, dev).view(1, -1)
+    if f["bits_q"] == 0:  # decimal mode: no scale; two's complement iff a negative value is present (:843)
+        words, weights, S, neg = _build_decimal(x, decimal_places)
+        h = PrebuiltBSIQueryCUDA()
+        h.S, h.W, h.dev_words, h.rows, h.decimals, h.fixed = S, words.shape[2], words[0], x.shape[1], int(decimal_places), False
+        h.twos_complement = bool(neg[0].item()) if x.shape[1] > 0 else False
+        h.slice_weights = weights[0]
+        h.mem_bytes = h.dev_words.numel() * 8
+        return h
     words, _shifts, scales, ints8 = _build_fixed(x, decimal_places, f["bits_q"], False, want_ints8=True)
     h = PrebuiltBSIQueryCUDA()
     h.S = f["bits_q"]
@@ -449,10 +498,22 @@ def build_bsi_keys_cuda(K: torch.Tensor, decimal_places: int, compress_threshold
     Returns (handle, total_bytes_of_words, num_keys, d, W)."""
     _check(K.dim() == 2, "K must be 2D [num_keys, d]")
     f = _flags()
-    _require_fixed(f["bits_k"], "build_bsi_keys_cuda")
     dev = _device()
     x = _as_build_input(K, dev)
     R, d = x.shape
+    if f["bits_k"] == 0:
+        # Decimal mode.  The reference builds these keys row by row on the host with the bsiCPP library
+        # (bsi_cuda.cpp:912-1000), which is not part of its tree; here the device builder the reference
+        # uses for decimal queries is applied to the key matrix (one slice count for all rows, so one group
+        # in identity order).  The integers each row stands for are the same rounded values either way.
+        words, weights, S, _neg = _build_decimal(x, int(decimal_places))
+        h = PrebuiltBSIKeysCUDA()
+        h.num_keys, h.d, h.W, h.Sb, h.fixed = int(R), int(d), words.shape[2], S, False
+        h.decimals, h.threshold = int(decimal_places), float(compress_threshold)
+        h.words, h.layout, h.slice_weights = words, _lib.LAYOUT_CANONICAL, weights
+        if f["debug"]:
+            print(f"[BSI_HIP] build_bsi_keys_cuda (decimal): R={R} slices={S} words_per_slice={h.W}")
+        return h, int(words.numel() * 8), int(R), int(d), int(h.W)
     words, shifts, scales, _ = _build_fixed(x, int(decimal_places), f["bits_k"], False, want_ints8=False)
     h = PrebuiltBSIKeysCUDA()
     h.num_keys, h.d = int(R), int(d)
@@ -557,6 +618,33 @@ def _dot(words, ints8, scales, scale_stride, Sa, W, keys: PrebuiltBSIKeysCUDA, Q
     return out, ns
 
 
+def _dot_weighted(words, slice_weights, Sa, W, keys: PrebuiltBSIKeysCUDA, Q, decimals_q, bias=None):
+    """The weighted-slice dot (bsi_hip_dot_weighted): any operand pair that is not fixed-bit on both sides."""
+    f = _flags()
+    R = keys.num_keys
+    out = torch.empty((Q, R), dtype=torch.float32, device=words.device)
+    Aw = slice_weights if slice_weights.is_contiguous() else slice_weights.contiguous()
+    prof = f["profile"]
+    if prof:
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+    check(lib.bsi_hip_dot_weighted(words.data_ptr(), Aw.data_ptr(), int(Sa), int(W), keys.words.data_ptr(), keys.layout,
+                                   keys.slice_weights.data_ptr(), keys.Sb, R, Q, None,
+                                   _scale_inv(decimals_q, keys.decimals), R, out.data_ptr(), _stream()),
+          "bsi_hip_dot_weighted")
+    if bias is not None:
+        out += bias
+    ns = 0
+    if prof:
+        e1.record()
+        e1.synchronize()
+        ns = int(e0.elapsed_time(e1) * 1.0e6)
+    if f["dot_debug"] and not _DOT_DEBUG_PRINTED[0]:
+        _DOT_DEBUG_PRINTED[0] = True
+        print(f"[BSI_DOT] core=weighted Sa={Sa} Sb={keys.Sb} Q={Q} R={R} W64={W} layout={keys.layout}", file=sys.stderr)
+    return out, ns
+
+
 def _dot_result(out, ns, Q, R):
     per_q = float(ns) / float(Q) if Q > 0 else 0.0
     per_s = float(ns) / (float(Q) * float(R)) if (Q > 0 and R > 0) else 0.0
@@ -580,7 +668,8 @@ def batch_dot_product_multiquery_cuda_batch_caps(query_batch_cap, keyset_cuda_ca
     _check(tuple(qb.slice_weights.shape) == (Q, Sa), f"slice_weights shape mismatch: expected [{Q}, {Sa}]")
     R = keys.num_keys
     _check(R > 0, "Empty keys")
-    if qb.chunk_scales is not None and qb.chunk_scales.numel() > 0:
+    have_chunk_scales = qb.chunk_scales is not None and qb.chunk_scales.numel() > 0
+    if have_chunk_scales:
         _check(qb.chunk_scales.is_cuda, "chunk_scales must be a CUDA tensor")
         _check(qb.chunk_scales.dim() == 2, "Expected [Q, chunks] chunk scales")
         _check(qb.chunk_scales.shape[0] == Q, "chunk_scales Q mismatch")
@@ -588,7 +677,7 @@ def batch_dot_product_multiquery_cuda_batch_caps(query_batch_cap, keyset_cuda_ca
         _check(qb.chunk_scales.shape[1] == keys.W // 4,
                f"Chunk scale stride mismatch: got {qb.chunk_scales.shape[1]} expected {keys.W // 4}")
         scales, stride = qb.chunk_scales, int(qb.chunk_scales.shape[1])
-    else:
+    elif qb.fixed:
         _check(qb.row_scales is not None, "Query batch has neither chunk scales nor row scales")
         scales, stride = qb.row_scales, 1
     _check(qb.decimals == keys.decimals,
@@ -596,7 +685,12 @@ def batch_dot_product_multiquery_cuda_batch_caps(query_batch_cap, keyset_cuda_ca
     if bias is not None:
         _check(bias.is_cuda and bias.dtype == torch.float32 and bias.dim() == 1 and bias.numel() == R and bias.is_contiguous(),
                "bias must be a contiguous float32 CUDA tensor of [R]")
-    out, ns = _dot(qb.words, qb.ints8, scales, stride, int(Sa), int(W), keys, int(Q), qb.decimals, bias=bias)
+    if qb.fixed and keys.fixed:
+        out, ns = _dot(qb.words, qb.ints8, scales, stride, int(Sa), int(W), keys, int(Q), qb.decimals, bias=bias)
+    else:
+        # a decimal-mode operand on either side: its slice weights carry everything, per-chunk scales cannot apply
+        _check(not have_chunk_scales, "chunk-scaled queries need fixed-bit keys (BSI_FIXED_BITS_KEYS > 0)")
+        out, ns = _dot_weighted(qb.words, qb.slice_weights, int(Sa), int(W), keys, int(Q), qb.decimals, bias=bias)
     return _dot_result(out, ns, Q, R)
 
 
@@ -612,7 +706,7 @@ def batch_dot_product_multiquery_cuda_caps(query_caps_list, keyset_cuda_cap):
         q = _capsule(cap, PrebuiltBSIQueryCUDA, f"Invalid BSI query capsule at index {qi}")
         _check(q.W == keys.W, "Word count mismatch between query and keys")
         _check(q.decimals == rows[0].decimals if rows else True, "Decimal mismatch across queries not supported")
-        _check(q.S == rows[0].S if rows else True, "Mixed slice counts across queries are not supported in fixed-bit mode")
+        _check(q.S == rows[0].S if rows else True, "Mixed slice counts across queries are not supported")
         rows.append(q)
     have_scales = rows[0].chunk_scales is not None and rows[0].chunk_scales.numel() > 0
     for q in rows:
@@ -620,6 +714,14 @@ def batch_dot_product_multiquery_cuda_caps(query_caps_list, keyset_cuda_cap):
                "Mixed chunk-scale and non-chunk-scale queries in the same group")
     f = _flags()
     q0 = rows[0]
+    if not (keys.fixed and all(q.fixed for q in rows)):
+        _check(all(q.fixed == q0.fixed for q in rows), "Mixed fixed-bit and decimal queries in the same group")
+        _check(not have_scales, "chunk-scaled queries need fixed-bit keys (BSI_FIXED_BITS_KEYS > 0)")
+        _check(q0.decimals == keys.decimals, f"Decimal mismatch between queries and keys: q={q0.decimals} k={keys.decimals}")
+        words = torch.stack([q.dev_words for q in rows]).contiguous()
+        weights = torch.stack([q.slice_weights for q in rows]).contiguous()
+        out, ns = _dot_weighted(words, weights, q0.S, keys.W, keys, Q, q0.decimals)
+        return _dot_result(out, ns, Q, R)
     if (Q == 1 and getattr(q0, "comp_words", None) is not None and q0.comp_words.numel() > 0 and f["ewah_inline"]
             and keys.layout == _lib.LAYOUT_TILED16 and keys.Sb == 6 and 2 <= q0.S <= 8
             and f["core"] != _lib.CORE_VALU and q0.S * ((keys.W + 3) // 4) * 32 <= 96 * 1024):
@@ -692,6 +794,7 @@ def debug_chunk_ints(query_batch_cap, keyset_cuda_cap, core: str = "auto"):
     No counterpart in the reference (its accumulators never leave the kernel)."""
     keys = _capsule(keyset_cuda_cap, PrebuiltBSIKeysCUDA, "Invalid CUDA keys capsule")
     qb = _capsule(query_batch_cap, PrebuiltBSIQueryBatchCUDA, "Invalid CUDA query-batch capsule")
+    _check(qb.fixed and keys.fixed, "debug_chunk_ints: per-chunk accumulators exist for fixed-bit operands only")
     Q, Sa, W = qb.words.shape
     chunks = (W + 3) // 4
     ints = torch.zeros((Q, keys.num_keys, chunks), dtype=torch.int32, device=qb.words.device)

@@ -650,6 +650,66 @@ extern "C" int bsi_hip_pack_bits_batch(const int64_t* ints, int64_t Q, int64_t d
     return BSI_OK;
 }
 
+// ---- decimal mode (no fixed bits): the slice count follows the data ----
+
+// One workgroup per row: largest |value| of the whole batch (atomic max into *max_abs, cleared by the
+// launcher) and, per row, whether any value is negative.
+__global__ __launch_bounds__(kBlock) void decimal_stats_kernel(const long long* __restrict__ ints, int64_t d,
+                                                               unsigned long long* __restrict__ max_abs,
+                                                               int* __restrict__ row_negative) {
+    __shared__ unsigned long long smax[kBlock / BSI_WAVE];
+    __shared__ int sneg[kBlock / BSI_WAVE];
+    const int64_t q = blockIdx.x;
+    const long long* row = ints + q * d;
+    unsigned long long m = 0;
+    int neg = 0;
+    for (int64_t e = threadIdx.x; e < d; e += kBlock) {
+        const long long v = row[e];
+        const unsigned long long a = v < 0 ? 0ULL - static_cast<unsigned long long>(v) : static_cast<unsigned long long>(v);
+        m = a > m ? a : m;
+        neg |= v < 0;
+    }
+#pragma unroll
+    for (int off = BSI_WAVE / 2; off > 0; off >>= 1) {
+        const unsigned long long o = __shfl_xor(m, off, BSI_WAVE);
+        m = o > m ? o : m;
+        neg |= __shfl_xor(neg, off, BSI_WAVE);
+    }
+    const int wave = threadIdx.x / BSI_WAVE;
+    if ((threadIdx.x & (BSI_WAVE - 1)) == 0) {
+        smax[wave] = m;
+        sneg[wave] = neg;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < kBlock / BSI_WAVE; ++w) {
+            m = smax[w] > m ? smax[w] : m;
+            neg |= sneg[w];
+        }
+        row_negative[q] = neg;
+        if (m != 0) atomicMax(max_abs, m);
+    }
+}
+
+__global__ void clear_u64_kernel(unsigned long long* p) { *p = 0ULL; }
+
+extern "C" int bsi_hip_decimal_stats(const int64_t* ints, int64_t Q, int64_t d, uint64_t* max_abs,
+                                     int32_t* row_negative, void* stream) {
+    BSI_REQUIRE(Q >= 0 && d >= 0, "negative size");
+    BSI_REQUIRE(max_abs != nullptr, "null pointer");
+    BSI_REQUIRE(Q <= 0x7fffffffLL, "too many rows for one launch");
+    hipLaunchKernelGGL(clear_u64_kernel, dim3(1), dim3(1), 0, as_stream(stream),
+                       reinterpret_cast<unsigned long long*>(max_abs));
+    BSI_LAUNCH_CHECK("clear_u64_kernel");
+    if (Q == 0) return BSI_OK;
+    BSI_REQUIRE(row_negative != nullptr && (ints != nullptr || d == 0), "null pointer");
+    hipLaunchKernelGGL(decimal_stats_kernel, dim3(static_cast<unsigned>(Q)), dim3(kBlock), 0, as_stream(stream),
+                       reinterpret_cast<const long long*>(ints), d, reinterpret_cast<unsigned long long*>(max_abs),
+                       row_negative);
+    BSI_LAUNCH_CHECK("decimal_stats_kernel");
+    return BSI_OK;
+}
+
 extern "C" int bsi_hip_build_fixed(const void* x, int dtype, int64_t Q, int64_t d, int decimal_places, int fixed_bits,
                                    int chunk_scale, float clip_k, uint64_t* words, int32_t* shifts, float* scales,
                                    int8_t* ints8, void* stream) {

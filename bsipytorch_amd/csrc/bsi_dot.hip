@@ -1374,6 +1374,95 @@ __global__ void dot_valu_generic_kernel(const unsigned long long* __restrict__ A
     out[static_cast<size_t>(q) * R_total + r] = (acc * Bw[r * Sb]) * scale_inv;
 }
 
+// Weighted-slice dot for operands whose slice weights are arbitrary floats (the decimal builder's
+// data-dependent slice counts, or fixed-bit operands without chunk scales):
+//   out[q, idx[r]] = float(sum over i, j, w of popcount(A[q,i,w] & B[r,j,w]) * double(Aw[q,i] * Bw[r,j])) * scale_inv
+// The coefficient is the float32 product; the sum runs in float64, exact while it stays below 2^53 (every
+// term is an integer times a power of two for the builders' weights), so the result does not depend on
+// the order of the terms.  Workgroup = 32 queries x 32 keys, 2 x 2 outputs per thread, WB words of every
+// slice staged through LDS per step.  Any Sa, Sb in [1, 64].
+template <int WB, bool kTiled>
+__global__ __launch_bounds__(256) void dot_weighted_kernel(
+    const unsigned long long* __restrict__ A, const float* __restrict__ Aw, int Sa, int W64,
+    const unsigned long long* __restrict__ B, const float* __restrict__ Bw, int Sb, int chunks, int64_t R, int64_t Q,
+    const long long* __restrict__ key_indices, float scale_inv, int64_t R_total, float* __restrict__ out) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char wlds[];
+    const int strideA = Sa * WB + 1, strideB = Sb * WB + 1;  // in 64-bit words; odd, so rows start in different banks
+    unsigned long long* As = reinterpret_cast<unsigned long long*>(wlds);  // [32][strideA]
+    unsigned long long* Bs = As + 32 * strideA;                            // [32][strideB]
+    float* Aws = reinterpret_cast<float*>(Bs + 32 * strideB);              // [32][Sa]
+    float* Bws = Aws + 32 * Sa;                                            // [32][Sb]
+    const int tid = threadIdx.x;
+    const int tq = tid >> 4, tr = tid & 15;
+    const int64_t q0 = static_cast<int64_t>(blockIdx.y) * 32, r0 = static_cast<int64_t>(blockIdx.x) * 32;
+    for (int idx = tid; idx < 32 * Sa; idx += 256) {
+        const int64_t q = q0 + idx / Sa;
+        Aws[idx] = q < Q ? Aw[q * Sa + idx % Sa] : 0.0f;
+    }
+    for (int idx = tid; idx < 32 * Sb; idx += 256) {
+        const int64_t r = r0 + idx / Sb;
+        Bws[idx] = r < R ? Bw[r * Sb + idx % Sb] : 0.0f;
+    }
+    double acc[2][2] = {{0.0, 0.0}, {0.0, 0.0}};
+    for (int w0 = 0; w0 < W64; w0 += WB) {
+        __syncthreads();  // the previous step's reads are done (and, first time, nothing)
+        for (int idx = tid; idx < 32 * Sa * WB; idx += 256) {
+            const int m = idx / (Sa * WB), rem = idx - m * (Sa * WB);
+            const int i = rem / WB, w = w0 + rem % WB;
+            const int64_t q = q0 + m;
+            As[m * strideA + rem] = (q < Q && w < W64) ? A[(q * Sa + i) * W64 + w] : 0ULL;
+        }
+        for (int idx = tid; idx < 32 * Sb * WB; idx += 256) {
+            const int m = idx / (Sb * WB), rem = idx - m * (Sb * WB);
+            const int j = rem / WB, w = w0 + rem % WB;
+            const int64_t r = r0 + m;
+            unsigned long long v = 0ULL;
+            if (r < R && w < W64)
+                v = kTiled ? B[((((r >> 4) * chunks + (w >> 2)) * Sb + j) * 64) + (w & 3) * 16 + (r & 15)]
+                           : B[(r * Sb + j) * W64 + w];
+            Bs[m * strideB + rem] = v;
+        }
+        __syncthreads();
+        for (int i = 0; i < Sa; ++i) {
+            unsigned long long a0[WB], a1[WB];
+#pragma unroll
+            for (int w = 0; w < WB; ++w) {
+                a0[w] = As[tq * strideA + i * WB + w];
+                a1[w] = As[(tq + 16) * strideA + i * WB + w];
+            }
+            const float aw0 = Aws[tq * Sa + i], aw1 = Aws[(tq + 16) * Sa + i];
+            for (int j = 0; j < Sb; ++j) {
+                const unsigned long long* b0 = Bs + tr * strideB + j * WB;
+                const unsigned long long* b1 = Bs + (tr + 16) * strideB + j * WB;
+                int c00 = 0, c01 = 0, c10 = 0, c11 = 0;
+#pragma unroll
+                for (int w = 0; w < WB; ++w) {
+                    const unsigned long long x0 = b0[w], x1 = b1[w];
+                    c00 += __popcll(a0[w] & x0);
+                    c01 += __popcll(a0[w] & x1);
+                    c10 += __popcll(a1[w] & x0);
+                    c11 += __popcll(a1[w] & x1);
+                }
+                const float bw0 = Bws[tr * Sb + j], bw1 = Bws[(tr + 16) * Sb + j];
+                acc[0][0] += static_cast<double>(c00) * static_cast<double>(aw0 * bw0);
+                acc[0][1] += static_cast<double>(c01) * static_cast<double>(aw0 * bw1);
+                acc[1][0] += static_cast<double>(c10) * static_cast<double>(aw1 * bw0);
+                acc[1][1] += static_cast<double>(c11) * static_cast<double>(aw1 * bw1);
+            }
+        }
+    }
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            const int64_t q = q0 + tq + 16 * a, r = r0 + tr + 16 * b;
+            if (q < Q && r < R) {
+                const int64_t col = key_indices ? key_indices[r] : r;
+                out[q * R_total + col] = static_cast<float>(acc[a][b]) * scale_inv;
+            }
+        }
+}
+
 // out[q, r] += bias[r] for the kernels that do not add the bias in their own epilogue
 __global__ void add_bias_kernel(float* __restrict__ out, const float* __restrict__ bias, int64_t Q, int64_t R,
                                 int64_t R_total) {
@@ -1749,6 +1838,49 @@ extern "C" int bsi_hip_dot_ewah_query(const uint64_t* comp_words, const int64_t*
                            pass_chunks, R, down_shift, scale_inv, out, chunk_ints);
     BSI_LAUNCH_CHECK("dot_mfma_stream_ewah_kernel");
     return BSI_OK;
+}
+
+template <int WB, bool kTiled>
+static int launch_dot_weighted(const uint64_t* A, const float* Aw, int Sa, int W64, const uint64_t* B, const float* Bw,
+                               int Sb, int64_t R, int64_t Q, const int64_t* key_indices, float scale_inv,
+                               int64_t R_total, float* out, hipStream_t st) {
+    const size_t lds = static_cast<size_t>(32) * ((Sa * WB + 1) + (Sb * WB + 1)) * 8 + static_cast<size_t>(32) * (Sa + Sb) * 4;
+    if (lds > 150 * 1024) return fail(BSI_ERR_UNSUPPORTED, "slice counts %d + %d do not fit the LDS tile", Sa, Sb);
+    static bool configured = false;
+    if (!configured) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dot_weighted_kernel<WB, kTiled>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+        configured = true;
+    }
+    const dim3 grid(static_cast<unsigned>((R + 31) / 32), static_cast<unsigned>((Q + 31) / 32));
+    hipLaunchKernelGGL((dot_weighted_kernel<WB, kTiled>), grid, dim3(256), lds, st,
+                       reinterpret_cast<const unsigned long long*>(A), Aw, Sa, W64,
+                       reinterpret_cast<const unsigned long long*>(B), Bw, Sb, (W64 + 3) / 4, R, Q,
+                       reinterpret_cast<const long long*>(key_indices), scale_inv, R_total, out);
+    BSI_LAUNCH_CHECK("dot_weighted_kernel");
+    return BSI_OK;
+}
+
+extern "C" int bsi_hip_dot_weighted(const uint64_t* A, const float* Aw, int Sa, int W64, const uint64_t* B,
+                                    int b_layout, const float* Bw, int Sb, int64_t R, int64_t Q,
+                                    const int64_t* key_indices, float scale_inv, int64_t R_total, float* out,
+                                    void* stream) {
+    BSI_REQUIRE(R >= 0 && Q >= 0 && W64 >= 1, "bad shape");
+    BSI_REQUIRE(Sa >= 1 && Sa <= 64 && Sb >= 1 && Sb <= 64, "slice counts must be in [1, 64] (got %d, %d)", Sa, Sb);
+    BSI_REQUIRE(R_total >= R, "R_total (%lld) < R (%lld)", static_cast<long long>(R_total), static_cast<long long>(R));
+    BSI_REQUIRE(b_layout == BSI_LAYOUT_CANONICAL || b_layout == BSI_LAYOUT_TILED16,
+                "the weighted dot reads key planes (canonical or tiled16), got layout %d", b_layout);
+    BSI_REQUIRE((Q + 31) / 32 <= 65535, "too many query rows for one launch");
+    if (R == 0 || Q == 0) return BSI_OK;
+    BSI_REQUIRE(A && Aw && B && Bw && out, "null pointer");
+    hipStream_t st = as_stream(stream);
+    const bool tiled = b_layout == BSI_LAYOUT_TILED16;
+    // 8 words of every slice per step while that fits 60 KiB of LDS, else 2
+    if (Sa + Sb <= 28)
+        return tiled ? launch_dot_weighted<8, true>(A, Aw, Sa, W64, B, Bw, Sb, R, Q, key_indices, scale_inv, R_total, out, st)
+                     : launch_dot_weighted<8, false>(A, Aw, Sa, W64, B, Bw, Sb, R, Q, key_indices, scale_inv, R_total, out, st);
+    return tiled ? launch_dot_weighted<2, true>(A, Aw, Sa, W64, B, Bw, Sb, R, Q, key_indices, scale_inv, R_total, out, st)
+                 : launch_dot_weighted<2, false>(A, Aw, Sa, W64, B, Bw, Sb, R, Q, key_indices, scale_inv, R_total, out, st);
 }
 
 extern "C" int bsi_hip_dot_timed(const uint64_t* A, const int8_t* A_ints8, const float* A_chunk_scales,

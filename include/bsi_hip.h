@@ -94,6 +94,16 @@ int bsi_hip_quantize_shift_pack_chunk_batch(const void* x_device, int dtype, int
                                             int slices, int words_per_slice, double dec_scale, int fixed_bits,
                                             const int32_t* shifts_device, uint64_t* words_device, void* stream);
 
+/* Decimal mode (no fixed bits; the slice count follows the data).  From the rounded ints [Q, d]:
+ * *max_abs_device = largest |value| of the batch (0 when all are zero) and row_negative_device[q] = 1
+ * when row q holds a negative value.  The caller reads max_abs back, takes
+ * S = min(64, bit_width(max_abs) + 2) (2 when all zero), packs with bsi_hip_pack_bits_batch and gives
+ * rows with a negative value the two's-complement slice weights, the others the unsigned ones.
+ * Replaces the ATen reductions of the non-fixed batch builder (bsi_vector_cuda.cpp:1088-1100, 1146-1152;
+ * slice-count rule :746-754) and of the 1-D builder (:788-797). */
+int bsi_hip_decimal_stats(const int64_t* ints_device, int64_t Q, int64_t d, uint64_t* max_abs_device,
+                          int32_t* row_negative_device, void* stream);
+
 /* int64 [Q, d] -> canonical words [Q, slices, words_per_slice] (low `slices` bits of each value).
  * Replaces launch_pack_bits_all_ballot_batch / launch_pack_bits_all_ballot (Q = 1)
  * (bsi_cuda_kernels_pack.cuh:176-230). */
@@ -199,6 +209,19 @@ int bsi_hip_dot_ewah_query(const uint64_t* comp_words, const int64_t* comp_off, 
                            int W64, const float* A_chunk_scales, int A_scale_stride, const uint64_t* B_tiled,
                            const float* Bw, int Sb, int64_t R, float scale_inv, float* out, int32_t* chunk_ints,
                            void* stream);
+
+/* Weighted-slice dot for operands with arbitrary per-slice float weights (decimal-mode operands, whose
+ * slice count follows the data, or fixed-bit operands without chunk scales):
+ *   out[q, idx[r]] = float(sum_{i,j,w} popcount(A[q,i,w] & B[r,j,w]) * double(Aw[q,i] * Bw[r,j])) * scale_inv
+ * A [Q, Sa, W64], Aw [Q, Sa], B [R, Sb, W64] (canonical or tiled16), Bw [R, Sb], Sa, Sb in [1, 64];
+ * key_indices (may be NULL = identity) maps row r of B to its output column, as the reference's keys grouped
+ * by slice count need (bsi_cuda.cpp:956-1000).  The sum is exact in float64 while it stays below 2^53 and is
+ * rounded once, where the reference adds the same terms in fp32 in an order set by its launch shape.
+ * Replaces launch_popcount_weighted_keys_literal_fused_multiq without chunk scales
+ * (bsi_cuda_kernels_dot.cuh:58-190 fallback kernel, :211-1283 tensor-core kernel, dispatch :2575-3090). */
+int bsi_hip_dot_weighted(const uint64_t* A, const float* Aw, int Sa, int W64, const uint64_t* B, int b_layout,
+                         const float* Bw, int Sb, int64_t R, int64_t Q, const int64_t* key_indices, float scale_inv,
+                         int64_t R_total, float* out, void* stream);
 
 /* Runs fn-independent timing of `iters` back-to-back bsi_hip_dot launches between two HIP events
  * recorded on `stream`, synchronises, and returns the mean launch duration in microseconds.

@@ -3,7 +3,8 @@
 TEST INFRASTRUCTURE ONLY: imported by ``tests/``, by the smoke check and by the CPU-baseline
 leg of the benchmark, never by the library.  Each function forwards to the C restatement of
 the reference block named in its docstring (paths relative to the reference's
-``bsi_ops/csrc/cuda/``).
+``bsi_ops/csrc/cuda/``); the decimal-mode functions at the end are numpy.  Every function is
+pinned by an independent check in ``tests/test_oracle_*.py`` (none is "parity unpinned").
 """
 from __future__ import annotations
 
@@ -228,3 +229,61 @@ def build_keys(k: np.ndarray, decimal_places: int = 2, fixed_bits: int = 6, clip
     ints, shifts, scales = quantize_fixed(k, decimal_places, fixed_bits, False, clip_k)
     bw = slice_weights(fixed_bits)[None, :] * scales[:, None]
     return dict(words=pack(ints, fixed_bits), ints=ints, shifts=shifts, scales=scales, slice_weights=bw.astype(np.float32))
+
+
+# --------------------------------------------------------------------------- decimal (data-dependent slice count) mode
+
+
+def choose_total_slices(any_non_zero: bool, max_abs: int) -> int:
+    """bsi_vector_cuda.cpp:746-754 with ``fixed_bits == 0``: magnitude bits of the largest |value| plus two,
+    at most 64; two slices for an all-zero input."""
+    if not any_non_zero:
+        return 2
+    return min(64, max(1, int(max_abs).bit_length()) + 2)
+
+
+def build_decimal(x: np.ndarray, decimal_places: int = 2):
+    """Batch builder without fixed bits, bsi_vector_cuda.cpp:565-577 (round half away of ``x * 10^dec``, no
+    scale) and :1088-1166: one slice count for the whole batch from its largest magnitude, the low ``S`` bits
+    of every two's-complement value packed into planes, and per row the two's-complement slice weights when
+    the row holds a negative value, the unsigned ones otherwise.  The 1-D builder (:778-852) is the Q = 1 case.
+
+    Returns dict(words [Q,S,W] uint64, ints [Q,d] int64, S, slice_weights [Q,S] float32, negative [Q] bool).
+    """
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    Q, d = x.shape
+    ints = round_to_int64(x, decimal_places) if x.size else np.zeros((Q, d), dtype=np.int64)
+    any_non_zero = bool(Q > 0 and np.any(ints != 0))
+    max_abs = int(np.abs(ints).max()) if any_non_zero else 0
+    S = max(1, choose_total_slices(any_non_zero, max_abs))
+    negative = (ints < 0).any(axis=1) if Q > 0 else np.zeros((0,), dtype=bool)
+    w_twos, w_unsigned = slice_weights(S, 0, True), slice_weights(S, 0, False)
+    weights = np.where(negative[:, None], w_twos[None, :], w_unsigned[None, :]).astype(np.float32)
+    return dict(words=pack(ints, S), ints=ints, S=S, slice_weights=weights, negative=negative)
+
+
+def dot_weighted(A: np.ndarray, Aw: np.ndarray, B: np.ndarray, Bw: np.ndarray, scale_inv: float) -> np.ndarray:
+    """The weighted-slice dot every non-chunk-scale call computes, bsi_cuda_kernels_dot.cuh:150-187:
+    ``out[q,r] = (sum over i, j, w of popcount(A[q,i,w] & B[r,j,w]) * (Aw[q,i] * Bw[r,j])) * scale_inv`` with the
+    coefficient ``Aw * Bw`` a float32 product.  The reference adds the terms in fp32 in an order fixed by its
+    launch shape (strided per thread, then shuffle trees); every term is an integer times a power of two, so
+    this restatement adds them exactly (float64; exact while the sum of magnitudes stays below 2^53) and
+    rounds once to float32 -- the value any fp32 order approximates to within its rounding error.
+    """
+    A = np.ascontiguousarray(A, dtype=np.uint64)
+    B = np.ascontiguousarray(B, dtype=np.uint64)
+    Aw = np.ascontiguousarray(Aw, dtype=np.float32)
+    Bw = np.ascontiguousarray(Bw, dtype=np.float32)
+    Q, Sa, W = A.shape
+    R, Sb, Wb = B.shape
+    assert W == Wb and Aw.shape == (Q, Sa) and Bw.shape == (R, Sb)
+    out = np.zeros((Q, R), dtype=np.float32)
+    for q in range(Q):
+        # cnt[r, i, j] = sum_w popcount(A[q,i,w] & B[r,j,w])
+        cnt = np.zeros((R, Sa, Sb), dtype=np.int64)
+        for i in range(Sa):
+            cnt[:, i, :] = np.bitwise_count(A[q, i][None, None, :] & B).sum(axis=2, dtype=np.int64)
+        coeff = (Aw[q][None, :, None] * Bw[:, None, :]).astype(np.float32)          # float32 products
+        acc = (cnt.astype(np.float64) * coeff.astype(np.float64)).sum(axis=(1, 2))   # exact
+        out[q] = acc.astype(np.float32) * np.float32(scale_inv)
+    return out

@@ -75,9 +75,8 @@ def test_flags_defaults_and_overrides(monkeypatch):
     assert f["core"] == 1
     monkeypatch.setenv("BSI_FIXED_BITS_QUERIES", "0")
     bsi_ops._reset_flag_cache()
-    assert bsi_ops._flags()["bits_q"] == 0
-    with pytest.raises(RuntimeError):
-        bsi_ops._require_fixed(0, "x")
+    assert bsi_ops._flags()["bits_q"] == 0   # decimal mode for queries; keys stay fixed
+    assert bsi_ops._flags()["bits_k"] == 2
     for k in ("BSI_FIXED_BITS", "BSI_FIXED_BITS_KEYS", "BSI_FIXED_CHUNK_SCALE", "BSI_FIXED_CLIP_K", "BSI_DOT_CORE",
               "BSI_FIXED_BITS_QUERIES"):
         monkeypatch.delenv(k)

@@ -816,3 +816,208 @@ def test_linear_drop_in(ops, oracle):
     m2 = Tiny()
     quantize_model_bsi(m2, scope="mlp", verbose=False)
     assert isinstance(m2.fc1, BSIQuantizedLinear) and isinstance(m2.q_proj, torch.nn.Linear)
+
+
+# ------------------------------------------------------------------ decimal mode (slice count from the data)
+
+
+def _decimal_case(Q, R, d, seed, qscale=1.0, kscale=0.5):
+    rng = np.random.default_rng(seed)
+    x = (rng.standard_normal((Q, d)) * qscale).astype(np.float32)
+    k = (rng.standard_normal((R, d)) * kscale).astype(np.float32)
+    if Q > 1:
+        x[1] = np.abs(x[1])  # a row without negatives: unsigned weights
+    if R > 2:
+        k[2] = 0.0
+    return x, k
+
+
+@pytest.mark.parametrize("Q,d,scale", [(9, 700, 1.0), (3, 64, 1.0e6), (70, 2048, 3.0), (2, 5, 1.0e15)])
+def test_decimal_stats_and_pack_match_oracle(hip, oracle, Q, d, scale):
+    L = hip.lib
+    x, _ = _decimal_case(Q, 1, d, seed=Q + d, qscale=scale)
+    want = oracle.build_decimal(x, 2)
+    xd = torch.from_numpy(x).cuda()
+    ints = torch.empty((Q, d), dtype=torch.int64, device="cuda")
+    hip.check(L.bsi_hip_quantize_round_to_int64(xd.data_ptr(), hip.DTYPE_F32, Q * d, 100.0, ints.data_ptr(), st()), "round")
+    max_abs = torch.full((1,), -5, dtype=torch.int64, device="cuda")   # must be cleared by the call
+    neg = torch.full((Q,), 7, dtype=torch.int32, device="cuda")
+    hip.check(L.bsi_hip_decimal_stats(ints.data_ptr(), Q, d, max_abs.data_ptr(), neg.data_ptr(), st()), "stats")
+    assert np.array_equal(ints.cpu().numpy(), want["ints"])
+    m = int(max_abs.item())
+    assert m == int(np.abs(want["ints"]).max())
+    assert np.array_equal(neg.cpu().numpy().astype(bool), want["negative"])
+    S = oracle.choose_total_slices(m != 0, m)
+    assert S == want["S"]
+    W = (d + 63) // 64
+    words = torch.full((Q, S, W), -1, dtype=torch.int64, device="cuda")
+    hip.check(L.bsi_hip_pack_bits_batch(ints.data_ptr(), Q, d, S, W, words.data_ptr(), st()), "pack")
+    assert np.array_equal(host_u64(words), want["words"])
+    # all-zero batch: max 0, no negatives
+    z = torch.zeros((4, 100), dtype=torch.int64, device="cuda")
+    negz = torch.full((4,), 7, dtype=torch.int32, device="cuda")
+    hip.check(L.bsi_hip_decimal_stats(z.data_ptr(), 4, 100, max_abs.data_ptr(), negz.data_ptr(), st()), "stats")
+    assert int(max_abs.item()) == 0 and not negz.any()
+
+
+def _run_weighted(hip, a, b, Q, R, W, layout=0, key_indices=None, R_total=None, scale_inv=1e-4):
+    L = hip.lib
+    A, Aw = dev(a["words"]), dev(a["slice_weights"])
+    B, Bw = dev(b["words"]), dev(b["slice_weights"])
+    Sa, Sb = a["words"].shape[1], b["words"].shape[1]
+    if layout == 1:
+        chunks = (W + 3) // 4
+        Bt = torch.full((((R + 15) // 16) * chunks * Sb * 64,), -1, dtype=torch.int64, device="cuda")
+        hip.check(L.bsi_hip_tile_key_planes(B.data_ptr(), R, Sb, W, Bt.data_ptr(), st()), "tile")
+        B = Bt
+    R_total = R if R_total is None else R_total
+    out = torch.full((Q, R_total), float("nan"), dtype=torch.float32, device="cuda")
+    idx = None if key_indices is None else torch.from_numpy(np.asarray(key_indices, dtype=np.int64)).cuda()
+    hip.check(L.bsi_hip_dot_weighted(A.data_ptr(), Aw.data_ptr(), Sa, W, B.data_ptr(), layout, Bw.data_ptr(), Sb, R, Q,
+                                     idx.data_ptr() if idx is not None else None, float(np.float32(scale_inv)), R_total,
+                                     out.data_ptr(), st()), "weighted dot")
+    torch.cuda.synchronize()
+    return out.cpu().numpy()
+
+
+@pytest.mark.parametrize("Q,R,d,qscale,layout", [(5, 7, 300, 1.0, 0), (33, 70, 2048, 1.0, 0), (64, 256, 2048, 1.0, 1),
+                                                 (40, 33, 700, 1.0, 1), (3, 50, 640, 3.0e4, 0), (17, 40, 512, 1.0e9, 0),
+                                                 (1, 1, 64, 1.0, 0), (32, 32, 512, 1.0, 0)])
+def test_dot_weighted_matches_oracle(hip, oracle, Q, R, d, qscale, layout):
+    """Decimal operands on both sides; large magnitudes take the narrow-step instantiation (Sa + Sb > 28).
+    Bit-exact against the oracle's exact sum, which is also the integer matrix product of the rounded values."""
+    x, k = _decimal_case(Q, R, d, seed=Q * 31 + R, qscale=qscale)
+    a, b = oracle.build_decimal(x, 2), oracle.build_decimal(k, 2)
+    W = (d + 63) // 64
+    want = oracle.dot_weighted(a["words"], a["slice_weights"], b["words"], b["slice_weights"], np.float32(1e-4))
+    got = _run_weighted(hip, a, b, Q, R, W, layout=layout)
+    assert np.array_equal(got, want)
+    exact = (a["ints"].astype(object) @ b["ints"].astype(object).T)
+    if max(abs(int(v)) for v in exact.reshape(-1)) < 2 ** 53:
+        assert np.array_equal(got, exact.astype(np.float64).astype(np.float32) * np.float32(1e-4))
+    np.testing.assert_allclose(got, want, rtol=FP32_RTOL)  # the stated bar
+
+
+def test_dot_weighted_key_indices_and_row_stride(hip, oracle):
+    """Keys of one slice-count group scattered into a wider output by key_indices; other columns untouched."""
+    Q, R, d, R_total = 10, 37, 300, 50
+    x, k = _decimal_case(Q, R, d, seed=5)
+    a, b = oracle.build_decimal(x, 2), oracle.build_decimal(k, 2)
+    perm = np.random.default_rng(1).permutation(R_total)[:R]
+    want = oracle.dot_weighted(a["words"], a["slice_weights"], b["words"], b["slice_weights"], np.float32(1e-4))
+    got = _run_weighted(hip, a, b, Q, R, 5, key_indices=perm, R_total=R_total)
+    assert np.array_equal(got[:, perm], want)
+    untouched = np.setdiff1d(np.arange(R_total), perm)
+    assert np.isnan(got[:, untouched]).all()
+
+
+def test_dot_weighted_mixed_with_fixed_bit_keys(hip, oracle):
+    x, k = _decimal_case(20, 45, 1024, seed=9, kscale=3.0)
+    a, b = oracle.build_decimal(x, 2), oracle.build_keys(k, 2, 6)
+    want = oracle.dot_weighted(a["words"], a["slice_weights"], b["words"], b["slice_weights"], np.float32(1e-4))
+    for layout in (0, 1):
+        assert np.array_equal(_run_weighted(hip, a, b, 20, 45, 16, layout=layout), want)
+
+
+def test_dot_weighted_rejects_bad_arguments(hip):
+    L = hip.lib
+    t = torch.zeros((64,), dtype=torch.int64, device="cuda")
+    f = torch.zeros((64,), dtype=torch.float32, device="cuda")
+    assert L.bsi_hip_dot_weighted(t.data_ptr(), f.data_ptr(), 65, 1, t.data_ptr(), 0, f.data_ptr(), 2, 1, 1, None, 1.0, 1,
+                                  f.data_ptr(), st()) != 0
+    assert b"slice counts" in L.bsi_hip_last_error()
+    assert L.bsi_hip_dot_weighted(t.data_ptr(), f.data_ptr(), 2, 1, t.data_ptr(), 2, f.data_ptr(), 2, 1, 1, None, 1.0, 1,
+                                  f.data_ptr(), st()) != 0
+    assert L.bsi_hip_dot_weighted(None, f.data_ptr(), 2, 1, t.data_ptr(), 0, f.data_ptr(), 2, 1, 1, None, 1.0, 1,
+                                  f.data_ptr(), st()) != 0
+
+
+def test_ops_decimal_mode_known_answers_and_pipeline(ops, oracle, monkeypatch):
+    """BSI_FIXED_BITS=0: the reference's decimal API end to end (its check scripts' known answers), then a random
+    batch against the oracle, the row-handle form, the 1-D builders and the keyset statistics."""
+    monkeypatch.setenv("BSI_FIXED_BITS", "0")
+    ops._reset_flag_cache()
+    kat = json.load(open(GOLDEN))
+    for case in kat["vector_dot"] + kat["batch_dot"]:
+        q = torch.tensor(case["q"] if "K" in case else [case["q"]], dtype=torch.float32)
+        K = torch.tensor(case["K"] if "K" in case else [case["k"]], dtype=torch.float32)
+        dec = case["decimal_places"]
+        kcap, *_ = ops.build_bsi_keys_cuda(K, dec, 0.2)
+        qcap = ops.build_bsi_queries_cuda_batch_packed(q.cuda(), dec, 0.2)
+        out, *_ = ops.batch_dot_product_multiquery_cuda_batch_caps(qcap, kcap)
+        want = torch.tensor(case["expected"], dtype=torch.float32).reshape(out.shape)
+        assert torch.allclose(out.cpu(), want, atol=1e-5), case["cite"]
+    x, k = _decimal_case(33, 70, 2048, seed=3)
+    a, b = oracle.build_decimal(x, 2), oracle.build_decimal(k, 2)
+    want = oracle.dot_weighted(a["words"], a["slice_weights"], b["words"], b["slice_weights"], oracle.scale_inv(2, 2))
+    kcap, nbytes, nk, d, W = ops.build_bsi_keys_cuda(torch.from_numpy(k), 2, 0.2)
+    assert (nk, d, W) == (70, 2048, 32) and nbytes == 70 * b["S"] * 32 * 8
+    assert ops.bsi_keys_cuda_stats(kcap)["Sb_counts"] == {b["S"]: 70}
+    qcap = ops.build_bsi_queries_cuda_batch_packed(torch.from_numpy(x).cuda(), 2, 0.2)
+    assert qcap.Sa == a["S"] and np.array_equal(host_u64(qcap.words), a["words"])
+    assert np.array_equal(qcap.slice_weights.cpu().numpy(), a["slice_weights"])
+    out, *_ = ops.batch_dot_product_multiquery_cuda_batch_caps(qcap, kcap)
+    assert np.array_equal(out.cpu().numpy(), want)
+    rows = ops.build_bsi_queries_cuda_batch(torch.from_numpy(x).cuda(), 2, 0.2)
+    out2, *_ = ops.batch_dot_product_multiquery_cuda_caps(rows, kcap)
+    assert torch.equal(out2, out)
+    assert ops.bsi_query_caps_stats(rows)["S_counts"] == {a["S"]: 33}
+    # 1-D builders: the slice count follows that vector alone
+    one = oracle.build_decimal(x[1:2], 2)
+    h, mem, S, W1 = ops.build_bsi_query_cuda(torch.from_numpy(x[1]).cuda(), 2, 0.2)
+    assert S == one["S"] and not h.twos_complement and np.array_equal(host_u64(h.dev_words), one["words"][0])
+    hh, *_ = ops.build_bsi_query_cuda_hybrid(torch.from_numpy(x[0]).cuda(), 2, 0.5)
+    assert hh.twos_complement
+    want0 = oracle.build_decimal(x[0:1], 2)
+    o0, *_ = ops.batch_dot_product_multiquery_cuda_caps([hh], kcap)
+    assert np.array_equal(o0.cpu().numpy(), oracle.dot_weighted(want0["words"], want0["slice_weights"], b["words"],
+                                                                 b["slice_weights"], oracle.scale_inv(2, 2)))
+    with pytest.raises(RuntimeError, match="fixed-bit operands only"):
+        ops.debug_chunk_ints(qcap, kcap)
+
+
+def test_ops_decimal_queries_with_fixed_keys_and_the_reverse(ops, oracle, monkeypatch):
+    x, k = _decimal_case(12, 40, 1024, seed=21, kscale=0.02)
+    monkeypatch.setenv("BSI_FIXED_BITS_QUERIES", "0")
+    ops._reset_flag_cache()
+    a, b = oracle.build_decimal(x, 2), oracle.build_keys(k, 2, 6)
+    kcap, *_ = ops.build_bsi_keys_cuda(torch.from_numpy(k), 2, 0.2)       # fixed 6-bit, tiled planes + int8 image
+    qcap = ops.build_bsi_queries_cuda_batch_packed(torch.from_numpy(x).cuda(), 2, 0.2)
+    out, *_ = ops.batch_dot_product_multiquery_cuda_batch_caps(qcap, kcap)
+    assert np.array_equal(out.cpu().numpy(), oracle.dot_weighted(a["words"], a["slice_weights"], b["words"],
+                                                                  b["slice_weights"], oracle.scale_inv(2, 2)))
+    # the reverse: chunk-scaled fixed queries cannot meet decimal keys; row-scaled ones can
+    monkeypatch.delenv("BSI_FIXED_BITS_QUERIES")
+    monkeypatch.setenv("BSI_FIXED_BITS_KEYS", "0")
+    ops._reset_flag_cache()
+    kcap, *_ = ops.build_bsi_keys_cuda(torch.from_numpy(k), 2, 0.2)
+    qcap = ops.build_bsi_queries_cuda_batch_packed(torch.from_numpy(x).cuda(), 2, 0.2)
+    with pytest.raises(RuntimeError, match="chunk-scaled queries need fixed-bit keys"):
+        ops.batch_dot_product_multiquery_cuda_batch_caps(qcap, kcap)
+    monkeypatch.setenv("BSI_FIXED_CHUNK_SCALE", "0")
+    ops._reset_flag_cache()
+    qcap = ops.build_bsi_queries_cuda_batch_packed(torch.from_numpy(x).cuda(), 2, 0.2)
+    out, *_ = ops.batch_dot_product_multiquery_cuda_batch_caps(qcap, kcap)
+    qa, kb = oracle.build_queries(x, 2, 7), oracle.build_decimal(k, 2)
+    ints, shifts, scales = oracle.quantize_fixed(x, 2, 7, False)
+    aw = (oracle.slice_weights(7)[None, :] * scales[:, None]).astype(np.float32)
+    want = oracle.dot_weighted(oracle.pack(ints, 7), aw, kb["words"], kb["slice_weights"], oracle.scale_inv(2, 2))
+    assert np.array_equal(out.cpu().numpy(), want)
+
+
+def test_linear_drop_in_decimal_mode(ops, monkeypatch):
+    """BSIQuantizedLinear with BSI_FIXED_BITS=0: the output is the dense layer's up to the 10^-dec rounding grid."""
+    from bsipytorch_amd import linear
+
+    monkeypatch.setenv("BSI_FIXED_BITS", "0")
+    ops._reset_flag_cache()
+    torch.manual_seed(4)
+    dense = torch.nn.Linear(512, 96).cuda()
+    layer = linear.BSIQuantizedLinear(dense, decimalPlaces=3, compress_threshold=0.5)
+    x = torch.randn(24, 512, device="cuda")
+    with torch.no_grad():
+        got, ref = layer(x), dense(x)
+    # |error| <= sum over d of (|x| + |w| + grid) * grid / 2, far below this bound in practice
+    assert (got - ref).abs().max().item() < 512 * 0.0005 * 5.0
+    cos = torch.nn.functional.cosine_similarity(got.flatten(), ref.flatten(), dim=0).item()
+    assert cos > 0.9999

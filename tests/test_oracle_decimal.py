@@ -1,0 +1,106 @@
+"""Pins the decimal-mode part of the CPU oracle (slice count from the data, weighted-slice dot).
+
+The checks are independent of the oracle's formulas: the slice-count rule against hand-worked bit
+widths, the planes and per-row weights by reconstructing every value from them, the dot against an
+integer matrix product of the rounded values, and the whole chain against the known answers the
+reference's own check scripts hold for its decimal API.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "reference_known_answers.json")
+
+
+def test_choose_total_slices_known_values(oracle):
+    # magnitude bits + 2, capped at 64; 2 for an all-zero input
+    assert oracle.choose_total_slices(False, 0) == 2
+    assert oracle.choose_total_slices(True, 1) == 3
+    assert oracle.choose_total_slices(True, 2) == 4
+    assert oracle.choose_total_slices(True, 3) == 4
+    assert oracle.choose_total_slices(True, 255) == 10
+    assert oracle.choose_total_slices(True, 256) == 11
+    assert oracle.choose_total_slices(True, (1 << 61) - 1) == 63
+    assert oracle.choose_total_slices(True, 1 << 61) == 64
+    assert oracle.choose_total_slices(True, 1 << 62) == 64  # 63 + 2 capped
+    assert oracle.choose_total_slices(True, 1 << 63) == 64
+
+
+def _reconstruct(words, weights, d):
+    """value[q, e] = sum_s bit_s(q, e) * weights[q, s], from the planes alone."""
+    Q, S, W = words.shape
+    e = np.arange(d)
+    bits = (words[:, :, e >> 6] >> (e & 63).astype(np.uint64)) & np.uint64(1)      # [Q, S, d]
+    return (bits.astype(np.float64) * weights.astype(np.float64)[:, :, None]).sum(axis=1)
+
+
+@pytest.mark.parametrize("d", [1, 63, 64, 65, 300])
+def test_build_decimal_reconstructs_every_value(oracle, d):
+    rng = np.random.default_rng(d)
+    x = (rng.standard_normal((6, d)) * 3).astype(np.float32)
+    x[0] = np.abs(x[0])          # a row without negatives: unsigned weights
+    x[1] = 0.0                   # an all-zero row
+    b = oracle.build_decimal(x, 2)
+    assert b["S"] == int(np.abs(b["ints"]).max()).bit_length() + 2
+    assert not b["negative"][0] and not b["negative"][1]
+    assert b["slice_weights"][0, -1] > 0 and (b["negative"][2:] == (b["ints"][2:] < 0).any(axis=1)).all()
+    for q in np.nonzero(b["negative"])[0]:
+        assert b["slice_weights"][q, -1] == -float(2 ** (b["S"] - 1))
+    np.testing.assert_array_equal(_reconstruct(b["words"], b["slice_weights"], d), b["ints"].astype(np.float64))
+    # bits past d stay clear
+    if d % 64:
+        assert not (b["words"][:, :, -1] >> np.uint64(d % 64)).any()
+
+
+def test_build_decimal_all_zero_and_rounding(oracle):
+    z = oracle.build_decimal(np.zeros((3, 70), dtype=np.float32), 2)
+    assert z["S"] == 2 and not z["words"].any() and (z["slice_weights"] == np.array([1, 2], dtype=np.float32)).all()
+    # ties go away from zero: 0.125 * 100 = 12.5 -> 13, -0.125 -> -13
+    b = oracle.build_decimal(np.array([[0.125, -0.125, 2.5]], dtype=np.float32), 2)
+    assert b["ints"].tolist() == [[13, -13, 250]] and b["S"] == 10
+
+
+@pytest.mark.parametrize("Q,R,d,dec", [(5, 7, 300, 2), (3, 4, 64, 0), (2, 9, 1000, 3)])
+def test_dot_weighted_equals_integer_matrix_product(oracle, Q, R, d, dec):
+    rng = np.random.default_rng(Q * 100 + R)
+    x = rng.standard_normal((Q, d)).astype(np.float32)
+    k = (rng.standard_normal((R, d)) * 0.5).astype(np.float32)
+    x[0] = np.abs(x[0])
+    a, b = oracle.build_decimal(x, dec), oracle.build_decimal(k, dec)
+    got = oracle.dot_weighted(a["words"], a["slice_weights"], b["words"], b["slice_weights"], oracle.scale_inv(dec, dec))
+    exact = a["ints"] @ b["ints"].T                       # int64, exact
+    want = exact.astype(np.float32) * oracle.scale_inv(dec, dec)
+    np.testing.assert_array_equal(got, want)
+    # and that is the float dot of the inputs up to the rounding grid
+    dense = x.astype(np.float64) @ k.astype(np.float64).T
+    assert np.abs(got - dense).max() <= d * (0.5 / 10 ** dec) * (np.abs(x).max() + np.abs(k).max()) + 1e-3
+
+
+def test_dot_weighted_with_fixed_bit_keys(oracle):
+    # decimal queries against fixed-bit keys: the key slice weights carry 2^shift
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((4, 256)).astype(np.float32)
+    k = (rng.standard_normal((6, 256)) * 3).astype(np.float32)
+    a, b = oracle.build_decimal(x, 2), oracle.build_keys(k, 2, 6)
+    got = oracle.dot_weighted(a["words"], a["slice_weights"], b["words"], b["slice_weights"], oracle.scale_inv(2, 2))
+    exact = a["ints"] @ (b["ints"] * (1 << b["shifts"].astype(np.int64))[:, None]).T
+    np.testing.assert_array_equal(got, exact.astype(np.float32) * oracle.scale_inv(2, 2))
+
+
+def test_reference_known_answers_decimal_mode(oracle):
+    """The reference's check scripts exercise exactly this API (decimal builder + weighted dot)."""
+    g = json.load(open(GOLDEN))
+    for case in g["vector_dot"]:
+        dec = case["decimal_places"]
+        a = oracle.build_decimal(np.array([case["q"]], dtype=np.float32), dec)
+        b = oracle.build_decimal(np.array([case["k"]], dtype=np.float32), dec)
+        out = oracle.dot_weighted(a["words"], a["slice_weights"], b["words"], b["slice_weights"], oracle.scale_inv(dec, dec))
+        assert abs(float(out[0, 0]) - case["expected"]) < 1e-4, case["cite"]
+    for case in g["batch_dot"]:
+        dec = case["decimal_places"]
+        a = oracle.build_decimal(np.array(case["q"], dtype=np.float32), dec)
+        b = oracle.build_decimal(np.array(case["K"], dtype=np.float32), dec)
+        out = oracle.dot_weighted(a["words"], a["slice_weights"], b["words"], b["slice_weights"], oracle.scale_inv(dec, dec))
+        np.testing.assert_allclose(out, np.array(case["expected"], dtype=np.float32), atol=1e-4, err_msg=case["cite"])
