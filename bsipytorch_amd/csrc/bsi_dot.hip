@@ -702,9 +702,9 @@ __device__ __forceinline__ void load16_to_lds(bsi_rsrc r, uint32_t lane_off, uin
                                              static_cast<int>(wave_off), 0, 0);
 }
 
-// Tile configuration: TM keys x TN queries per workgroup (128 x 128, 128 x 64 or 64 x 64; the smaller ones
-// for grids that would leave CUs without a workgroup), MFMA waves arranged 2 (keys) x kWavesN (queries),
-// each WM x WN tiles of 16 x 16; one loader wave per 64 operand rows.
+// Tile configuration: TM keys x TN queries per workgroup (128 x 128, 128 x 64, 64 x 64 or 64 x 32; the smaller
+// ones for grids that would leave CUs without a workgroup), MFMA waves arranged 2 (keys) x kWavesN (queries),
+// each WM x WN tiles of 16 x 16; one loader wave per (up to) 64 operand rows.
 static int g_i8_tile = 0;  // 0 = by grid size; 128, 12864 (128 keys x 64 queries) or 64 force a tile
 
 template <int TM, int TN>
@@ -713,7 +713,9 @@ struct I8Cfg {
     static constexpr int kWN = 2;                      // 16-query tiles per wave
     static constexpr int kWavesN = TN / 32;            // waves along the queries
     static constexpr int kConsumers = 2 * kWavesN;
-    static constexpr int kLoaders = (TM + TN) / 64;    // a loader wave moves 64 of the TM + TN operand rows
+    static constexpr int kGroups = (TM + TN) / 8;      // groups of 8 operand rows (1 KiB per half-chunk) in a stage
+    static constexpr int kLoaders = (kGroups + 7) / 8;  // a loader wave moves up to 8 groups per stage
+    static constexpr int kLoads = (kGroups + kLoaders - 1) / kLoaders;  // loads per loader wave and stage
     static constexpr int kBlock = (kConsumers + kLoaders) * 64;
     static constexpr int kOperandK = TM * 128;         // bytes of the key tile of one half-chunk
     static constexpr int kStage = (TM + TN) * 128;     // keys then queries
@@ -789,12 +791,15 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
         const bsi_rsrc rk = make_rsrc(K8 + static_cast<size_t>(r0) * rowbytes, static_cast<size_t>(R - r0) * rowbytes);
         const bsi_rsrc rq = make_rsrc(A8 + static_cast<size_t>(q0) * rowbytes, static_cast<size_t>(Q - q0) * rowbytes);
         const bsi_rsrc rs = make_rsrc(qscale + q0 * qscale_stride, static_cast<size_t>(Q - q0) * qscale_stride * 4);
-        // the stage has (TM + TN) / 8 groups of 8 rows, keys first; loader lw moves groups lw, lw + kLoaders, ...
-        uint32_t off[8];
-        bool is_key[8];  // wave-uniform
+        // the stage has kGroups groups of 8 rows, keys first; loader lw moves groups lw, lw + kLoaders, ... (when
+        // the groups do not divide evenly the last load wraps around and fetches a group a second time, so that
+        // every loader wave has the same number of loads in flight)
+        constexpr int NI = C::kLoads;
+        uint32_t off[NI];
+        bool is_key[NI];  // wave-uniform
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int g = lw + C::kLoaders * i;
+        for (int i = 0; i < NI; ++i) {
+            const int g = (lw + C::kLoaders * i) % C::kGroups;
             is_key[i] = g < TM / 8;
             const int rowl = (is_key[i] ? g : g - TM / 8) * 8 + (lane >> 3);  // row of its operand tile
             const uint32_t col = static_cast<uint32_t>((lane & 7) ^ ((rowl >> 1) & 7)) * 16;  // logical column landing here
@@ -804,16 +809,16 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
         }
         // scales: loader wave lw fetches the 64 queries of group lw % (TN / 64) (waves fetching the same group
         // write their own regions, so that every loader wave has the same number of loads in flight)
-        const int sq = (lw % (TN / 64)) * 64 + lane;
+        const int sq = (lw % (TN >= 64 ? TN / 64 : 1)) * 64 + lane;
         const uint32_t soff = static_cast<uint32_t>(((q0 + sq < Q) ? sq : (Q - 1 - q0)) * qscale_stride * 4);
         const int sstep = (qscale_stride == 1) ? 0 : 4;
         auto issue = [&](int h) {  // stage of half-chunk h (clamped to the last) into its ring slot
             const int hc = h < halves ? h : halves - 1;
-            unsigned char* slot = lds + (h & 3) * C::kStage + lw * 1024;
             const uint32_t so = static_cast<uint32_t>(hc) * 128;
 #pragma unroll
-            for (int i = 0; i < 8; ++i)
-                load16_to_lds(is_key[i] ? rk : rq, off[i], so, slot + i * (C::kLoaders * 1024));
+            for (int i = 0; i < NI; ++i)
+                load16_to_lds(is_key[i] ? rk : rq, off[i], so,
+                              lds + (h & 3) * C::kStage + ((lw + C::kLoaders * i) % C::kGroups) * 1024);
             if (h & 1) {  // with the second half of chunk c = h / 2: its scales
                 const int c = hc >> 1;
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(
@@ -824,13 +829,14 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
         issue(0);
         issue(1);
         issue(2);
-        asm volatile("s_waitcnt vmcnt(17)" ::: "memory");  // stage 0 landed (stage 1 + scales + stage 2 may be in flight)
+        // stage 0 landed (stage 1 + scales + stage 2, 2 NI + 1 instructions, may be in flight)
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NI + 1) : "memory");
         lds_barrier();
         for (int h = 0; h < halves; ++h) {
             issue(h + 3);  // its slot was released by the barrier that ended half h - 1
             // stage h + 1 (and the scales issued right behind it) landed; stages h + 2, h + 3 and one
-            // scale load, 17 instructions, may still be in flight
-            asm volatile("s_waitcnt vmcnt(17)" ::: "memory");
+            // scale load, 2 NI + 1 instructions, may still be in flight
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NI + 1) : "memory");
             lds_barrier();
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still be writing LDS when the workgroup ends
@@ -1555,20 +1561,21 @@ static void launch_mfma_i8_t(const int8_t* A8, const float* qscale, int stride, 
 
 // Tile choice.  The 128 x 128 tile moves the fewest operand bytes per MAC and is the fastest whenever its grid
 // covers the 256 CUs (one workgroup per CU at a time) -- measured up to several rounds of 256.  A smaller grid
-// leaves CUs idle that smaller tiles would use: a workgroup's time per half-chunk is about 1 : 0.63 : 0.35 for
-// 128 x 128 : 128 x 64 : 64 x 64, so take the least (rounds of 256 workgroups x time), the larger tile on a tie.
-// g_i8_tile forces a tile (tuning and tests).
+// leaves CUs idle that smaller tiles would use: a workgroup's time per half-chunk is about 1 : 0.63 : 0.35 : 0.31
+// for 128 x 128 : 128 x 64 : 64 x 64 : 64 x 32, so take the least (rounds of 256 workgroups x time), the larger
+// tile on a tie.  g_i8_tile forces a tile (tuning and tests).
 static int choose_i8_tile(int64_t R, int64_t Q) {
     if (g_i8_tile != 0) return g_i8_tile;
     const int64_t n128 = ((R + 127) / 128) * ((Q + 127) / 128);
     if (n128 > 256) return 128;
-    const int64_t n12864 = ((R + 127) / 128) * ((Q + 63) / 64);
-    const int64_t n64 = ((R + 63) / 64) * ((Q + 63) / 64);
-    const int64_t cost128 = 100;
-    const int64_t cost12864 = ((n12864 + 255) / 256) * 63;
-    const int64_t cost64 = ((n64 + 255) / 256) * 35;
-    if (cost128 <= cost12864 && cost128 <= cost64) return 128;
-    return cost12864 <= cost64 ? 12864 : 64;
+    const int64_t cost[4] = {100, ((((R + 127) / 128) * ((Q + 63) / 64) + 255) / 256) * 63,
+                             ((((R + 63) / 64) * ((Q + 63) / 64) + 255) / 256) * 35,
+                             ((((R + 63) / 64) * ((Q + 31) / 32) + 255) / 256) * 31};
+    const int tiles[4] = {128, 12864, 64, 6432};
+    int best = 0;
+    for (int i = 1; i < 4; ++i)
+        if (cost[i] < cost[best]) best = i;
+    return tiles[best];
 }
 
 static void launch_mfma_i8(const int8_t* A8, const float* qscale, int stride, const int8_t* K8, const float* Bw, int Sb,
@@ -1578,7 +1585,8 @@ static void launch_mfma_i8(const int8_t* A8, const float* qscale, int stride, co
 #define BSI_I8_ARGS A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias, st
     if (tile == 128) launch_mfma_i8_t<128, 128>(BSI_I8_ARGS);
     else if (tile == 12864) launch_mfma_i8_t<128, 64>(BSI_I8_ARGS);
-    else launch_mfma_i8_t<64, 64>(BSI_I8_ARGS);
+    else if (tile == 64) launch_mfma_i8_t<64, 64>(BSI_I8_ARGS);
+    else launch_mfma_i8_t<64, 32>(BSI_I8_ARGS);
 #undef BSI_I8_ARGS
 }
 
@@ -1651,7 +1659,8 @@ extern "C" int bsi_hip_planes_to_int8(const uint64_t* words, int64_t rows, int S
 extern "C" int bsi_hip_set_option(int option, int value) {
     switch (option) {
         case BSI_OPT_I8_TILE:
-            BSI_REQUIRE(value == 0 || value == 128 || value == 12864 || value == 64, "tile must be 0, 128, 12864 or 64");
+            BSI_REQUIRE(value == 0 || value == 128 || value == 12864 || value == 64 || value == 6432,
+                        "tile must be 0, 128, 12864, 64 or 6432");
             g_i8_tile = value;
             return BSI_OK;
         default:

@@ -161,8 +161,9 @@ int bsi_hip_planes_to_int8(const uint64_t* words_device, int64_t rows, int S, in
 
 /* Tuning knobs (process-wide, not thread-safe; set before launching).  No counterpart in the reference,
  * whose kernel selection is read from environment variables on every call (bsi_cuda_kernels_dot.cuh:2642). */
-#define BSI_OPT_I8_TILE 1 /* tile of the int8-image kernel: 128 (128 keys x 128 queries), 12864 (128 x 64) or 64 (64 x 64);
-                             0 (default) = chosen per call from the grid each tile would give on the 256 CUs */
+#define BSI_OPT_I8_TILE 1 /* tile of the int8-image kernel: 128 (128 keys x 128 queries), 12864 (128 x 64), 64 (64 x 64)
+                             or 6432 (64 x 32); 0 (default) = chosen per call from the grid each tile would give on
+                             the 256 CUs */
 int bsi_hip_set_option(int option, int value);
 
 /* Bytes of device workspace bsi_hip_dot needs for this shape and core (0 when none). */

@@ -184,6 +184,7 @@ def test_set_option_validates_on_host():
     from bsipytorch_amd import _lib
 
     assert _lib.lib.bsi_hip_set_option(_lib.OPT_I8_TILE, 12864) == 0
+    assert _lib.lib.bsi_hip_set_option(_lib.OPT_I8_TILE, 6432) == 0
     assert _lib.lib.bsi_hip_set_option(_lib.OPT_I8_TILE, 96) == 1
     assert _lib.lib.bsi_hip_set_option(_lib.OPT_I8_TILE, 0) == 0
     assert _lib.lib.bsi_hip_set_option(999, 1) == 1
