@@ -19,6 +19,7 @@ code paths (``BSI_TC_DOT``, ``BSI_TC_TMA``, ``BSI_TC_CPASYNC``, ``BSI_TC_R_SWEEP
 """
 from __future__ import annotations
 
+import json
 import os
 import sys
 from typing import List, Optional
@@ -493,6 +494,38 @@ def build_bsi_query_cuda_hybrid(q: torch.Tensor, decimal_places: int, compress_t
     return h, int(h.mem_bytes), h.S, h.W
 
 
+def _install_fixed_key_planes(h: "PrebuiltBSIKeysCUDA", words: torch.Tensor) -> None:
+    """Derive the representations the dot reads from canonical fixed-bit planes [R, Sb, W]: the cached int8
+    image (BSI_KEY_INT8_IMAGE) and the tiled planes (BSI_KEY_LAYOUT), or the canonical planes themselves."""
+    f = _flags()
+    dev = words.device
+    R = h.num_keys
+    if f["key_image"] and R > 0 and 2 <= h.Sb <= 8:
+        # compute-bound shapes contract this image on the matrix cores; the planes stay the stored form
+        h.ints8 = torch.empty((R, ((h.W + 3) // 4) * 256), dtype=torch.int8, device=dev)
+        check(lib.bsi_hip_planes_to_int8(words.data_ptr(), R, h.Sb, h.W, h.ints8.data_ptr(), _stream()),
+              "bsi_hip_planes_to_int8")
+    if f["tiled"] and R > 0:
+        chunks = (h.W + 3) // 4
+        tiled = torch.empty(((R + 15) // 16, chunks, h.Sb, 64), dtype=torch.int64, device=dev)
+        check(lib.bsi_hip_tile_key_planes(words.data_ptr(), R, h.Sb, h.W, tiled.data_ptr(), _stream()),
+              "bsi_hip_tile_key_planes")
+        h.words, h.layout = tiled, _lib.LAYOUT_TILED16
+    else:
+        h.words, h.layout = words, _lib.LAYOUT_CANONICAL
+
+
+def canonical_key_planes(keys: "PrebuiltBSIKeysCUDA") -> torch.Tensor:
+    """The keyset's planes as canonical words [R, Sb, W] int64 on the device (undoes the 16-row tiling:
+    word (r, j, 4c + g) sits at tile r // 16, chunk c, slice j, position g * 16 + r % 16)."""
+    if keys.layout == _lib.LAYOUT_CANONICAL:
+        return keys.words
+    R, Sb, W = keys.num_keys, keys.Sb, keys.W
+    tiles, chunks = keys.words.shape[0], keys.words.shape[1]
+    t = keys.words.view(tiles, chunks, Sb, 4, 16).permute(0, 4, 2, 1, 3)  # [tile, r % 16, j, c, g]
+    return t.reshape(tiles * 16, Sb, chunks * 4)[:R, :, :W].contiguous()
+
+
 def build_bsi_keys_cuda(K: torch.Tensor, decimal_places: int, compress_threshold: float = 0.2):
     """bsi_cuda.cpp:863-910 (fixed-bit branch): per-row scale, Sb slices, ``Bw[r, j] = w_j * 2^shift_r``.
     Returns (handle, total_bytes_of_words, num_keys, d, W)."""
@@ -524,22 +557,89 @@ def build_bsi_keys_cuda(K: torch.Tensor, decimal_places: int, compress_threshold
     h.shifts = shifts
     h.slice_weights = (_slice_weights(h.Sb, 0, True, dev).unsqueeze(0) * scales.unsqueeze(1)).contiguous()
     total_bytes = words.numel() * 8
-    if f["key_image"] and R > 0 and 2 <= h.Sb <= 8:
-        # compute-bound shapes contract this image on the matrix cores; the planes stay the stored form
-        h.ints8 = torch.empty((R, ((h.W + 3) // 4) * 256), dtype=torch.int8, device=dev)
-        check(lib.bsi_hip_planes_to_int8(words.data_ptr(), R, h.Sb, h.W, h.ints8.data_ptr(), _stream()),
-              "bsi_hip_planes_to_int8")
-    if f["tiled"] and R > 0:
-        chunks = (h.W + 3) // 4
-        tiled = torch.empty(((R + 15) // 16, chunks, h.Sb, 64), dtype=torch.int64, device=dev)
-        check(lib.bsi_hip_tile_key_planes(words.data_ptr(), R, h.Sb, h.W, tiled.data_ptr(), _stream()),
-              "bsi_hip_tile_key_planes")
-        h.words, h.layout = tiled, _lib.LAYOUT_TILED16
-    else:
-        h.words, h.layout = words, _lib.LAYOUT_CANONICAL
+    _install_fixed_key_planes(h, words)
     if f["debug"]:
         print(f"[BSI_HIP] build_bsi_keys_cuda: R={R} slices={h.Sb} words_per_slice={h.W} layout={h.layout}")
     return h, int(total_bytes), int(R), int(d), int(h.W)
+
+
+# --------------------------------------------------------------------------- keyset files
+
+_KEYSET_MAGIC = b"BSIKEYS1"
+_KEYSET_FILE = "keyset.bsik"
+
+
+def _keyset_header(keys: "PrebuiltBSIKeysCUDA") -> dict:
+    return {"format": 1, "num_keys": keys.num_keys, "d": keys.d, "W": keys.W, "Sb": keys.Sb, "decimals": keys.decimals,
+            "threshold": keys.threshold, "fixed": bool(keys.fixed), "byte_order": "little",
+            "arrays": ["planes uint64 [num_keys, Sb, W]", "slice_weights float32 [num_keys, Sb]"]
+                      + (["shifts int32 [num_keys]"] if keys.fixed else [])}
+
+
+def keyset_size_on_disk_cuda(keyset_cuda_cap):
+    """(bytes of the planes in device memory, bytes save_keyset_cuda would write); counterpart of
+    keyset_size_on_disk (bsiFunctions.cpp:775-790) for device keysets."""
+    keys = _capsule(keyset_cuda_cap, PrebuiltBSIKeysCUDA, "Invalid CUDA keys capsule")
+    plane_bytes = keys.num_keys * keys.Sb * keys.W * 8
+    head = len(json.dumps(_keyset_header(keys)).encode())
+    head = 16 + (head + 63) // 64 * 64
+    return plane_bytes, head + plane_bytes + keys.num_keys * keys.Sb * 4 + (keys.num_keys * 4 if keys.fixed else 0)
+
+
+def save_keyset_cuda(keyset_cuda_cap, out_dir: str) -> int:
+    """Write a device keyset to ``out_dir/keyset.bsik`` and return the bytes written.  Counterpart of save_keyset
+    (bsiFunctions.cpp:792-808), which writes one bsiCPP ``.hb`` file per key and slice; here one file holds an
+    8-byte magic, the length of a JSON header, the header (padded to 64 bytes), then the packed planes
+    (canonical [R, Sb, W] uint64, 0.75 byte per weight at 6 bits), the slice weights and the row shifts.
+    The int8 image and the tiled planes are derived again on load."""
+    keys = _capsule(keyset_cuda_cap, PrebuiltBSIKeysCUDA, "Invalid CUDA keys capsule")
+    os.makedirs(out_dir, exist_ok=True)
+    head = json.dumps(_keyset_header(keys)).encode()
+    head += b" " * ((-len(head)) % 64)
+    planes = canonical_key_planes(keys).cpu().numpy()
+    path = os.path.join(out_dir, _KEYSET_FILE)
+    with open(path, "wb") as fh:
+        fh.write(_KEYSET_MAGIC)
+        fh.write(len(head).to_bytes(8, "little"))
+        fh.write(head)
+        fh.write(planes.astype("<i8", copy=False).tobytes())
+        fh.write(keys.slice_weights.cpu().numpy().astype("<f4", copy=False).tobytes())
+        if keys.fixed:
+            fh.write(keys.shifts.cpu().numpy().astype("<i4", copy=False).tobytes())
+    return os.path.getsize(path)
+
+
+def load_keyset_cuda(out_dir: str):
+    """Read ``out_dir/keyset.bsik`` back into a device keyset without re-quantising; returns the tuple
+    build_bsi_keys_cuda returns: (handle, total_bytes_of_words, num_keys, d, W)."""
+    import numpy as np
+
+    path = os.path.join(out_dir, _KEYSET_FILE)
+    with open(path, "rb") as fh:
+        _check(fh.read(8) == _KEYSET_MAGIC, f"{path}: not a BSI keyset file")
+        head_len = int.from_bytes(fh.read(8), "little")
+        _check(0 < head_len <= (1 << 20), f"{path}: bad header length")
+        meta = json.loads(fh.read(head_len).decode())
+        _check(meta.get("format") == 1, f"{path}: unknown keyset format {meta.get('format')}")
+        R, d, W, Sb = int(meta["num_keys"]), int(meta["d"]), int(meta["W"]), int(meta["Sb"])
+        _check(R >= 0 and 1 <= Sb <= 64 and W == ((d + 63) // 64 if d > 0 else 1), f"{path}: inconsistent header")
+        planes = np.fromfile(fh, dtype="<i8", count=R * Sb * W)
+        weights = np.fromfile(fh, dtype="<f4", count=R * Sb)
+        shifts = np.fromfile(fh, dtype="<i4", count=R) if meta["fixed"] else None
+        _check(planes.size == R * Sb * W and weights.size == R * Sb and (shifts is None or shifts.size == R),
+               f"{path}: truncated file")
+    dev = _device()
+    h = PrebuiltBSIKeysCUDA()
+    h.num_keys, h.d, h.W, h.Sb = R, d, W, Sb
+    h.decimals, h.threshold, h.fixed = int(meta["decimals"]), float(meta["threshold"]), bool(meta["fixed"])
+    words = torch.from_numpy(planes.reshape(R, Sb, W)).to(dev)
+    h.slice_weights = torch.from_numpy(weights.reshape(R, Sb)).to(dev)
+    if h.fixed:
+        h.shifts = torch.from_numpy(shifts).to(dev)
+        _install_fixed_key_planes(h, words)
+    else:
+        h.words, h.layout = words, _lib.LAYOUT_CANONICAL
+    return h, int(R * Sb * W * 8), R, d, W
 
 
 # --------------------------------------------------------------------------- dot

@@ -7,6 +7,7 @@ planes -> cast to x.dtype -> add bias -> restore the leading shape.
 """
 from __future__ import annotations
 
+import json
 import os
 import time
 from typing import Any, Dict, List, Union
@@ -41,13 +42,31 @@ class BSIQuantizedLinear(nn.Module):
     """Linear layer whose weight lives as BSI key planes (verify_accuracy_bsi.py:46-215)."""
 
     def __init__(self, original_linear, decimalPlaces=2, compress_threshold=0.2, query_threshold=None,
-                 prefer_cuda: bool = True):
+                 prefer_cuda: bool = True, prebuilt_keys=None):
         super().__init__()
         self.decimalPlaces = int(decimalPlaces)
         self.compress_threshold = float(compress_threshold)
         self.query_compress_threshold = float(query_threshold) if query_threshold is not None else float(compress_threshold)
         self.in_features = original_linear.in_features
         self.out_features = original_linear.out_features
+
+        if prebuilt_keys is not None:
+            # keys read back from disk (load_bsi_model): the dense weight of `original_linear` is not looked at
+            self.weight_fp32 = None
+            self.weight_dense_memory_bytes = self.in_features * self.out_features * 4
+            bias = original_linear.bias
+            self.register_buffer("bias", None if bias is None else bias.detach().to(torch.float32))
+            self.bias_fp32 = None if bias is None else self.bias.cpu()
+            self.bias_memory_bytes = 0 if bias is None else self.bias.numel() * 4
+            self._bsi_keys_cuda, total_mem_bytes, num_keys, d, _W = prebuilt_keys
+            assert num_keys == self.out_features and d == self.in_features, "keyset does not fit this layer"
+            assert self._bsi_keys_cuda.decimals == self.decimalPlaces, "keyset was built with other decimal places"
+            self.weight_bsi_memory_bytes = int(total_mem_bytes)
+            self.total_bsi_static_bytes = self.weight_bsi_memory_bytes + self.bias_memory_bytes
+            self.verbose = False
+            self.collect_stats = False
+            self._reset_counters()
+            return
 
         dense_weight = original_linear.weight.detach().to(torch.float32)
         self.weight_fp32 = dense_weight.cpu()
@@ -242,4 +261,55 @@ def quantize_model_bsi(model, decimalPlaces=2, skip_lm_head=True, scope="all", c
             prefer_cuda=prefer_cuda))
     if verbose:
         print(f"Quantized {len(targets)} linear layers to BSI with decimalPlaces={decimalPlaces} (scope={scope})")
+    return model
+
+
+def save_bsi_model(model: nn.Module, out_dir: str) -> List[Dict[str, Any]]:
+    """Write every BSI layer's keyset (and bias) under ``out_dir`` with a ``manifest.json`` holding the fields the
+    reference's save_bsi_model records (verify_accuracy_bsi.py:370-386: name, in, out, decimalPlaces,
+    compress_threshold) plus the file sizes.  One ``keyset.bsik`` per layer instead of one file per key and slice."""
+    os.makedirs(out_dir, exist_ok=True)
+    meta = []
+    for name, module in model.named_modules():
+        if not isinstance(module, BSIQuantizedLinear):
+            continue
+        layer_dir = os.path.join(out_dir, name.replace(".", "_"))
+        nbytes = bsi_ops.save_keyset_cuda(module._bsi_keys_cuda, layer_dir)
+        if module.bias is not None:
+            with open(os.path.join(layer_dir, "bias.f32"), "wb") as fh:
+                fh.write(module.bias.detach().cpu().numpy().astype("<f4", copy=False).tobytes())
+        meta.append({"name": name, "in": module.in_features, "out": module.out_features,
+                     "decimalPlaces": module.decimalPlaces, "compress_threshold": module.compress_threshold,
+                     "dir": os.path.basename(layer_dir), "keyset_bytes": int(nbytes), "has_bias": module.bias is not None})
+    with open(os.path.join(out_dir, "manifest.json"), "w") as f:
+        json.dump(meta, f, indent=2)
+    return meta
+
+
+def load_bsi_model(model: nn.Module, out_dir: str, verbose: bool = False) -> nn.Module:
+    """Replace the ``nn.Linear`` layers named in ``out_dir/manifest.json`` by BSI layers whose keys (and bias) are
+    read from disk: no re-quantisation, and the dense weights of ``model`` are never read for those layers."""
+    import numpy as np
+
+    with open(os.path.join(out_dir, "manifest.json")) as f:
+        meta = json.load(f)
+    for entry in meta:
+        parent = model
+        parts = entry["name"].split(".")
+        for part in parts[:-1]:
+            parent = getattr(parent, part)
+        module = getattr(parent, parts[-1])
+        assert (module.in_features, module.out_features) == (entry["in"], entry["out"]), \
+            f"{entry['name']}: layer shape differs from the saved keyset"
+        layer_dir = os.path.join(out_dir, entry["dir"])
+        shell = nn.Linear(entry["in"], entry["out"], bias=entry["has_bias"], device="meta")
+        if entry["has_bias"]:
+            b = np.fromfile(os.path.join(layer_dir, "bias.f32"), dtype="<f4")
+            assert b.size == entry["out"], f"{entry['name']}: truncated bias file"
+            shell.bias = nn.Parameter(torch.from_numpy(b).cuda(), requires_grad=False)
+        setattr(parent, parts[-1], BSIQuantizedLinear(
+            shell, decimalPlaces=entry["decimalPlaces"], compress_threshold=entry["compress_threshold"],
+            prebuilt_keys=bsi_ops.load_keyset_cuda(layer_dir)))
+    if verbose:
+        print(f"Loaded {len(meta)} BSI layers from {out_dir}")
     return model

@@ -189,3 +189,14 @@ def test_set_option_validates_on_host():
     assert _lib.lib.bsi_hip_set_option(_lib.OPT_I8_TILE, 0) == 0
     assert _lib.lib.bsi_hip_set_option(999, 1) == 1
     assert b"unknown option" in _lib.lib.bsi_hip_last_error()
+
+
+def test_load_keyset_refuses_foreign_files_before_touching_the_device(tmp_path):
+    from bsipytorch_amd import bsi_ops
+
+    (tmp_path / "keyset.bsik").write_bytes(b"something else entirely")
+    with pytest.raises(RuntimeError, match="not a BSI keyset file"):
+        bsi_ops.load_keyset_cuda(str(tmp_path))
+    (tmp_path / "keyset.bsik").write_bytes(b"BSIKEYS1" + (1 << 40).to_bytes(8, "little"))
+    with pytest.raises(RuntimeError, match="bad header length"):
+        bsi_ops.load_keyset_cuda(str(tmp_path))

@@ -1022,3 +1022,75 @@ def test_linear_drop_in_decimal_mode(ops, monkeypatch):
     assert (got - ref).abs().max().item() < 512 * 0.0005 * 5.0
     cos = torch.nn.functional.cosine_similarity(got.flatten(), ref.flatten(), dim=0).item()
     assert cos > 0.9999
+
+
+# ------------------------------------------------------------------ keyset files
+
+
+@pytest.mark.parametrize("mode", ["fixed-tiled", "fixed-canonical", "decimal"])
+def test_keyset_file_round_trip(ops, oracle, monkeypatch, tmp_path, mode):
+    """save_keyset_cuda / load_keyset_cuda: the planes on disk are the oracle's canonical planes, and the loaded
+    keyset gives bit-identical dot outputs without re-quantising."""
+    if mode == "fixed-canonical":
+        monkeypatch.setenv("BSI_KEY_LAYOUT", "canonical")
+    if mode == "decimal":
+        monkeypatch.setenv("BSI_FIXED_BITS_KEYS", "0")
+        monkeypatch.setenv("BSI_FIXED_CHUNK_SCALE", "0")
+    ops._reset_flag_cache()
+    R, d = 70, 1100  # ragged: 18 words per slice, 5 key tiles of 16
+    rng = np.random.default_rng(8)
+    k = (rng.standard_normal((R, d)) * 0.02).astype(np.float32)
+    x = rng.standard_normal((40, d)).astype(np.float32)
+    kcap, nbytes, *_ = ops.build_bsi_keys_cuda(torch.from_numpy(k), 2, 0.5)
+    want = oracle.build_decimal(k, 2) if mode == "decimal" else oracle.build_keys(k, 2, 6)
+    assert np.array_equal(host_u64(ops.canonical_key_planes(kcap)), want["words"])
+    written = ops.save_keyset_cuda(kcap, str(tmp_path / "layer"))
+    mem, disk = ops.keyset_size_on_disk_cuda(kcap)
+    assert written == disk and mem == nbytes == want["words"].size * 8
+    assert disk < mem + R * want["words"].shape[1] * 4 + R * 4 + 1024
+    loaded, nbytes2, nk, d2, W = ops.load_keyset_cuda(str(tmp_path / "layer"))
+    assert (nbytes2, nk, d2, W) == (nbytes, R, d, 18)
+    assert (loaded.Sb, loaded.decimals, loaded.fixed, loaded.layout) == (kcap.Sb, 2, kcap.fixed, kcap.layout)
+    assert torch.equal(loaded.words, kcap.words) and torch.equal(loaded.slice_weights, kcap.slice_weights)
+    if kcap.fixed:
+        assert torch.equal(loaded.shifts, kcap.shifts) and torch.equal(loaded.ints8, kcap.ints8)
+    qcap = ops.build_bsi_queries_cuda_batch_packed(torch.from_numpy(x).cuda(), 2, 0.5)
+    a, *_ = ops.batch_dot_product_multiquery_cuda_batch_caps(qcap, kcap)
+    b, *_ = ops.batch_dot_product_multiquery_cuda_batch_caps(qcap, loaded)
+    assert torch.equal(a, b)
+    # damaged files are refused
+    path = tmp_path / "layer" / "keyset.bsik"
+    raw = path.read_bytes()
+    path.write_bytes(raw[:-100])
+    with pytest.raises(RuntimeError, match="truncated"):
+        ops.load_keyset_cuda(str(tmp_path / "layer"))
+    path.write_bytes(b"NOTAKEYS" + raw[8:])
+    with pytest.raises(RuntimeError, match="not a BSI keyset file"):
+        ops.load_keyset_cuda(str(tmp_path / "layer"))
+
+
+def test_save_and_load_bsi_model(ops, tmp_path):
+    from bsipytorch_amd import linear
+
+    torch.manual_seed(2)
+
+    def make():
+        return torch.nn.Sequential(torch.nn.Linear(512, 256), torch.nn.ReLU(), torch.nn.Linear(256, 64, bias=False)).cuda()
+
+    model = make()
+    linear.quantize_model_bsi(model, decimalPlaces=2, compress_threshold=0.5, verbose=False)
+    x = torch.randn(33, 512, device="cuda")
+    with torch.no_grad():
+        want = model(x)
+    meta = linear.save_bsi_model(model, str(tmp_path / "m"))
+    assert [m["name"] for m in meta] == ["0", "2"] and meta[0]["has_bias"] and not meta[1]["has_bias"]
+    saved = json.load(open(tmp_path / "m" / "manifest.json"))
+    assert saved[0]["in"] == 512 and saved[0]["out"] == 256 and saved[0]["decimalPlaces"] == 2
+    # 6 planes of 512 bits per row = 0.75 byte per weight, plus weights, shifts and the header
+    assert saved[0]["keyset_bytes"] < 512 * 256 * 0.75 + 256 * 6 * 4 + 256 * 4 + 1024
+    other = make()  # different random weights: the loaded layers must not depend on them
+    linear.load_bsi_model(other, str(tmp_path / "m"))
+    assert isinstance(other[0], linear.BSIQuantizedLinear) and other[0].weight_fp32 is None
+    with torch.no_grad():
+        got = other(x)
+    assert torch.equal(got, want)
