@@ -723,46 +723,39 @@ struct I8Cfg {
     static constexpr int kLds = 4 * kStage + kScaleBytes;
 };
 
-// One half-chunk (two k-steps) of an MFMA wave: 2 WM WN MFMAs into `acc`, 2 (WM + WN) operand
-// reads, and as many epilogue elements of the previous chunk (held in `prev`) as MFMAs.
-// kHalf: first or second half of the chunk.
-template <int WM, int WN, int kHalf, bool kInts>
-__device__ __forceinline__ void i8_consume_half(const unsigned char* __restrict__ krow,
-                                                const unsigned char* __restrict__ qrow, const int (&pcol)[2],
-                                                v4i (&acc)[WM][WN], const v4i (&prev)[WM][WN],
-                                                float (&accf)[WM][WN][4], const float (&qs_prev)[WN],
-                                                int* __restrict__ ints_prev, const int64_t (&int_off)[WM][WN],
-                                                const int (&int_rows)[WM], int down_shift, int chunks) {
+// One k-step (64 of a chunk's 256 elements) of an MFMA wave: WM WN MFMAs on the operands in (ka, qb), one
+// epilogue element of the previous chunk (held in `prev`) behind each MFMA, and behind the first WM + WN of them
+// the reads of the NEXT k-step's operands into (ka_n, qb_n), so that the LDS latency of every k-step hides
+// behind the MFMAs of the one before it -- also across the barrier between two stages of the ring.
+// KS: k-step of the chunk (0..3); krow_n / qrow_n: the wave's rows of the next k-step's stage, column included.
+template <int WM, int WN, int KS, bool kInts>
+__device__ __forceinline__ void i8_kstep(const v4i (&ka)[WM], const v4i (&qb)[WN], v4i (&ka_n)[WM], v4i (&qb_n)[WN],
+                                         const unsigned char* __restrict__ krow_n,
+                                         const unsigned char* __restrict__ qrow_n, v4i (&acc)[WM][WN],
+                                         const v4i (&prev)[WM][WN], float (&accf)[WM][WN][4],
+                                         const float (&qs_prev)[WN], int* __restrict__ ints_prev,
+                                         const int64_t (&int_off)[WM][WN], const int (&int_rows)[WM], int down_shift,
+                                         int chunks) {
     static_assert(WM + WN <= WM * WN, "one operand read behind each MFMA of a k-step");
-    v4i ka[2][WM], qb[2][WN];
-    // read number t of a k-step, in the order its MFMAs first need them: ka[0], qb[0..], ka[1..]
-    auto read = [&](int set, int t) {
-        if (t == 0) ka[set][0] = *reinterpret_cast<const v4i*>(krow + pcol[set]);
-        else if (t <= WN) qb[set][t - 1] = *reinterpret_cast<const v4i*>(qrow + (t - 1) * 16 * 128 + pcol[set]);
-        else ka[set][t - WN] = *reinterpret_cast<const v4i*>(krow + (t - WN) * 16 * 128 + pcol[set]);
-    };
 #pragma unroll
-    for (int t = 0; t < WM + WN; ++t) read(0, t);
-    __builtin_amdgcn_sched_barrier(0);
+    for (int a = 0; a < WM; ++a)
 #pragma unroll
-    for (int kk = 0; kk < 2; ++kk) {
-#pragma unroll
-        for (int a = 0; a < WM; ++a)
-#pragma unroll
-            for (int b = 0; b < WN; ++b) {
-                const int ks = kHalf * 2 + kk, t = a * WN + b;
-                const v4i c0 = (ks == 0) ? (v4i){0, 0, 0, 0} : acc[a][b];
-                acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ka[kk][a], qb[kk][b], c0, 0, 0, 0);
-                {
-                    const int idx = ks * (WM * WN) + t, tt = idx >> 2, e = idx & 3, ea = tt / WN, eb = tt % WN;
-                    accf[ea][eb][e] = fmaf(static_cast<float>(prev[ea][eb][e]), qs_prev[eb], accf[ea][eb][e]);
-                    if (kInts && ints_prev != nullptr && int_off[ea][eb] >= 0 && e < int_rows[ea])
-                        ints_prev[int_off[ea][eb] + static_cast<int64_t>(e) * chunks] = prev[ea][eb][e] >> down_shift;
-                }
-                if (kk == 0 && t < WM + WN) read(1, t);  // operands of the second k-step
-                __builtin_amdgcn_sched_barrier(0);
+        for (int b = 0; b < WN; ++b) {
+            const int t = a * WN + b;
+            const v4i c0 = (KS == 0) ? (v4i){0, 0, 0, 0} : acc[a][b];
+            acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ka[a], qb[b], c0, 0, 0, 0);
+            {
+                const int idx = KS * (WM * WN) + t, tt = idx >> 2, e = idx & 3, ea = tt / WN, eb = tt % WN;
+                accf[ea][eb][e] = fmaf(static_cast<float>(prev[ea][eb][e]), qs_prev[eb], accf[ea][eb][e]);
+                if (kInts && ints_prev != nullptr && int_off[ea][eb] >= 0 && e < int_rows[ea])
+                    ints_prev[int_off[ea][eb] + static_cast<int64_t>(e) * chunks] = prev[ea][eb][e] >> down_shift;
             }
-    }
+            // read number t of the next k-step, in the order its MFMAs first need them: ka[0], qb[0..], ka[1..]
+            if (t == 0) ka_n[0] = *reinterpret_cast<const v4i*>(krow_n);
+            else if (t <= WN) qb_n[t - 1] = *reinterpret_cast<const v4i*>(qrow_n + (t - 1) * 16 * 128);
+            else if (t < WM + WN) ka_n[t - WN] = *reinterpret_cast<const v4i*>(krow_n + (t - WN) * 16 * 128);
+            __builtin_amdgcn_sched_barrier(0);
+        }
 }
 
 template <int TM, int TN, bool kInts>
@@ -889,34 +882,53 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
         _Pragma("unroll") for (int b = 0; b < WN; ++b) dst[b] =                                                \
             *reinterpret_cast<const float*>(sread + ((c) & 3) * (C::kLoaders * 256) + b * 64);                 \
     }
-#define BSI_I8_HALF(kHalf, slot, acc, prev, qs, ip)                                                                  \
-    i8_consume_half<WM, WN, kHalf, kInts>(lds + (slot) * C::kStage + krow_off, lds + (slot) * C::kStage + qrow_off,  \
-                                          pcol, acc, prev, accf, qs, ip, int_off, int_rows, down_shift, chunks);     \
-    lds_barrier();
+    // The k-steps run one behind their operand reads: k-step j's MFMAs cover the reads of k-step j + 1.  A
+    // stage (half-chunk, two k-steps) is released to the loaders by the barrier that follows the k-step in
+    // which its last operands were read (the even ones); the same barrier tells that the next stage has landed.
+    v4i ka[2][WM], qb[2][WN];  // operand sets of even / odd k-steps
+#define BSI_I8_KSTEP(KS, nslot, acc, prev, qs, ip)                                                                  \
+    i8_kstep<WM, WN, KS, kInts>(ka[(KS) & 1], qb[(KS) & 1], ka[((KS) + 1) & 1], qb[((KS) + 1) & 1],                 \
+                                lds + (nslot) * C::kStage + krow_off + pcol[((KS) + 1) & 1],                        \
+                                lds + (nslot) * C::kStage + qrow_off + pcol[((KS) + 1) & 1], acc, prev, accf, qs,   \
+                                ip, int_off, int_rows, down_shift, chunks);
+    // a chunk whose halves sit in ring slots s0, s0 + 1; nslot: slot of the next chunk's first half
+#define BSI_I8_CHUNK(s0, nslot, acc, prev, qs, ip)                                                                  \
+    BSI_I8_KSTEP(0, s0, acc, prev, qs, ip);                                                                         \
+    lds_barrier();                                                                                                  \
+    BSI_I8_KSTEP(1, (s0) + 1, acc, prev, qs, ip);                                                                   \
+    BSI_I8_KSTEP(2, (s0) + 1, acc, prev, qs, ip);                                                                   \
+    lds_barrier();                                                                                                  \
+    BSI_I8_KSTEP(3, nslot, acc, prev, qs, ip);
 
     lds_barrier();  // stage 0 is there
+#pragma unroll
+    for (int t = 0; t < WM; ++t) ka[0][t] = *reinterpret_cast<const v4i*>(lds + krow_off + t * 16 * 128 + pcol[0]);
+#pragma unroll
+    for (int t = 0; t < WN; ++t) qb[0][t] = *reinterpret_cast<const v4i*>(lds + qrow_off + t * 16 * 128 + pcol[0]);
+    __builtin_amdgcn_sched_barrier(0);
     int c = 0;
     for (; c + 1 < chunks; c += 2) {
         int* const ip = c > 0 ? chunk_ints + (c - 1) : nullptr;
         // even chunk c -> acc0, ring slots 0 and 1; epilogue of chunk c-1 (acc1, scales qsb)
-        BSI_I8_HALF(0, 0, acc0, acc1, qsb, ip);
-        BSI_I8_HALF(1, 1, acc0, acc1, qsb, ip);
+        BSI_I8_CHUNK(0, 2, acc0, acc1, qsb, ip);
         BSI_I8_SCALES(qsa, c);  // landed with the second half of chunk c
         // odd chunk c+1 -> acc1, ring slots 2 and 3; epilogue of chunk c (acc0, scales qsa)
-        BSI_I8_HALF(0, 2, acc1, acc0, qsa, chunk_ints + c);
-        BSI_I8_HALF(1, 3, acc1, acc0, qsa, chunk_ints + c);
+        BSI_I8_CHUNK(2, 0, acc1, acc0, qsa, chunk_ints + c);
         BSI_I8_SCALES(qsb, c + 1);
     }
     bool last_in_acc0 = false;
     if (c < chunks) {  // odd number of chunks: one more even chunk; its halves sit in slots 0 and 1
         int* const ip = c > 0 ? chunk_ints + (c - 1) : nullptr;
-        BSI_I8_HALF(0, 0, acc0, acc1, qsb, ip);
-        BSI_I8_HALF(1, 1, acc0, acc1, qsb, ip);
+        BSI_I8_CHUNK(0, 2, acc0, acc1, qsb, ip);
         BSI_I8_SCALES(qsa, c);
         last_in_acc0 = true;
     }
+    // the last k-step read ahead into a stage that does not exist (the loaders fill it with a copy of the last
+    // one); nothing uses those operands
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#undef BSI_I8_CHUNK
+#undef BSI_I8_KSTEP
 #undef BSI_I8_SCALES
-#undef BSI_I8_HALF
     // epilogue of the last chunk
 #pragma unroll
     for (int a = 0; a < WM; ++a)
