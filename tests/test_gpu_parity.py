@@ -1094,3 +1094,45 @@ def test_save_and_load_bsi_model(ops, tmp_path):
     with torch.no_grad():
         got = other(x)
     assert torch.equal(got, want)
+
+
+# ------------------------------------------------------------------ empty and degenerate inputs
+
+
+@pytest.mark.parametrize("bits", ["fixed", "decimal"])
+def test_empty_and_degenerate_inputs(ops, hip, monkeypatch, bits):
+    """Zero rows, zero columns, a single element: builders return well-formed handles, the dot refuses empty
+    operands with the reference's messages (bsi_cuda.cpp:672-682), and the raw entry points accept zero sizes."""
+    if bits == "decimal":
+        monkeypatch.setenv("BSI_FIXED_BITS", "0")
+        ops._reset_flag_cache()
+    L = hip.lib
+    kcap, nbytes, nk, d, W = ops.build_bsi_keys_cuda(torch.randn(5, 64), 2, 0.2)
+    q0 = ops.build_bsi_queries_cuda_batch_packed(torch.zeros((0, 64)).cuda(), 2, 0.2)
+    assert q0.Q == 0 and q0.words.shape[0] == 0 and q0.W == 1
+    with pytest.raises(RuntimeError, match="Empty query batch"):
+        ops.batch_dot_product_multiquery_cuda_batch_caps(q0, kcap)
+    k0, nb0, nk0, d0, W0 = ops.build_bsi_keys_cuda(torch.zeros((0, 64)), 2, 0.2)
+    assert (nb0, nk0, d0, W0) == (0, 0, 64, 1)
+    q1 = ops.build_bsi_queries_cuda_batch_packed(torch.randn(3, 64).cuda(), 2, 0.2)
+    with pytest.raises(RuntimeError, match="Empty keys"):
+        ops.batch_dot_product_multiquery_cuda_batch_caps(q1, k0)
+    with pytest.raises(RuntimeError, match="Empty keys or queries"):
+        ops.batch_dot_product_multiquery_cuda_caps([], kcap)
+    # one element per row
+    k1, *_ = ops.build_bsi_keys_cuda(torch.tensor([[0.25], [-0.5]]), 2, 0.2)
+    qq = ops.build_bsi_queries_cuda_batch_packed(torch.tensor([[2.0], [-1.0], [0.0]]).cuda(), 2, 0.2)
+    out, *_ = ops.batch_dot_product_multiquery_cuda_batch_caps(qq, k1)
+    assert torch.allclose(out.cpu(), torch.tensor([[0.5, -1.0], [-0.25, 0.5], [0.0, 0.0]]), atol=1e-6)
+    # all-zero operands
+    kz, *_ = ops.build_bsi_keys_cuda(torch.zeros((4, 256)), 2, 0.2)
+    qz = ops.build_bsi_queries_cuda_batch_packed(torch.zeros((2, 256)).cuda(), 2, 0.2)
+    out, *_ = ops.batch_dot_product_multiquery_cuda_batch_caps(qz, kz)
+    assert not out.any() and out.shape == (2, 4)
+    # raw entry points: zero sizes are accepted without touching the pointers
+    assert L.bsi_hip_build_fixed(None, hip.DTYPE_F32, 0, 64, 2, 7, 1, 0.0, None, None, None, None, st()) == 0
+    assert L.bsi_hip_pack_bits_batch(None, 0, 64, 7, 1, None, st()) == 0
+    assert L.bsi_hip_dot(None, None, None, 1, 7, 1, None, 0, None, 6, 0, 4, 1.0, 0, None, None, 0, None, 0, st()) == 0
+    assert L.bsi_hip_dot_weighted(None, None, 7, 1, None, 0, None, 6, 0, 4, None, 1.0, 0, None, st()) == 0
+    m = torch.full((1,), 9, dtype=torch.int64, device="cuda")
+    assert L.bsi_hip_decimal_stats(None, 0, 64, m.data_ptr(), None, st()) == 0 and int(m.item()) == 0
