@@ -72,7 +72,10 @@ def _run_weighted(qcap, kcap, Q, R, D, W, key_bytes, warmup, iters):
     t = e0.elapsed_time(e1) * 1e-3 / iters
     bit_ops = 2.0 * qcap.Sa * kcap.Sb * Q * R * D
     alg_bytes = Q * qcap.Sa * W * 8 + R * kcap.Sb * W * 8 + (Q * qcap.Sa + R * kcap.Sb) * 4 + Q * R * 4
-    return {"Q": Q, "R": R, "D": D, "core": "weighted", "layout": "canonical" if kcap.layout == 0 else "tiled16",
+    on_mfma = (getattr(qcap, "digits8", None) is not None or (qcap.fixed and qcap.ints8 is not None)) and \
+              (getattr(kcap, "digits8", None) is not None or (kcap.fixed and kcap.ints8 is not None))
+    return {"Q": Q, "R": R, "D": D, "core": "int8 digits on MFMA" if on_mfma else "weighted popcount (VALU)",
+            "layout": "canonical" if kcap.layout == 0 else "tiled16",
             "Sa": qcap.Sa, "Sb": kcap.Sb, "avg_dot_us": t * 1e6, "dot_q_us": t * 1e6 / Q, "dot_s_ns": t * 1e9 / (Q * R),
             "effective_bitop_TOPS": bit_ops / t / 1e12, "popcount_word_ops_per_s": qcap.Sa * kcap.Sb * Q * R * W / t,
             "algorithmic_GBps": alg_bytes / t / 1e9, "key_plane_GBps": key_bytes / t / 1e9, "iters": iters}

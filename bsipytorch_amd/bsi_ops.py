@@ -81,6 +81,7 @@ def _flags() -> dict:
         tiled=(layout != "canonical"),
         key_image=(_env_int("BSI_KEY_INT8_IMAGE", 1) or 0) != 0,
         ewah_inline=(_env_int("BSI_EWAH_INLINE", 1) or 0) != 0,
+        decimal_mfma=(_env_int("BSI_DECIMAL_MFMA", 1) or 0) != 0,
     )
     return _flag_cache
 
@@ -150,6 +151,7 @@ class PrebuiltBSIKeysCUDA(_Capsule):
         self.slice_weights: torch.Tensor = None  # [R, Sb] float32
         self.shifts: torch.Tensor = None         # [R] int32 (fixed-bit keys only)
         self.fixed = True                        # False: decimal-mode keys (slice count from the data, canonical planes)
+        self.digits8: Optional[torch.Tensor] = None  # decimal keys: int8 digit images [ceil(Sb/7), R, chunks*256]
         self.Sb = 0
         self.W = 0
         self.d = 0
@@ -170,6 +172,7 @@ class PrebuiltBSIQueryBatchCUDA(_Capsule):
         self.row_scales: Optional[torch.Tensor] = None    # [Q] float32 when there are no chunk scales
         self.ints8: Optional[torch.Tensor] = None         # [Q, chunks*256] int8 (MFMA operand) or None
         self.fixed = True                                 # False: decimal-mode batch (no scales; weighted-slice dot)
+        self.digits8: Optional[torch.Tensor] = None       # decimal batch: int8 digit images [ceil(Sa/7), Q, chunks*256]
         self.Sa = 0
         self.W = 0
         self.decimals = 0
@@ -189,6 +192,7 @@ class PrebuiltBSIQueryCUDA(_Capsule):
         self.row_scale: Optional[torch.Tensor] = None     # [] when no chunk scales
         self.ints8: Optional[torch.Tensor] = None         # [chunks*256]
         self.fixed = True                                 # False: decimal-mode row (no scale)
+        self.digits8: Optional[torch.Tensor] = None       # decimal row: int8 digit images [ceil(S/7), chunks*256]
         self.S = 0
         self.W = 0
         self.rows = 0
@@ -310,6 +314,22 @@ def _build_decimal(x2d: torch.Tensor, decimal_places: int):
     return words, weights, S, negative
 
 
+_MAX_DIGIT_PAIRS = 9  # above this the digit GEMM does more work than the popcount kernel saves
+
+
+def _digit_images(words: torch.Tensor) -> Optional[torch.Tensor]:
+    """int8 digit images [ceil(S/7), rows, chunks*256] of decimal-mode planes [rows, S, W] for the matrix cores
+    (bsi_hip_planes_to_int8_digits), or None when the flag is off, the operand is empty or a row has more than
+    2^17 elements (the int32 sums of the digit products could overflow)."""
+    rows, S, W = words.shape
+    if not _flags()["decimal_mfma"] or rows == 0 or W > 2048:
+        return None
+    out = torch.empty(((S + 6) // 7, rows, ((W + 3) // 4) * 256), dtype=torch.int8, device=words.device)
+    check(lib.bsi_hip_planes_to_int8_digits(words.data_ptr(), rows, S, W, out.data_ptr(), _stream()),
+          "bsi_hip_planes_to_int8_digits")
+    return out
+
+
 _expanded_cache: dict = {}
 
 
@@ -349,6 +369,7 @@ def _build_query_batch(q2d: torch.Tensor, decimal_places: int) -> PrebuiltBSIQue
             _last_build_profile[:] = [0, 0, 0]
         h = PrebuiltBSIQueryBatchCUDA()
         h.words, h.slice_weights, h.fixed = words, weights, False
+        h.digits8 = _digit_images(words) if S <= 7 * _MAX_DIGIT_PAIRS else None
         h.Sa, h.W, h.decimals, h.Q = S, W, int(decimal_places), Q
         h.mem_bytes = words.numel() * 8 + weights.numel() * 4
         if f["debug"]:
@@ -401,6 +422,7 @@ def build_bsi_queries_cuda_batch(q2d: torch.Tensor, decimal_places: int, compres
         h.dev_words = b.words[qi]
         h.slice_weights = b.slice_weights[qi]
         h.fixed = b.fixed
+        h.digits8 = b.digits8[:, qi] if b.digits8 is not None else None
         if b.chunk_scales is not None and b.chunk_scales.numel() > 0:
             h.chunk_scales = b.chunk_scales[qi]
         elif b.row_scales is not None:
@@ -424,6 +446,8 @@ def _build_query_1d(q: torch.Tensor, decimal_places: int) -> PrebuiltBSIQueryCUD
         h = PrebuiltBSIQueryCUDA()
         h.S, h.W, h.dev_words, h.rows, h.decimals, h.fixed = S, words.shape[2], words[0], x.shape[1], int(decimal_places), False
         h.twos_complement = bool(neg[0].item()) if x.shape[1] > 0 else False
+        d8 = _digit_images(words) if S <= 7 * _MAX_DIGIT_PAIRS else None
+        h.digits8 = d8[:, 0] if d8 is not None else None
         h.slice_weights = weights[0]
         h.mem_bytes = h.dev_words.numel() * 8
         return h
@@ -544,6 +568,7 @@ def build_bsi_keys_cuda(K: torch.Tensor, decimal_places: int, compress_threshold
         h.num_keys, h.d, h.W, h.Sb, h.fixed = int(R), int(d), words.shape[2], S, False
         h.decimals, h.threshold = int(decimal_places), float(compress_threshold)
         h.words, h.layout, h.slice_weights = words, _lib.LAYOUT_CANONICAL, weights
+        h.digits8 = _digit_images(words) if S <= 7 * _MAX_DIGIT_PAIRS else None
         if f["debug"]:
             print(f"[BSI_HIP] build_bsi_keys_cuda (decimal): R={R} slices={S} words_per_slice={h.W}")
         return h, int(words.numel() * 8), int(R), int(d), int(h.W)
@@ -639,6 +664,7 @@ def load_keyset_cuda(out_dir: str):
         _install_fixed_key_planes(h, words)
     else:
         h.words, h.layout = words, _lib.LAYOUT_CANONICAL
+        h.digits8 = _digit_images(words) if Sb <= 7 * _MAX_DIGIT_PAIRS else None
     return h, int(R * Sb * W * 8), R, d, W
 
 
@@ -718,22 +744,46 @@ def _dot(words, ints8, scales, scale_stride, Sa, W, keys: PrebuiltBSIKeysCUDA, Q
     return out, ns
 
 
-def _dot_weighted(words, slice_weights, Sa, W, keys: PrebuiltBSIKeysCUDA, Q, decimals_q, bias=None):
-    """The weighted-slice dot (bsi_hip_dot_weighted): any operand pair that is not fixed-bit on both sides."""
+def _dot_weighted(words, slice_weights, Sa, W, keys: PrebuiltBSIKeysCUDA, Q, decimals_q, bias=None, q_digits=None,
+                  q_image=None):
+    """The weighted-slice dot: any operand pair that is not fixed-bit on both sides.  With int8 digit images on
+    both sides (``q_digits`` [nq, Q, chunks*256] or the int8 image ``q_image`` of fixed-bit queries, pre-shifted by
+    8 - Sa; the keys' own digits, or the int8 image of fixed-bit keys) it
+    runs as one int8 GEMM on the matrix cores (bsi_hip_dot_digits), else on the popcount kernel
+    (bsi_hip_dot_weighted); both give the exact sum rounded once, so the results are bit-identical."""
     f = _flags()
     R = keys.num_keys
     out = torch.empty((Q, R), dtype=torch.float32, device=words.device)
     Aw = slice_weights if slice_weights.is_contiguous() else slice_weights.contiguous()
+    k_digits, nk, preshift = None, 0, 0
+    if q_digits is None and q_image is not None and 2 <= Sa <= 8:
+        q_digits, preshift = q_image.unsqueeze(0), 8 - int(Sa)
+    if keys.fixed and keys.ints8 is not None:
+        k_digits, nk, preshift = keys.ints8, 1, preshift + 8 - keys.Sb
+    elif not keys.fixed and keys.digits8 is not None:
+        k_digits, nk = keys.digits8, int(keys.digits8.shape[0])
+    use_digits = (f["decimal_mfma"] and f["core"] != _lib.CORE_VALU and q_digits is not None and k_digits is not None
+                  and int(q_digits.shape[0]) * nk <= _MAX_DIGIT_PAIRS and W <= 2048)
     prof = f["profile"]
     if prof:
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
-    check(lib.bsi_hip_dot_weighted(words.data_ptr(), Aw.data_ptr(), int(Sa), int(W), keys.words.data_ptr(), keys.layout,
-                                   keys.slice_weights.data_ptr(), keys.Sb, R, Q, None,
-                                   _scale_inv(decimals_q, keys.decimals), R, out.data_ptr(), _stream()),
-          "bsi_hip_dot_weighted")
-    if bias is not None:
-        out += bias
+    if use_digits:
+        nq = int(q_digits.shape[0])
+        qd = q_digits if q_digits.is_contiguous() else q_digits.contiguous()
+        ws_bytes = int(lib.bsi_hip_dot_digits_workspace_bytes(Q, nq, R, nk))
+        ws = _get_workspace(ws_bytes, words.device)
+        check(lib.bsi_hip_dot_digits(qd.data_ptr(), nq, Aw.data_ptr(), int(Sa), k_digits.data_ptr(), nk, preshift,
+                                     keys.slice_weights.data_ptr(), keys.Sb, int(W), R, Q, None,
+                                     _scale_inv(decimals_q, keys.decimals), R, _ptr(bias), out.data_ptr(),
+                                     ws.data_ptr(), ws_bytes, _stream()), "bsi_hip_dot_digits")
+    else:
+        check(lib.bsi_hip_dot_weighted(words.data_ptr(), Aw.data_ptr(), int(Sa), int(W), keys.words.data_ptr(),
+                                       keys.layout, keys.slice_weights.data_ptr(), keys.Sb, R, Q, None,
+                                       _scale_inv(decimals_q, keys.decimals), R, out.data_ptr(), _stream()),
+              "bsi_hip_dot_weighted")
+        if bias is not None:
+            out += bias
     ns = 0
     if prof:
         e1.record()
@@ -741,7 +791,8 @@ def _dot_weighted(words, slice_weights, Sa, W, keys: PrebuiltBSIKeysCUDA, Q, dec
         ns = int(e0.elapsed_time(e1) * 1.0e6)
     if f["dot_debug"] and not _DOT_DEBUG_PRINTED[0]:
         _DOT_DEBUG_PRINTED[0] = True
-        print(f"[BSI_DOT] core=weighted Sa={Sa} Sb={keys.Sb} Q={Q} R={R} W64={W} layout={keys.layout}", file=sys.stderr)
+        print(f"[BSI_DOT] core={'digits-mfma' if use_digits else 'weighted-valu'} Sa={Sa} Sb={keys.Sb} Q={Q} R={R} "
+              f"W64={W} layout={keys.layout}", file=sys.stderr)
     return out, ns
 
 
@@ -790,7 +841,9 @@ def batch_dot_product_multiquery_cuda_batch_caps(query_batch_cap, keyset_cuda_ca
     else:
         # a decimal-mode operand on either side: its slice weights carry everything, per-chunk scales cannot apply
         _check(not have_chunk_scales, "chunk-scaled queries need fixed-bit keys (BSI_FIXED_BITS_KEYS > 0)")
-        out, ns = _dot_weighted(qb.words, qb.slice_weights, int(Sa), int(W), keys, int(Q), qb.decimals, bias=bias)
+        out, ns = _dot_weighted(qb.words, qb.slice_weights, int(Sa), int(W), keys, int(Q), qb.decimals, bias=bias,
+                                q_digits=qb.digits8 if not qb.fixed else None,
+                                q_image=qb.ints8 if qb.fixed else None)
     return _dot_result(out, ns, Q, R)
 
 
@@ -820,7 +873,10 @@ def batch_dot_product_multiquery_cuda_caps(query_caps_list, keyset_cuda_cap):
         _check(q0.decimals == keys.decimals, f"Decimal mismatch between queries and keys: q={q0.decimals} k={keys.decimals}")
         words = torch.stack([q.dev_words for q in rows]).contiguous()
         weights = torch.stack([q.slice_weights for q in rows]).contiguous()
-        out, ns = _dot_weighted(words, weights, q0.S, keys.W, keys, Q, q0.decimals)
+        digits = None
+        if not q0.fixed and all(q.digits8 is not None for q in rows):
+            digits = torch.stack([q.digits8 for q in rows], dim=1).contiguous()
+        out, ns = _dot_weighted(words, weights, q0.S, keys.W, keys, Q, q0.decimals, q_digits=digits)
         return _dot_result(out, ns, Q, R)
     if (Q == 1 and getattr(q0, "comp_words", None) is not None and q0.comp_words.numel() > 0 and f["ewah_inline"]
             and keys.layout == _lib.LAYOUT_TILED16 and keys.Sb == 6 and 2 <= q0.S <= 8

@@ -120,6 +120,56 @@ __global__ void planes_to_int8_kernel(const uint32_t* __restrict__ words32, int6
     dst[1] = make_uint4(y[4], y[5], y[6], y[7]);
 }
 
+// Planes of two's-complement values of any width -> int8 digit images for the matrix cores:
+// value = sum_j digit_j * 128^j with digits 0 .. n-2 the unsigned 7-bit groups of planes and digit n-1 the
+// remaining top planes, sign-extended.  out[j][row][chunks * 256] in the same in-chunk element order as
+// planes_to_int8_kernel (no pre-shift).  One thread per (digit, row, 32-bit column).
+__global__ void planes_to_digits_kernel(const uint32_t* __restrict__ words32, int64_t rows, int S, int W64, int chunks,
+                                        int ndig, uint32_t* __restrict__ out32) {
+    const int cols = chunks * 8;
+    const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= static_cast<int64_t>(ndig) * rows * cols) return;
+    const int col = static_cast<int>(idx % cols);
+    const int64_t t = idx / cols;
+    const int64_t row = t % rows;
+    const int j = static_cast<int>(t / rows);
+    const bool top = (j == ndig - 1);
+    uint32_t y[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+        int plane = 7 * j + s;
+        if (top && plane >= S) plane = S - 1;  // sign extension of the top digit
+        const bool have = (s < 7 || top) && plane < S && col < 2 * W64;
+        y[s] = have ? words32[(static_cast<size_t>(row) * S + plane) * (2 * W64) + col] : 0u;
+    }
+    transpose8x8(y);
+    uint4* dst = reinterpret_cast<uint4*>(out32 + (static_cast<size_t>(t) * cols + col) * 8);
+    dst[0] = make_uint4(y[0], y[1], y[2], y[3]);
+    dst[1] = make_uint4(y[4], y[5], y[6], y[7]);
+}
+
+// out[q, idx[r]] = float(sum_{i,j} I[i Q + q, j R + r] * 2^(7 (i + j) - preshift) * Aw[q, 0] * Bw[r, 0]) * scale_inv
+// (+ bias[r]): the digit products of the int32 GEMM put back together, exactly, in float64.
+__global__ void digits_combine_kernel(const int* __restrict__ I, int nq, int nk, int64_t Q, int64_t R, int preshift,
+                                      const float* __restrict__ Aw, int Sa, const float* __restrict__ Bw, int Sb,
+                                      const long long* __restrict__ key_indices, float scale_inv, int64_t R_total,
+                                      const float* __restrict__ bias, float* __restrict__ out) {
+    const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= Q * R) return;
+    const int64_t q = idx / R, r = idx - q * R;
+    const int64_t ld = static_cast<int64_t>(nk) * R;
+    double acc = 0.0;
+    for (int i = 0; i < nq; ++i)
+        for (int j = 0; j < nk; ++j)
+            acc += ldexp(static_cast<double>(I[(static_cast<int64_t>(i) * Q + q) * ld + static_cast<int64_t>(j) * R + r]),
+                         7 * (i + j) - preshift);
+    acc = acc * static_cast<double>(Aw[q * Sa]) * static_cast<double>(Bw[r * Sb]);
+    const int64_t col = key_indices ? key_indices[r] : r;
+    float v = static_cast<float>(acc) * scale_inv;
+    if (bias != nullptr) v = v + bias[r];
+    out[q * R_total + col] = v;
+}
+
 // ------------------------------------------------------------------ key plane tiling
 __global__ void tile_key_planes_kernel(const unsigned long long* __restrict__ in, int64_t R, int Sb, int W64,
                                        int chunks, int64_t total, unsigned long long* __restrict__ out) {
@@ -728,7 +778,10 @@ struct I8Cfg {
 // the reads of the NEXT k-step's operands into (ka_n, qb_n), so that the LDS latency of every k-step hides
 // behind the MFMAs of the one before it -- also across the barrier between two stages of the ring.
 // KS: k-step of the chunk (0..3); krow_n / qrow_n: the wave's rows of the next k-step's stage, column included.
-template <int WM, int WN, int KS, bool kInts>
+// kMode: kI8Chain (fp32 chunk-scale chain), kI8Ints (the same, and the per-chunk integers are stored) or kI8Sum
+// (plain int32 sum over all chunks: no scales, no epilogue).
+constexpr int kI8Chain = 0, kI8Ints = 1, kI8Sum = 2;
+template <int WM, int WN, int KS, int kMode>
 __device__ __forceinline__ void i8_kstep(const v4i (&ka)[WM], const v4i (&qb)[WN], v4i (&ka_n)[WM], v4i (&qb_n)[WN],
                                          const unsigned char* __restrict__ krow_n,
                                          const unsigned char* __restrict__ qrow_n, v4i (&acc)[WM][WN],
@@ -742,9 +795,10 @@ __device__ __forceinline__ void i8_kstep(const v4i (&ka)[WM], const v4i (&qb)[WN
 #pragma unroll
         for (int b = 0; b < WN; ++b) {
             const int t = a * WN + b;
-            const v4i c0 = (KS == 0) ? (v4i){0, 0, 0, 0} : acc[a][b];
+            constexpr bool kInts = (kMode == kI8Ints);
+            const v4i c0 = (KS == 0 && kMode != kI8Sum) ? (v4i){0, 0, 0, 0} : acc[a][b];
             acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ka[a], qb[b], c0, 0, 0, 0);
-            {
+            if (kMode != kI8Sum) {
                 const int idx = KS * (WM * WN) + t, tt = idx >> 2, e = idx & 3, ea = tt / WN, eb = tt % WN;
                 accf[ea][eb][e] = fmaf(static_cast<float>(prev[ea][eb][e]), qs_prev[eb], accf[ea][eb][e]);
                 if (kInts && ints_prev != nullptr && int_off[ea][eb] >= 0 && e < int_rows[ea])
@@ -758,7 +812,7 @@ __device__ __forceinline__ void i8_kstep(const v4i (&ka)[WM], const v4i (&qb)[WN
         }
 }
 
-template <int TM, int TN, bool kInts>
+template <int TM, int TN, int kMode>
 __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
     const int8_t* __restrict__ A8, const float* __restrict__ qscale, int qscale_stride,
     const int8_t* __restrict__ K8,  // int8 key image [R, chunks * 256]
@@ -766,6 +820,7 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
     int64_t R_total, float* __restrict__ out, int* __restrict__ chunk_ints, const float* __restrict__ bias) {
     using C = I8Cfg<TM, TN>;
     constexpr int WM = C::kWM, WN = C::kWN;
+    constexpr bool kInts = (kMode == kI8Ints), kSum = (kMode == kI8Sum);
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];  // C::kLds
 
     const int tid = threadIdx.x;
@@ -812,7 +867,7 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
             for (int i = 0; i < NI; ++i)
                 load16_to_lds(is_key[i] ? rk : rq, off[i], so,
                               lds + (h & 3) * C::kStage + ((lw + C::kLoaders * i) % C::kGroups) * 1024);
-            if (h & 1) {  // with the second half of chunk c = h / 2: its scales
+            if (!kSum && (h & 1)) {  // with the second half of chunk c = h / 2: its scales
                 const int c = hc >> 1;
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(
                     rs, BSI_LDS_PTR(scale_lds + ((c & 3) * C::kLoaders + lw) * 256), 4, static_cast<int>(soff),
@@ -823,13 +878,13 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
         issue(1);
         issue(2);
         // stage 0 landed (stage 1 + scales + stage 2, 2 NI + 1 instructions, may be in flight)
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NI + 1) : "memory");
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NI + (kSum ? 0 : 1)) : "memory");
         lds_barrier();
         for (int h = 0; h < halves; ++h) {
             issue(h + 3);  // its slot was released by the barrier that ended half h - 1
             // stage h + 1 (and the scales issued right behind it) landed; stages h + 2, h + 3 and one
             // scale load, 2 NI + 1 instructions, may still be in flight
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NI + 1) : "memory");
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NI + (kSum ? 0 : 1)) : "memory");
             lds_barrier();
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still be writing LDS when the workgroup ends
@@ -887,7 +942,7 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
     // which its last operands were read (the even ones); the same barrier tells that the next stage has landed.
     v4i ka[2][WM], qb[2][WN];  // operand sets of even / odd k-steps
 #define BSI_I8_KSTEP(KS, nslot, acc, prev, qs, ip)                                                                  \
-    i8_kstep<WM, WN, KS, kInts>(ka[(KS) & 1], qb[(KS) & 1], ka[((KS) + 1) & 1], qb[((KS) + 1) & 1],                 \
+    i8_kstep<WM, WN, KS, kMode>(ka[(KS) & 1], qb[(KS) & 1], ka[((KS) + 1) & 1], qb[((KS) + 1) & 1],                 \
                                 lds + (nslot) * C::kStage + krow_off + pcol[((KS) + 1) & 1],                        \
                                 lds + (nslot) * C::kStage + qrow_off + pcol[((KS) + 1) & 1], acc, prev, accf, qs,   \
                                 ip, int_off, int_rows, down_shift, chunks);
@@ -911,16 +966,20 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
         int* const ip = c > 0 ? chunk_ints + (c - 1) : nullptr;
         // even chunk c -> acc0, ring slots 0 and 1; epilogue of chunk c-1 (acc1, scales qsb)
         BSI_I8_CHUNK(0, 2, acc0, acc1, qsb, ip);
-        BSI_I8_SCALES(qsa, c);  // landed with the second half of chunk c
+        if (!kSum) BSI_I8_SCALES(qsa, c);  // landed with the second half of chunk c
         // odd chunk c+1 -> acc1, ring slots 2 and 3; epilogue of chunk c (acc0, scales qsa)
-        BSI_I8_CHUNK(2, 0, acc1, acc0, qsa, chunk_ints + c);
-        BSI_I8_SCALES(qsb, c + 1);
+        if (kSum) {
+            BSI_I8_CHUNK(2, 0, acc0, acc1, qsb, ip);  // int32 sum: one accumulator set over all chunks
+        } else {
+            BSI_I8_CHUNK(2, 0, acc1, acc0, qsa, chunk_ints + c);
+            BSI_I8_SCALES(qsb, c + 1);
+        }
     }
     bool last_in_acc0 = false;
     if (c < chunks) {  // odd number of chunks: one more even chunk; its halves sit in slots 0 and 1
         int* const ip = c > 0 ? chunk_ints + (c - 1) : nullptr;
         BSI_I8_CHUNK(0, 2, acc0, acc1, qsb, ip);
-        BSI_I8_SCALES(qsa, c);
+        if (!kSum) BSI_I8_SCALES(qsa, c);
         last_in_acc0 = true;
     }
     // the last k-step read ahead into a stage that does not exist (the loaders fill it with a copy of the last
@@ -929,6 +988,27 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
 #undef BSI_I8_CHUNK
 #undef BSI_I8_KSTEP
 #undef BSI_I8_SCALES
+    if (kSum) {  // out is an int32 matrix [Q, R_total]: the plain integer products
+        int* const iout = reinterpret_cast<int*>(out);
+#pragma unroll
+        for (int a = 0; a < WM; ++a) {
+            const int64_t rb = r0 + wr * (WM * 16) + a * 16 + lg * 4;
+#pragma unroll
+            for (int b = 0; b < WN; ++b) {
+                const int64_t q = q0 + wq * (WN * 16) + b * 16 + ln;
+                if (q >= Q) continue;
+                int* dst = iout + static_cast<size_t>(q) * R_total + rb;
+                if (rb + 3 < R && ((reinterpret_cast<uintptr_t>(dst) & 15) == 0)) {
+                    *reinterpret_cast<v4i*>(dst) = acc0[a][b];
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (rb + e < R) dst[e] = acc0[a][b][e];
+                }
+            }
+        }
+        return;
+    }
     // epilogue of the last chunk
 #pragma unroll
     for (int a = 0; a < WM; ++a)
@@ -1549,26 +1629,36 @@ static void launch_mfma_ws(const int8_t* A8, const float* qscale, int stride, co
                            R_total, out, chunk_ints);
 }
 
-template <int TM, int TN>
-static void launch_mfma_i8_t(const int8_t* A8, const float* qscale, int stride, const int8_t* K8, const float* Bw,
-                             int Sb, int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv,
-                             int64_t R_total, float* out, int32_t* chunk_ints, const float* bias, hipStream_t st) {
+template <int TM, int TN, int kMode>
+static void launch_mfma_i8_tm(const int8_t* A8, const float* qscale, int stride, const int8_t* K8, const float* Bw,
+                              int Sb, int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv,
+                              int64_t R_total, float* out, int32_t* chunk_ints, const float* bias, hipStream_t st) {
     using C = I8Cfg<TM, TN>;
     const dim3 grid(static_cast<unsigned>((R + TM - 1) / TM), static_cast<unsigned>((Q + TN - 1) / TN));
     static bool configured = false;
     if (!configured) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dot_mfma_i8_kernel<TM, TN, true>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, C::kLds);
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dot_mfma_i8_kernel<TM, TN, false>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dot_mfma_i8_kernel<TM, TN, kMode>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, C::kLds);
         configured = true;
     }
-    if (chunk_ints)
-        hipLaunchKernelGGL((dot_mfma_i8_kernel<TM, TN, true>), grid, dim3(C::kBlock), C::kLds, st, A8, qscale, stride,
-                           K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias);
+    hipLaunchKernelGGL((dot_mfma_i8_kernel<TM, TN, kMode>), grid, dim3(C::kBlock), C::kLds, st, A8, qscale, stride, K8,
+                       Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias);
+}
+
+// mode: kI8Sum when `sum` (out is then int32 [Q, R_total]), else the chain with or without stored integers
+template <int TM, int TN>
+static void launch_mfma_i8_t(bool sum, const int8_t* A8, const float* qscale, int stride, const int8_t* K8,
+                             const float* Bw, int Sb, int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv,
+                             int64_t R_total, float* out, int32_t* chunk_ints, const float* bias, hipStream_t st) {
+    if (sum)
+        launch_mfma_i8_tm<TM, TN, kI8Sum>(A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total,
+                                          out, chunk_ints, bias, st);
+    else if (chunk_ints)
+        launch_mfma_i8_tm<TM, TN, kI8Ints>(A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total,
+                                           out, chunk_ints, bias, st);
     else
-        hipLaunchKernelGGL((dot_mfma_i8_kernel<TM, TN, false>), grid, dim3(C::kBlock), C::kLds, st, A8, qscale, stride,
-                           K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias);
+        launch_mfma_i8_tm<TM, TN, kI8Chain>(A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv,
+                                            R_total, out, chunk_ints, bias, st);
 }
 
 // Tile choice.  The 128 x 128 tile moves the fewest operand bytes per MAC and is the fastest whenever its grid
@@ -1592,9 +1682,9 @@ static int choose_i8_tile(int64_t R, int64_t Q) {
 
 static void launch_mfma_i8(const int8_t* A8, const float* qscale, int stride, const int8_t* K8, const float* Bw, int Sb,
                            int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv, int64_t R_total,
-                           float* out, int32_t* chunk_ints, const float* bias, hipStream_t st) {
+                           float* out, int32_t* chunk_ints, const float* bias, hipStream_t st, bool sum = false) {
     const int tile = choose_i8_tile(R, Q);
-#define BSI_I8_ARGS A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias, st
+#define BSI_I8_ARGS sum, A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias, st
     if (tile == 128) launch_mfma_i8_t<128, 128>(BSI_I8_ARGS);
     else if (tile == 12864) launch_mfma_i8_t<128, 64>(BSI_I8_ARGS);
     else if (tile == 64) launch_mfma_i8_t<64, 64>(BSI_I8_ARGS);
@@ -1902,6 +1992,57 @@ extern "C" int bsi_hip_dot_weighted(const uint64_t* A, const float* Aw, int Sa, 
                      : launch_dot_weighted<8, false>(A, Aw, Sa, W64, B, Bw, Sb, R, Q, key_indices, scale_inv, R_total, out, st);
     return tiled ? launch_dot_weighted<2, true>(A, Aw, Sa, W64, B, Bw, Sb, R, Q, key_indices, scale_inv, R_total, out, st)
                  : launch_dot_weighted<2, false>(A, Aw, Sa, W64, B, Bw, Sb, R, Q, key_indices, scale_inv, R_total, out, st);
+}
+
+extern "C" int bsi_hip_planes_to_int8_digits(const uint64_t* words, int64_t rows, int S, int W64, int8_t* out,
+                                             void* stream) {
+    BSI_REQUIRE(rows >= 0 && W64 >= 1, "bad shape");
+    BSI_REQUIRE(S >= 1 && S <= 64, "S must be in [1, 64] (got %d)", S);
+    if (rows == 0) return BSI_OK;
+    BSI_REQUIRE(words && out, "null pointer");
+    const int chunks = (W64 + 3) / 4, ndig = (S + 6) / 7;
+    const int64_t total = static_cast<int64_t>(ndig) * rows * chunks * 8;
+    BSI_REQUIRE((total + 255) / 256 <= 0x7fffffffLL, "too large for one launch");
+    hipLaunchKernelGGL(planes_to_digits_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0,
+                       as_stream(stream), reinterpret_cast<const uint32_t*>(words), rows, S, W64, chunks, ndig,
+                       reinterpret_cast<uint32_t*>(out));
+    BSI_LAUNCH_CHECK("planes_to_digits_kernel");
+    return BSI_OK;
+}
+
+extern "C" size_t bsi_hip_dot_digits_workspace_bytes(int64_t Q, int nq, int64_t R, int nk) {
+    if (Q <= 0 || R <= 0 || nq <= 0 || nk <= 0) return 0;
+    return static_cast<size_t>(nq) * static_cast<size_t>(Q) * static_cast<size_t>(nk) * static_cast<size_t>(R) * 4;
+}
+
+extern "C" int bsi_hip_dot_digits(const int8_t* A_digits, int nq, const float* Aw, int Sa, const int8_t* K_digits, int nk,
+                                  int preshift, const float* Bw, int Sb, int W64, int64_t R, int64_t Q,
+                                  const int64_t* key_indices, float scale_inv, int64_t R_total, const float* bias,
+                                  float* out, void* workspace, size_t workspace_bytes, void* stream) {
+    BSI_REQUIRE(R >= 0 && Q >= 0 && W64 >= 1, "bad shape");
+    BSI_REQUIRE(nq >= 1 && nq <= 10 && nk >= 1 && nk <= 10, "digit counts must be in [1, 10] (got %d, %d)", nq, nk);
+    BSI_REQUIRE(Sa >= 1 && Sb >= 1 && preshift >= 0 && preshift <= 14, "bad slice counts or preshift");
+    BSI_REQUIRE(R_total >= R, "R_total (%lld) < R (%lld)", static_cast<long long>(R_total), static_cast<long long>(R));
+    // |sum| <= 256 chunks' worth of 128 * 128 per element: int32 holds D up to 2^17 elements
+    BSI_REQUIRE(W64 <= 2048, "more than 2^17 elements per row could overflow the int32 sums (W64 = %d)", W64);
+    if (R == 0 || Q == 0) return BSI_OK;
+    BSI_REQUIRE(A_digits && Aw && K_digits && Bw && out, "null pointer");
+    const size_t need = bsi_hip_dot_digits_workspace_bytes(Q, nq, R, nk);
+    BSI_REQUIRE(workspace != nullptr && workspace_bytes >= need, "workspace too small: %zu < %zu bytes", workspace_bytes,
+                need);
+    const int64_t Qd = static_cast<int64_t>(nq) * Q, Rd = static_cast<int64_t>(nk) * R;
+    BSI_REQUIRE((Qd + 31) / 32 <= 65535, "too many query rows for one launch");
+    hipStream_t st = as_stream(stream);
+    // one int8 GEMM over the stacked digits: I[i Q + q, j R + r] = sum_d A_i[q, d] K_j[r, d]
+    launch_mfma_i8(A_digits, Bw, 1, K_digits, Bw, 1, (W64 + 3) / 4, Rd, Qd, 0, 1.0f, Rd,
+                   reinterpret_cast<float*>(workspace), nullptr, nullptr, st, /*sum=*/true);
+    BSI_LAUNCH_CHECK("dot_mfma_i8_kernel (int32 sum)");
+    const int64_t total = Q * R;
+    hipLaunchKernelGGL(digits_combine_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, st,
+                       reinterpret_cast<const int*>(workspace), nq, nk, Q, R, preshift, Aw, Sa, Bw, Sb,
+                       reinterpret_cast<const long long*>(key_indices), scale_inv, R_total, bias, out);
+    BSI_LAUNCH_CHECK("digits_combine_kernel");
+    return BSI_OK;
 }
 
 extern "C" int bsi_hip_dot_timed(const uint64_t* A, const int8_t* A_ints8, const float* A_chunk_scales,

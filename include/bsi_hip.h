@@ -224,6 +224,26 @@ int bsi_hip_dot_weighted(const uint64_t* A, const float* Aw, int Sa, int W64, co
                          const float* Bw, int Sb, int64_t R, int64_t Q, const int64_t* key_indices, float scale_inv,
                          int64_t R_total, float* out, void* stream);
 
+/* Decimal-mode operands on the matrix cores.  bsi_hip_planes_to_int8_digits splits the two's-complement values
+ * of S planes [rows, S, W64] into ceil(S / 7) int8 digit images out[digit][row][chunks * 256] (value =
+ * sum_j digit_j * 128^j: unsigned 7-bit groups of planes, the top group sign-extended; in-chunk element order as
+ * bsi_hip_planes_to_int8, no pre-shift).  bsi_hip_dot_digits multiplies the stacked digit images with one int8
+ * GEMM into int32 (workspace: nq * Q * nk * R * 4 bytes, see bsi_hip_dot_digits_workspace_bytes) and puts the
+ * digit products back together exactly in float64:
+ *   out[q, idx[r]] = float(sum_{i,j} I_ij[q, r] * 2^(7 (i + j) - preshift) * Aw[q, 0] * Bw[r, 0]) * scale_inv (+ bias[r])
+ * which is the weighted-slice dot of bsi_hip_dot_weighted whenever the slice weights are the builders' own
+ * (w_s = 2^s times a per-row power of two, top slice negative for two's-complement rows).  A fixed-bit key image
+ * from bsi_hip_planes_to_int8 is one digit pre-shifted by 8 - S bits; preshift is the sum of both operands'
+ * pre-shifts (0 for digit images).  Rows of at most 2^17 elements.
+ * No counterpart in the reference, whose decimal-mode dot is the popcount kernel cited at bsi_hip_dot_weighted. */
+int bsi_hip_planes_to_int8_digits(const uint64_t* words_device, int64_t rows, int S, int W64, int8_t* out_device,
+                                  void* stream);
+size_t bsi_hip_dot_digits_workspace_bytes(int64_t Q, int nq, int64_t R, int nk);
+int bsi_hip_dot_digits(const int8_t* A_digits, int nq, const float* Aw, int Sa, const int8_t* K_digits, int nk,
+                       int preshift, const float* Bw, int Sb, int W64, int64_t R, int64_t Q,
+                       const int64_t* key_indices, float scale_inv, int64_t R_total, const float* bias, float* out,
+                       void* workspace, size_t workspace_bytes, void* stream);
+
 /* Runs fn-independent timing of `iters` back-to-back bsi_hip_dot launches between two HIP events
  * recorded on `stream`, synchronises, and returns the mean launch duration in microseconds.
  * Mirrors the reference's BSI_PROFILE event pair (bsi_cuda.cpp:713-722,798-806). */

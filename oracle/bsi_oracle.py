@@ -287,3 +287,17 @@ def dot_weighted(A: np.ndarray, Aw: np.ndarray, B: np.ndarray, Bw: np.ndarray, s
         acc = (cnt.astype(np.float64) * coeff.astype(np.float64)).sum(axis=(1, 2))   # exact
         out[q] = acc.astype(np.float32) * np.float32(scale_inv)
     return out
+
+
+def int8_digits(ints: np.ndarray, S: int) -> np.ndarray:
+    """Base-128 digits of S-bit two's-complement values, ``[ceil(S/7), ...]`` int64: the low digits are the
+    unsigned 7-bit groups, the top digit the remaining bits with their sign, so that
+    ``value = sum_j digit_j * 128^j`` and every digit fits an int8.  No counterpart in the reference: this is the
+    operand form of the matrix-core route for decimal-mode operands."""
+    v = np.asarray(ints, dtype=np.int64)
+    n = (int(S) + 6) // 7
+    out = np.zeros((n,) + v.shape, dtype=np.int64)
+    for j in range(n - 1):
+        out[j] = (v >> (7 * j)) & 127
+    out[n - 1] = v >> (7 * (n - 1))  # arithmetic shift keeps the sign
+    return out

@@ -1136,3 +1136,126 @@ def test_empty_and_degenerate_inputs(ops, hip, monkeypatch, bits):
     assert L.bsi_hip_dot_weighted(None, None, 7, 1, None, 0, None, 6, 0, 4, None, 1.0, 0, None, st()) == 0
     m = torch.full((1,), 9, dtype=torch.int64, device="cuda")
     assert L.bsi_hip_decimal_stats(None, 0, 64, m.data_ptr(), None, st()) == 0 and int(m.item()) == 0
+
+
+# ------------------------------------------------------------------ decimal mode on the matrix cores
+
+
+def _image_order(a: np.ndarray, chunks: int) -> np.ndarray:
+    """[..., d] values -> [..., chunks*256] in the int8 images' element order (element 32w + 8m + t of a chunk at
+    byte 32w + 4t + m), zero padded."""
+    d = a.shape[-1]
+    padded = np.zeros(a.shape[:-1] + (chunks * 256,), dtype=np.int64)
+    padded[..., :d] = a
+    e = np.arange(chunks * 256)
+    pos = (e // 32) * 32 + ((e % 32) % 8) * 4 + (e % 32) // 8
+    out = np.zeros_like(padded)
+    out[..., pos] = padded
+    return out
+
+
+def _digits_dev(hip, words: np.ndarray):
+    rows, S, W = words.shape
+    chunks = (W + 3) // 4
+    out = torch.full(((S + 6) // 7, rows, chunks * 256), 77, dtype=torch.int8, device="cuda")
+    hip.check(hip.lib.bsi_hip_planes_to_int8_digits(dev(words).data_ptr(), rows, S, W, out.data_ptr(), st()), "digits")
+    return out
+
+
+@pytest.mark.parametrize("Q,d,scale", [(9, 700, 1.0), (3, 64, 1.0e6), (33, 2048, 3.0), (2, 5, 1.0e15), (4, 256, 0.0)])
+def test_digit_images_match_oracle(hip, oracle, Q, d, scale):
+    x, _ = _decimal_case(Q, 1, d, seed=Q + d, qscale=scale)
+    b = oracle.build_decimal(x, 2)
+    got = _digits_dev(hip, b["words"]).cpu().numpy().astype(np.int64)
+    want = _image_order(oracle.int8_digits(b["ints"], b["S"]), (b["words"].shape[2] + 3) // 4)
+    assert got.shape == want.shape and np.array_equal(got, want)
+
+
+def _run_digits(hip, a_dig, aw, Sa, k_dig, preshift, bw, Sb, W, Q, R, key_indices=None, R_total=None, bias=None):
+    L = hip.lib
+    nq, nk = a_dig.shape[0], k_dig.shape[0]
+    R_total = R if R_total is None else R_total
+    out = torch.full((Q, R_total), float("nan"), dtype=torch.float32, device="cuda")
+    nbytes = int(L.bsi_hip_dot_digits_workspace_bytes(Q, nq, R, nk))
+    assert nbytes == nq * Q * nk * R * 4
+    ws = torch.empty((nbytes,), dtype=torch.uint8, device="cuda")
+    idx = None if key_indices is None else torch.from_numpy(np.asarray(key_indices, dtype=np.int64)).cuda()
+    Aw, Bw = dev(aw), dev(bw)
+    hip.check(L.bsi_hip_dot_digits(a_dig.data_ptr(), nq, Aw.data_ptr(), Sa, k_dig.data_ptr(), nk, preshift, Bw.data_ptr(),
+                                   Sb, W, R, Q, idx.data_ptr() if idx is not None else None, float(np.float32(1e-4)),
+                                   R_total, bias.data_ptr() if bias is not None else None, out.data_ptr(), ws.data_ptr(),
+                                   nbytes, st()), "digit dot")
+    torch.cuda.synchronize()
+    return out.cpu().numpy()
+
+
+@pytest.mark.parametrize("tile", [0, 128, 12864, 64, 6432])
+@pytest.mark.parametrize("Q,R,d,qscale", [(5, 7, 300, 1.0), (70, 150, 2048, 1.0), (64, 256, 2048, 30.0),
+                                          (17, 40, 512, 1.0e6), (1, 33, 8192, 1.0)])
+def test_dot_digits_matches_oracle(hip, oracle, Q, R, d, qscale, tile):
+    """Decimal operands as int8 digits through the int32-sum mode of the MFMA kernel (every tile): bit-identical
+    to the oracle's exact weighted-slice sum, i.e. to the integer matrix product of the rounded values."""
+    x, k = _decimal_case(Q, R, d, seed=Q * 31 + R, qscale=qscale)
+    a, b = oracle.build_decimal(x, 2), oracle.build_decimal(k, 2)
+    W = (d + 63) // 64
+    want = oracle.dot_weighted(a["words"], a["slice_weights"], b["words"], b["slice_weights"], np.float32(1e-4))
+    hip.check(hip.lib.bsi_hip_set_option(hip.OPT_I8_TILE, tile), "opt")
+    try:
+        got = _run_digits(hip, _digits_dev(hip, a["words"]), a["slice_weights"], a["S"], _digits_dev(hip, b["words"]), 0,
+                          b["slice_weights"], b["S"], W, Q, R)
+    finally:
+        hip.check(hip.lib.bsi_hip_set_option(hip.OPT_I8_TILE, 0), "opt")
+    assert np.array_equal(got, want)
+    exact = a["ints"].astype(object) @ b["ints"].astype(object).T
+    if max(abs(int(v)) for v in exact.reshape(-1)) < 2 ** 53:
+        assert np.array_equal(got, exact.astype(np.float64).astype(np.float32) * np.float32(1e-4))
+
+
+def test_dot_digits_fixed_images_indices_bias_and_stride(hip, oracle):
+    """Fixed-bit key image (one digit pre-shifted by 8 - Sb) under decimal queries, and a row-scaled fixed query
+    image against decimal keys; key_indices scatter into a wider output; the bias is added after the scale."""
+    Q, R, d, W = 20, 45, 1024, 16
+    x, k = _decimal_case(Q, R, d, seed=9, kscale=3.0)
+    a, b = oracle.build_decimal(x, 2), oracle.build_keys(k, 2, 6)
+    want = oracle.dot_weighted(a["words"], a["slice_weights"], b["words"], b["slice_weights"], np.float32(1e-4))
+    k8 = torch.empty((1, R, 4 * 256), dtype=torch.int8, device="cuda")
+    hip.check(hip.lib.bsi_hip_planes_to_int8(dev(b["words"]).data_ptr(), R, 6, W, k8.data_ptr(), st()), "image")
+    a_dig = _digits_dev(hip, a["words"])
+    got = _run_digits(hip, a_dig, a["slice_weights"], a["S"], k8, 2, b["slice_weights"], 6, W, Q, R)
+    assert np.array_equal(got, want)
+    perm = np.random.default_rng(3).permutation(60)[:R]
+    bias = torch.randn(R, device="cuda")
+    got = _run_digits(hip, a_dig, a["slice_weights"], a["S"], k8, 2, b["slice_weights"], 6, W, Q, R, key_indices=perm,
+                      R_total=60, bias=bias)
+    assert np.array_equal(got[:, perm], want + bias.cpu().numpy()[None, :])
+    assert np.isnan(got[:, np.setdiff1d(np.arange(60), perm)]).all()
+    # the reverse: 7-bit row-scaled queries (image pre-shifted by 1) against decimal keys
+    ints, shifts, scales = oracle.quantize_fixed(x, 2, 7, False)
+    aw = (oracle.slice_weights(7)[None, :] * scales[:, None]).astype(np.float32)
+    kb = oracle.build_decimal(k, 2)
+    want = oracle.dot_weighted(oracle.pack(ints, 7), aw, kb["words"], kb["slice_weights"], np.float32(1e-4))
+    q8 = torch.empty((1, Q, 4 * 256), dtype=torch.int8, device="cuda")
+    hip.check(hip.lib.bsi_hip_planes_to_int8(dev(oracle.pack(ints, 7)).data_ptr(), Q, 7, W, q8.data_ptr(), st()), "image")
+    got = _run_digits(hip, q8, aw, 7, _digits_dev(hip, kb["words"]), 1, kb["slice_weights"], kb["S"], W, Q, R)
+    assert np.array_equal(got, want)
+
+
+def test_ops_decimal_mfma_and_popcount_routes_agree(ops, monkeypatch):
+    """BSI_DECIMAL_MFMA=0 keeps decimal operands on the popcount kernel; both routes give the same bits."""
+    torch.manual_seed(6)
+    X, K = torch.randn(70, 2048), torch.randn(150, 2048) * 0.02
+    outs = {}
+    for flag in ("1", "0"):
+        monkeypatch.setenv("BSI_FIXED_BITS", "0")
+        monkeypatch.setenv("BSI_DECIMAL_MFMA", flag)
+        ops._reset_flag_cache()
+        kcap, *_ = ops.build_bsi_keys_cuda(K, 2, 0.2)
+        qcap = ops.build_bsi_queries_cuda_batch_packed(X.cuda(), 2, 0.2)
+        assert (qcap.digits8 is not None) == (flag == "1") and (kcap.digits8 is not None) == (flag == "1")
+        outs[flag], *_ = ops.batch_dot_product_multiquery_cuda_batch_caps(qcap, kcap)
+        rows = ops.build_bsi_queries_cuda_batch(X.cuda(), 2, 0.2)
+        o2, *_ = ops.batch_dot_product_multiquery_cuda_caps(rows, kcap)
+        assert torch.equal(o2, outs[flag])
+    assert torch.equal(outs["0"], outs["1"])
+    dense = (X.double() @ K.double().T).float().cuda()
+    assert (outs["1"] - dense).abs().max().item() < 2048 * 0.005 * 4.0

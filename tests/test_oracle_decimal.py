@@ -104,3 +104,18 @@ def test_reference_known_answers_decimal_mode(oracle):
         b = oracle.build_decimal(np.array(case["K"], dtype=np.float32), dec)
         out = oracle.dot_weighted(a["words"], a["slice_weights"], b["words"], b["slice_weights"], oracle.scale_inv(dec, dec))
         np.testing.assert_allclose(out, np.array(case["expected"], dtype=np.float32), atol=1e-4, err_msg=case["cite"])
+
+
+@pytest.mark.parametrize("S", [2, 7, 8, 12, 14, 15, 33, 64])
+def test_int8_digits_recompose_and_fit(oracle, S):
+    rng = np.random.default_rng(S)
+    lo, hi = -(1 << (S - 1)), (1 << (S - 1)) - 1
+    v = rng.integers(lo, hi, size=500, dtype=np.int64, endpoint=True)
+    v[:4] = [lo, hi, 0, -1]
+    dig = oracle.int8_digits(v, S)
+    assert dig.shape[0] == -(-S // 7)
+    assert dig.min() >= -128 and dig.max() <= 127 and (dig[:-1] >= 0).all()
+    total = sum(int(dig[j][i]) * 128 ** j for j in range(dig.shape[0]) for i in [0])  # spot check with big ints
+    assert total == int(v[0])
+    recomposed = [sum(int(dig[j][i]) << (7 * j) for j in range(dig.shape[0])) for i in range(v.size)]
+    assert recomposed == [int(x) for x in v]
