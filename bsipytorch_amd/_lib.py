@@ -16,6 +16,7 @@ DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
 CORE_AUTO, CORE_VALU, CORE_MFMA = 0, 1, 2
 LAYOUT_CANONICAL, LAYOUT_TILED16, LAYOUT_INT8 = 0, 1, 2
 OPT_I8_TILE = 1
+OPT_DIGITS_ROUTE = 2
 
 _vp = ctypes.c_void_p
 _i = ctypes.c_int

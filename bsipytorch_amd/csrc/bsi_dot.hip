@@ -756,6 +756,7 @@ __device__ __forceinline__ void load16_to_lds(bsi_rsrc r, uint32_t lane_off, uin
 // ones for grids that would leave CUs without a workgroup), MFMA waves arranged 2 (keys) x kWavesN (queries),
 // each WM x WN tiles of 16 x 16; one loader wave per (up to) 64 operand rows.
 static int g_i8_tile = 0;  // 0 = by grid size; 128, 12864 (128 keys x 64 queries) or 64 force a tile
+static int g_digits_route = 0;  // bsi_hip_dot_digits: 0 = by cost, 1 = stacked digits + combine pass, 2 = in-accumulator
 
 template <int TM, int TN>
 struct I8Cfg {
@@ -817,7 +818,13 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
     const int8_t* __restrict__ A8, const float* __restrict__ qscale, int qscale_stride,
     const int8_t* __restrict__ K8,  // int8 key image [R, chunks * 256]
     const float* __restrict__ Bw, int Sb, int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv,
-    int64_t R_total, float* __restrict__ out, int* __restrict__ chunk_ints, const float* __restrict__ bias) {
+    int64_t R_total, float* __restrict__ out, int* __restrict__ chunk_ints, const float* __restrict__ bias,
+    int ndig, long long dig_stride, const long long* __restrict__ key_indices) {
+    // kI8Sum only: A8 holds ndig digit images of the queries, dig_stride bytes apart, lowest digit first; the
+    // chunk loop runs over them from the top digit down and the accumulators are shifted left by 7 between two
+    // digits (Horner), so that they end as sum_d (sum_i digit_i[q, d] 128^i) K8[r, d].  With chunk_ints the int32
+    // sums are stored there ([Q, R_total]); without, out[q, idx[r]] = float(sum * 2^-down_shift * qscale[q *
+    // qscale_stride] * Bw[r * Sb]) * scale_inv (+ bias[r]), the product formed in float64.
     using C = I8Cfg<TM, TN>;
     constexpr int WM = C::kWM, WN = C::kWN;
     constexpr bool kInts = (kMode == kI8Ints), kSum = (kMode == kI8Sum);
@@ -829,7 +836,8 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
     const int64_t r0 = static_cast<int64_t>(blockIdx.x) * TM;
     const int64_t q0 = static_cast<int64_t>(blockIdx.y) * TN;
     const size_t rowbytes = static_cast<size_t>(chunks) * 256;
-    const int halves = chunks * 2;
+    const int vchunks = kSum ? chunks * ndig : chunks;  // chunks of the loop: every digit image runs over all chunks
+    const int halves = vchunks * 2;
     unsigned char* const scale_lds = lds + 4 * C::kStage;  // [chunk & 3][loader][64] floats
 
     if (wave >= C::kConsumers) {
@@ -837,7 +845,9 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
         // load moves 1 KiB = 8 rows x 128 bytes), plus the chunk scales of 64 queries once per chunk.
         const int lw = wave - C::kConsumers;
         const bsi_rsrc rk = make_rsrc(K8 + static_cast<size_t>(r0) * rowbytes, static_cast<size_t>(R - r0) * rowbytes);
-        const bsi_rsrc rq = make_rsrc(A8 + static_cast<size_t>(q0) * rowbytes, static_cast<size_t>(Q - q0) * rowbytes);
+        const bsi_rsrc rq = make_rsrc(A8 + static_cast<size_t>(q0) * rowbytes,
+                                      static_cast<size_t>(Q - q0) * rowbytes +
+                                          (kSum ? static_cast<size_t>(ndig - 1) * static_cast<size_t>(dig_stride) : 0));
         const bsi_rsrc rs = make_rsrc(qscale + q0 * qscale_stride, static_cast<size_t>(Q - q0) * qscale_stride * 4);
         // the stage has kGroups groups of 8 rows, keys first; loader lw moves groups lw, lw + kLoaders, ... (when
         // the groups do not divide evenly the last load wraps around and fetches a group a second time, so that
@@ -860,12 +870,29 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
         const int sq = (lw % (TN >= 64 ? TN / 64 : 1)) * 64 + lane;
         const uint32_t soff = static_cast<uint32_t>(((q0 + sq < Q) ? sq : (Q - 1 - q0)) * qscale_stride * 4);
         const int sstep = (qscale_stride == 1) ? 0 : 4;
+        // issue() is called for h = 0, 1, 2, ... in order; in the sum mode (next_c, next_dg) follow the chunk and
+        // the digit (counted from the top one) of the half-chunk to come
+        int next_c = 0, next_dg = 0;
+        uint32_t so_k = 0, so_q = 0;
         auto issue = [&](int h) {  // stage of half-chunk h (clamped to the last) into its ring slot
             const int hc = h < halves ? h : halves - 1;
-            const uint32_t so = static_cast<uint32_t>(hc) * 128;
+            if (kSum) {
+                if (h < halves) {
+                    so_k = static_cast<uint32_t>(next_c) * 256 + static_cast<uint32_t>(h & 1) * 128;
+                    so_q = so_k + static_cast<uint32_t>(ndig - 1 - next_dg) * static_cast<uint32_t>(dig_stride);
+                    if (h & 1) {
+                        if (++next_c == chunks) {
+                            next_c = 0;
+                            ++next_dg;
+                        }
+                    }
+                }
+            } else {
+                so_k = so_q = static_cast<uint32_t>(hc) * 128;
+            }
 #pragma unroll
             for (int i = 0; i < NI; ++i)
-                load16_to_lds(is_key[i] ? rk : rq, off[i], so,
+                load16_to_lds(is_key[i] ? rk : rq, off[i], is_key[i] ? so_k : so_q,
                               lds + (h & 3) * C::kStage + ((lw + C::kLoaders * i) % C::kGroups) * 1024);
             if (!kSum && (h & 1)) {  // with the second half of chunk c = h / 2: its scales
                 const int c = hc >> 1;
@@ -961,14 +988,28 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
 #pragma unroll
     for (int t = 0; t < WN; ++t) qb[0][t] = *reinterpret_cast<const v4i*>(lds + qrow_off + t * 16 * 128 + pcol[0]);
     __builtin_amdgcn_sched_barrier(0);
+    // sum mode: before the first chunk of every digit but the top one, the sums so far move up by one digit
+    int to_next_digit = chunks;
+#define BSI_I8_HORNER()                                                               \
+    if (kSum && ndig > 1) {                                                           \
+        if (to_next_digit == 0) {                                                     \
+            _Pragma("unroll") for (int a = 0; a < WM; ++a)                            \
+                _Pragma("unroll") for (int b = 0; b < WN; ++b)                        \
+                    _Pragma("unroll") for (int e = 0; e < 4; ++e) acc0[a][b][e] <<= 7; \
+            to_next_digit = chunks;                                                   \
+        }                                                                             \
+        --to_next_digit;                                                              \
+    }
     int c = 0;
-    for (; c + 1 < chunks; c += 2) {
-        int* const ip = c > 0 ? chunk_ints + (c - 1) : nullptr;
+    for (; c + 1 < vchunks; c += 2) {
+        int* const ip = (!kSum && c > 0) ? chunk_ints + (c - 1) : nullptr;
         // even chunk c -> acc0, ring slots 0 and 1; epilogue of chunk c-1 (acc1, scales qsb)
+        BSI_I8_HORNER();
         BSI_I8_CHUNK(0, 2, acc0, acc1, qsb, ip);
         if (!kSum) BSI_I8_SCALES(qsa, c);  // landed with the second half of chunk c
         // odd chunk c+1 -> acc1, ring slots 2 and 3; epilogue of chunk c (acc0, scales qsa)
         if (kSum) {
+            BSI_I8_HORNER();
             BSI_I8_CHUNK(2, 0, acc0, acc1, qsb, ip);  // int32 sum: one accumulator set over all chunks
         } else {
             BSI_I8_CHUNK(2, 0, acc1, acc0, qsa, chunk_ints + c);
@@ -976,8 +1017,9 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
         }
     }
     bool last_in_acc0 = false;
-    if (c < chunks) {  // odd number of chunks: one more even chunk; its halves sit in slots 0 and 1
-        int* const ip = c > 0 ? chunk_ints + (c - 1) : nullptr;
+    if (c < vchunks) {  // odd number of chunks: one more even chunk; its halves sit in slots 0 and 1
+        int* const ip = (!kSum && c > 0) ? chunk_ints + (c - 1) : nullptr;
+        BSI_I8_HORNER();
         BSI_I8_CHUNK(0, 2, acc0, acc1, qsb, ip);
         if (!kSum) BSI_I8_SCALES(qsa, c);
         last_in_acc0 = true;
@@ -985,11 +1027,11 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
     // the last k-step read ahead into a stage that does not exist (the loaders fill it with a copy of the last
     // one); nothing uses those operands
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#undef BSI_I8_HORNER
 #undef BSI_I8_CHUNK
 #undef BSI_I8_KSTEP
 #undef BSI_I8_SCALES
-    if (kSum) {  // out is an int32 matrix [Q, R_total]: the plain integer products
-        int* const iout = reinterpret_cast<int*>(out);
+    if (kSum && chunk_ints != nullptr) {  // the plain integer sums, int32 [Q, R_total]
 #pragma unroll
         for (int a = 0; a < WM; ++a) {
             const int64_t rb = r0 + wr * (WM * 16) + a * 16 + lg * 4;
@@ -997,13 +1039,43 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
             for (int b = 0; b < WN; ++b) {
                 const int64_t q = q0 + wq * (WN * 16) + b * 16 + ln;
                 if (q >= Q) continue;
-                int* dst = iout + static_cast<size_t>(q) * R_total + rb;
+                int* dst = chunk_ints + static_cast<size_t>(q) * R_total + rb;
                 if (rb + 3 < R && ((reinterpret_cast<uintptr_t>(dst) & 15) == 0)) {
                     *reinterpret_cast<v4i*>(dst) = acc0[a][b];
                 } else {
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
                         if (rb + e < R) dst[e] = acc0[a][b][e];
+                }
+            }
+        }
+        return;
+    }
+    if (kSum) {  // float(sum * 2^-down_shift * query factor * key factor) * scale_inv (+ bias), the product in float64
+        const double down2 = __longlong_as_double(static_cast<long long>(1023 - down_shift) << 52);
+        double qf[WN];
+#pragma unroll
+        for (int b = 0; b < WN; ++b) {
+            const int64_t q = q0 + wq * (WN * 16) + b * 16 + ln;
+            qf[b] = (q < Q) ? static_cast<double>(qscale[q * qscale_stride]) * down2 : 0.0;
+        }
+#pragma unroll
+        for (int a = 0; a < WM; ++a) {
+            const int64_t rb = r0 + wr * (WM * 16) + a * 16 + lg * 4;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int64_t r = rb + e;
+                if (r >= R) continue;
+                const double kf = static_cast<double>(Bw[r * Sb]);
+                const float bi = bias != nullptr ? bias[r] : 0.0f;
+                const int64_t col = key_indices ? key_indices[r] : r;
+#pragma unroll
+                for (int b = 0; b < WN; ++b) {
+                    const int64_t q = q0 + wq * (WN * 16) + b * 16 + ln;
+                    if (q >= Q) continue;
+                    float v = static_cast<float>(static_cast<double>(acc0[a][b][e]) * qf[b] * kf) * scale_inv;
+                    if (bias != nullptr) v = v + bi;
+                    out[static_cast<size_t>(q) * R_total + col] = v;
                 }
             }
         }
@@ -1632,7 +1704,8 @@ static void launch_mfma_ws(const int8_t* A8, const float* qscale, int stride, co
 template <int TM, int TN, int kMode>
 static void launch_mfma_i8_tm(const int8_t* A8, const float* qscale, int stride, const int8_t* K8, const float* Bw,
                               int Sb, int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv,
-                              int64_t R_total, float* out, int32_t* chunk_ints, const float* bias, hipStream_t st) {
+                              int64_t R_total, float* out, int32_t* chunk_ints, const float* bias, hipStream_t st,
+                              int ndig, long long dig_stride, const long long* key_indices) {
     using C = I8Cfg<TM, TN>;
     const dim3 grid(static_cast<unsigned>((R + TM - 1) / TM), static_cast<unsigned>((Q + TN - 1) / TN));
     static bool configured = false;
@@ -1642,23 +1715,26 @@ static void launch_mfma_i8_tm(const int8_t* A8, const float* qscale, int stride,
         configured = true;
     }
     hipLaunchKernelGGL((dot_mfma_i8_kernel<TM, TN, kMode>), grid, dim3(C::kBlock), C::kLds, st, A8, qscale, stride, K8,
-                       Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias);
+                       Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias, ndig, dig_stride,
+                       key_indices);
 }
 
-// mode: kI8Sum when `sum` (out is then int32 [Q, R_total]), else the chain with or without stored integers
+// Sum mode (ndig >= 1 digit images of the queries; int32 sums into chunk_ints when given, else the float epilogue)
+// or, with ndig == 0, the chain with or without stored integers.
 template <int TM, int TN>
-static void launch_mfma_i8_t(bool sum, const int8_t* A8, const float* qscale, int stride, const int8_t* K8,
-                             const float* Bw, int Sb, int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv,
-                             int64_t R_total, float* out, int32_t* chunk_ints, const float* bias, hipStream_t st) {
-    if (sum)
+static void launch_mfma_i8_t(int ndig, long long dig_stride, const long long* key_indices, const int8_t* A8,
+                             const float* qscale, int stride, const int8_t* K8, const float* Bw, int Sb, int chunks,
+                             int64_t R, int64_t Q, int down_shift, float scale_inv, int64_t R_total, float* out,
+                             int32_t* chunk_ints, const float* bias, hipStream_t st) {
+    if (ndig > 0)
         launch_mfma_i8_tm<TM, TN, kI8Sum>(A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total,
-                                          out, chunk_ints, bias, st);
+                                          out, chunk_ints, bias, st, ndig, dig_stride, key_indices);
     else if (chunk_ints)
         launch_mfma_i8_tm<TM, TN, kI8Ints>(A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total,
-                                           out, chunk_ints, bias, st);
+                                           out, chunk_ints, bias, st, 1, 0, nullptr);
     else
         launch_mfma_i8_tm<TM, TN, kI8Chain>(A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv,
-                                            R_total, out, chunk_ints, bias, st);
+                                            R_total, out, chunk_ints, bias, st, 1, 0, nullptr);
 }
 
 // Tile choice.  The 128 x 128 tile moves the fewest operand bytes per MAC and is the fastest whenever its grid
@@ -1666,9 +1742,10 @@ static void launch_mfma_i8_t(bool sum, const int8_t* A8, const float* qscale, in
 // leaves CUs idle that smaller tiles would use: a workgroup's time per half-chunk is about 1 : 0.63 : 0.35 : 0.31
 // for 128 x 128 : 128 x 64 : 64 x 64 : 64 x 32, so take the least (rounds of 256 workgroups x time), the larger
 // tile on a tie.  g_i8_tile forces a tile (tuning and tests).
-static int choose_i8_tile(int64_t R, int64_t Q) {
-    if (g_i8_tile != 0) return g_i8_tile;
+static int choose_i8_tile(int64_t R, int64_t Q, int64_t* cost_out = nullptr) {
     const int64_t n128 = ((R + 127) / 128) * ((Q + 127) / 128);
+    if (cost_out) *cost_out = ((n128 + 255) / 256) * 100;
+    if (g_i8_tile != 0) return g_i8_tile;
     if (n128 > 256) return 128;
     const int64_t cost[4] = {100, ((((R + 127) / 128) * ((Q + 63) / 64) + 255) / 256) * 63,
                              ((((R + 63) / 64) * ((Q + 63) / 64) + 255) / 256) * 35,
@@ -1677,14 +1754,16 @@ static int choose_i8_tile(int64_t R, int64_t Q) {
     int best = 0;
     for (int i = 1; i < 4; ++i)
         if (cost[i] < cost[best]) best = i;
+    if (cost_out) *cost_out = cost[best];
     return tiles[best];
 }
 
 static void launch_mfma_i8(const int8_t* A8, const float* qscale, int stride, const int8_t* K8, const float* Bw, int Sb,
                            int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv, int64_t R_total,
-                           float* out, int32_t* chunk_ints, const float* bias, hipStream_t st, bool sum = false) {
+                           float* out, int32_t* chunk_ints, const float* bias, hipStream_t st, int ndig = 0,
+                           long long dig_stride = 0, const long long* key_indices = nullptr) {
     const int tile = choose_i8_tile(R, Q);
-#define BSI_I8_ARGS sum, A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias, st
+#define BSI_I8_ARGS ndig, dig_stride, key_indices, A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias, st
     if (tile == 128) launch_mfma_i8_t<128, 128>(BSI_I8_ARGS);
     else if (tile == 12864) launch_mfma_i8_t<128, 64>(BSI_I8_ARGS);
     else if (tile == 64) launch_mfma_i8_t<64, 64>(BSI_I8_ARGS);
@@ -1760,6 +1839,10 @@ extern "C" int bsi_hip_planes_to_int8(const uint64_t* words, int64_t rows, int S
 
 extern "C" int bsi_hip_set_option(int option, int value) {
     switch (option) {
+        case BSI_OPT_DIGITS_ROUTE:
+            BSI_REQUIRE(value >= 0 && value <= 2, "route must be 0, 1 or 2");
+            g_digits_route = value;
+            return BSI_OK;
         case BSI_OPT_I8_TILE:
             BSI_REQUIRE(value == 0 || value == 128 || value == 12864 || value == 64 || value == 6432,
                         "tile must be 0, 128, 12864, 64 or 6432");
@@ -2027,15 +2110,43 @@ extern "C" int bsi_hip_dot_digits(const int8_t* A_digits, int nq, const float* A
     BSI_REQUIRE(W64 <= 2048, "more than 2^17 elements per row could overflow the int32 sums (W64 = %d)", W64);
     if (R == 0 || Q == 0) return BSI_OK;
     BSI_REQUIRE(A_digits && Aw && K_digits && Bw && out, "null pointer");
-    const size_t need = bsi_hip_dot_digits_workspace_bytes(Q, nq, R, nk);
-    BSI_REQUIRE(workspace != nullptr && workspace_bytes >= need, "workspace too small: %zu < %zu bytes", workspace_bytes,
-                need);
     const int64_t Qd = static_cast<int64_t>(nq) * Q, Rd = static_cast<int64_t>(nk) * R;
     BSI_REQUIRE((Qd + 31) / 32 <= 65535, "too many query rows for one launch");
     hipStream_t st = as_stream(stream);
-    // one int8 GEMM over the stacked digits: I[i Q + q, j R + r] = sum_d A_i[q, d] K_j[r, d]
-    launch_mfma_i8(A_digits, Bw, 1, K_digits, Bw, 1, (W64 + 3) / 4, Rd, Qd, 0, 1.0f, Rd,
-                   reinterpret_cast<float*>(workspace), nullptr, nullptr, st, /*sum=*/true);
+    const int chunks = (W64 + 3) / 4;
+    const long long dig_stride = static_cast<long long>(Q) * chunks * 256;
+    // One key digit: the query digits are put back together in the accumulator (shift by 7 between digits) and the
+    // epilogue writes the floats -- if int32 holds sum_d |query value| |key digit|: query bits (Sa - 1 + preshift
+    // when nq == 1, as the image is pre-shifted) + 7 key bits + log2(elements) <= 31, and the digit images lie
+    // within reach of a 32-bit buffer offset.
+    int log2_elems = 0;
+    while ((1LL << log2_elems) < static_cast<long long>(chunks) * 256) ++log2_elems;
+    const int qbits = (nq == 1) ? 7 : (Sa - 1);
+    const int kbits = (preshift == 0 && Sb <= 7) ? (Sb - 1) : 7;
+    const bool can_fold = nk == 1 && qbits + kbits + log2_elems <= 31 && static_cast<long long>(nq) * dig_stride < (1LL << 31);
+    // folding runs nq times the chunks on the grid of Q rows; stacking runs the chunks once on the grid of nq Q rows
+    // and then reads the int32 products back (about 3 us + 4 bytes per product at 4 TB/s; one cost unit of the tile
+    // model is about 0.012 us per chunk)
+    int64_t cost_fold = 0, cost_stack = 0;
+    const int tile_fold = choose_i8_tile(R, Q, &cost_fold);
+    const int tile_stack = choose_i8_tile(Rd, Qd, &cost_stack);
+    // without the chain's epilogue to overlap, the 64-key tiles come out about 1.3 times their modelled cost
+    const double us_fold = 0.012 * static_cast<double>(cost_fold) * chunks * nq * ((tile_fold == 64 || tile_fold == 6432) ? 1.3 : 1.0);
+    const double us_stack = 0.012 * static_cast<double>(cost_stack) * chunks * ((tile_stack == 64 || tile_stack == 6432) ? 1.3 : 1.0) + 3.0 +
+                            static_cast<double>(nq * nk + 1) * static_cast<double>(Q) * static_cast<double>(R) * 4.0 / 4.0e6;
+    const bool fold = g_digits_route == 2 || (g_digits_route == 0 && (nq == 1 || us_fold <= us_stack));
+    if (can_fold && fold) {
+        launch_mfma_i8(A_digits, Aw, Sa, K_digits, Bw, Sb, chunks, R, Q, preshift, scale_inv, R_total, out, nullptr, bias,
+                       st, nq, dig_stride, reinterpret_cast<const long long*>(key_indices));
+        BSI_LAUNCH_CHECK("dot_mfma_i8_kernel (int32 sum, digits recombined in the accumulator)");
+        return BSI_OK;
+    }
+    const size_t need = bsi_hip_dot_digits_workspace_bytes(Q, nq, R, nk);
+    BSI_REQUIRE(workspace != nullptr && workspace_bytes >= need, "workspace too small: %zu < %zu bytes", workspace_bytes,
+                need);
+    // else one int8 GEMM over the stacked digits: I[i Q + q, j R + r] = sum_d A_i[q, d] K_j[r, d]
+    launch_mfma_i8(A_digits, Bw, 1, K_digits, Bw, 1, chunks, Rd, Qd, 0, 1.0f, Rd, nullptr,
+                   reinterpret_cast<int32_t*>(workspace), nullptr, st, 1, 0, nullptr);
     BSI_LAUNCH_CHECK("dot_mfma_i8_kernel (int32 sum)");
     const int64_t total = Q * R;
     hipLaunchKernelGGL(digits_combine_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, st,

@@ -164,6 +164,8 @@ int bsi_hip_planes_to_int8(const uint64_t* words_device, int64_t rows, int S, in
 #define BSI_OPT_I8_TILE 1 /* tile of the int8-image kernel: 128 (128 keys x 128 queries), 12864 (128 x 64), 64 (64 x 64)
                              or 6432 (64 x 32); 0 (default) = chosen per call from the grid each tile would give on
                              the 256 CUs */
+#define BSI_OPT_DIGITS_ROUTE 2 /* bsi_hip_dot_digits: 1 = stacked digits and a combine pass, 2 = digits recombined in the
+                                  accumulator where the int32 bound allows; 0 (default) = the cheaper by a cost estimate */
 int bsi_hip_set_option(int option, int value);
 
 /* Bytes of device workspace bsi_hip_dot needs for this shape and core (0 when none). */

@@ -1201,11 +1201,14 @@ def test_dot_digits_matches_oracle(hip, oracle, Q, R, d, qscale, tile):
     want = oracle.dot_weighted(a["words"], a["slice_weights"], b["words"], b["slice_weights"], np.float32(1e-4))
     hip.check(hip.lib.bsi_hip_set_option(hip.OPT_I8_TILE, tile), "opt")
     try:
-        got = _run_digits(hip, _digits_dev(hip, a["words"]), a["slice_weights"], a["S"], _digits_dev(hip, b["words"]), 0,
-                          b["slice_weights"], b["S"], W, Q, R)
+        for route in (1, 2, 0):  # stacked digits + combine pass; digits recombined in the accumulator; by cost
+            hip.check(hip.lib.bsi_hip_set_option(hip.OPT_DIGITS_ROUTE, route), "opt")
+            got = _run_digits(hip, _digits_dev(hip, a["words"]), a["slice_weights"], a["S"], _digits_dev(hip, b["words"]),
+                              0, b["slice_weights"], b["S"], W, Q, R)
+            assert np.array_equal(got, want), route
     finally:
         hip.check(hip.lib.bsi_hip_set_option(hip.OPT_I8_TILE, 0), "opt")
-    assert np.array_equal(got, want)
+        hip.check(hip.lib.bsi_hip_set_option(hip.OPT_DIGITS_ROUTE, 0), "opt")
     exact = a["ints"].astype(object) @ b["ints"].astype(object).T
     if max(abs(int(v)) for v in exact.reshape(-1)) < 2 ** 53:
         assert np.array_equal(got, exact.astype(np.float64).astype(np.float32) * np.float32(1e-4))
@@ -1221,14 +1224,17 @@ def test_dot_digits_fixed_images_indices_bias_and_stride(hip, oracle):
     k8 = torch.empty((1, R, 4 * 256), dtype=torch.int8, device="cuda")
     hip.check(hip.lib.bsi_hip_planes_to_int8(dev(b["words"]).data_ptr(), R, 6, W, k8.data_ptr(), st()), "image")
     a_dig = _digits_dev(hip, a["words"])
-    got = _run_digits(hip, a_dig, a["slice_weights"], a["S"], k8, 2, b["slice_weights"], 6, W, Q, R)
-    assert np.array_equal(got, want)
     perm = np.random.default_rng(3).permutation(60)[:R]
     bias = torch.randn(R, device="cuda")
-    got = _run_digits(hip, a_dig, a["slice_weights"], a["S"], k8, 2, b["slice_weights"], 6, W, Q, R, key_indices=perm,
-                      R_total=60, bias=bias)
-    assert np.array_equal(got[:, perm], want + bias.cpu().numpy()[None, :])
-    assert np.isnan(got[:, np.setdiff1d(np.arange(60), perm)]).all()
+    for route in (1, 2):
+        hip.check(hip.lib.bsi_hip_set_option(hip.OPT_DIGITS_ROUTE, route), "opt")
+        got = _run_digits(hip, a_dig, a["slice_weights"], a["S"], k8, 2, b["slice_weights"], 6, W, Q, R)
+        assert np.array_equal(got, want), route
+        got = _run_digits(hip, a_dig, a["slice_weights"], a["S"], k8, 2, b["slice_weights"], 6, W, Q, R, key_indices=perm,
+                          R_total=60, bias=bias)
+        assert np.array_equal(got[:, perm], want + bias.cpu().numpy()[None, :]), route
+        assert np.isnan(got[:, np.setdiff1d(np.arange(60), perm)]).all()
+    hip.check(hip.lib.bsi_hip_set_option(hip.OPT_DIGITS_ROUTE, 0), "opt")
     # the reverse: 7-bit row-scaled queries (image pre-shifted by 1) against decimal keys
     ints, shifts, scales = oracle.quantize_fixed(x, 2, 7, False)
     aw = (oracle.slice_weights(7)[None, :] * scales[:, None]).astype(np.float32)
