@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(_HERE, "libbsi_hip.so")
 BSI_OK = 0
 DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
 CORE_AUTO, CORE_VALU, CORE_MFMA = 0, 1, 2
-LAYOUT_CANONICAL, LAYOUT_TILED16, LAYOUT_INT8 = 0, 1, 2
+LAYOUT_CANONICAL, LAYOUT_TILED16, LAYOUT_INT8, LAYOUT_INT8_TILED = 0, 1, 2, 3
 OPT_I8_TILE = 1
 OPT_DIGITS_ROUTE = 2
 
@@ -52,11 +52,14 @@ PROTOTYPES = {
     "bsi_hip_dot_workspace_bytes": [_i64, _i, _i],
     "bsi_hip_dot": [_vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _i, _i64, _i64, _f, _i64, _vp, _vp, _i, _vp, _sz, _vp],
     "bsi_hip_dot_bias": [_vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _i, _i64, _i64, _f, _i64, _vp, _vp, _i, _vp, _sz, _vp],
+    "bsi_hip_dot_bias_warm": [_vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _i, _i64, _i64, _f, _i64, _vp, _vp, _i, _vp, _sz, _vp, _sz, _vp],
     "bsi_hip_dot_ewah_query": [_vp, _vp, _vp, _i, _i, _vp, _i, _vp, _vp, _i, _i64, _f, _vp, _vp, _vp],
     "bsi_hip_planes_to_int8_digits": [_vp, _i64, _i, _i, _vp, _vp],
     "bsi_hip_dot_digits_workspace_bytes": [_i64, _i, _i64, _i],
     "bsi_hip_dot_digits": [_vp, _i, _vp, _i, _vp, _i, _i, _vp, _i, _i, _i64, _i64, _vp, _f, _i64, _vp, _vp, _vp,
-                           _sz, _vp],
+                           _sz, _i, _vp],
+    "bsi_hip_int8_tiled_bytes": [_i64, _i],
+    "bsi_hip_planes_to_int8_tiled": [_vp, _i64, _i, _i, _vp, _vp],
     "bsi_hip_dot_weighted": [_vp, _vp, _i, _i, _vp, _i, _vp, _i, _i64, _i64, _vp, _f, _i64, _vp, _vp],
     "bsi_hip_dot_timed": [_vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _i, _i64, _i64, _f, _i64, _vp, _i, _vp, _sz, _i,
                           ctypes.POINTER(_f), _vp],
@@ -71,6 +74,7 @@ _RESTYPES = {
     "bsi_hip_last_error": ctypes.c_char_p,
     "bsi_hip_dot_workspace_bytes": _sz,
     "bsi_hip_dot_digits_workspace_bytes": _sz,
+    "bsi_hip_int8_tiled_bytes": _sz,
 }
 
 

@@ -82,6 +82,7 @@ def _flags() -> dict:
         key_image=(_env_int("BSI_KEY_INT8_IMAGE", 1) or 0) != 0,
         ewah_inline=(_env_int("BSI_EWAH_INLINE", 1) or 0) != 0,
         decimal_mfma=(_env_int("BSI_DECIMAL_MFMA", 1) or 0) != 0,
+        image_tiled=(_env_int("BSI_KEY_IMAGE_TILED", 0) or 0) != 0,
     )
     return _flag_cache
 
@@ -147,7 +148,8 @@ class PrebuiltBSIKeysCUDA(_Capsule):
     def __init__(self):
         self.words: torch.Tensor = None          # canonical [R, Sb, W] or tiled [ceil(R/16), chunks, Sb, 64]
         self.layout = _lib.LAYOUT_CANONICAL
-        self.ints8: Optional[torch.Tensor] = None  # cached int8 image [R, chunks*256] of the same integers, or None
+        self.ints8: Optional[torch.Tensor] = None  # cached int8 image of the same integers, or None: row-major
+        self.ints8_tiled = False                   # [R, chunks*256], or tiled [ceil(R/64), 2 chunks, 64, 128] (flat)
         self.slice_weights: torch.Tensor = None  # [R, Sb] float32
         self.shifts: torch.Tensor = None         # [R] int32 (fixed-bit keys only)
         self.fixed = True                        # False: decimal-mode keys (slice count from the data, canonical planes)
@@ -526,9 +528,18 @@ def _install_fixed_key_planes(h: "PrebuiltBSIKeysCUDA", words: torch.Tensor) -> 
     R = h.num_keys
     if f["key_image"] and R > 0 and 2 <= h.Sb <= 8:
         # compute-bound shapes contract this image on the matrix cores; the planes stay the stored form
-        h.ints8 = torch.empty((R, ((h.W + 3) // 4) * 256), dtype=torch.int8, device=dev)
-        check(lib.bsi_hip_planes_to_int8(words.data_ptr(), R, h.Sb, h.W, h.ints8.data_ptr(), _stream()),
-              "bsi_hip_planes_to_int8")
+        if f["image_tiled"]:
+            # tiled by 64 rows and half-chunks: a workgroup's key rows of a half-chunk are contiguous (off by
+            # default: measured no faster than the row-major image, cache-resident or not)
+            h.ints8 = torch.empty((int(lib.bsi_hip_int8_tiled_bytes(R, h.W)),), dtype=torch.int8, device=dev)
+            h.ints8_tiled = True
+            check(lib.bsi_hip_planes_to_int8_tiled(words.data_ptr(), R, h.Sb, h.W, h.ints8.data_ptr(), _stream()),
+                  "bsi_hip_planes_to_int8_tiled")
+        else:
+            h.ints8 = torch.empty((R, ((h.W + 3) // 4) * 256), dtype=torch.int8, device=dev)
+            h.ints8_tiled = False
+            check(lib.bsi_hip_planes_to_int8(words.data_ptr(), R, h.Sb, h.W, h.ints8.data_ptr(), _stream()),
+                  "bsi_hip_planes_to_int8")
     if f["tiled"] and R > 0:
         chunks = (h.W + 3) // 4
         tiled = torch.empty(((R + 15) // 16, chunks, h.Sb, 64), dtype=torch.int64, device=dev)
@@ -695,12 +706,21 @@ def key_operand(keys: "PrebuiltBSIKeysCUDA", Q: int, Sa: int, core: int):
     """(device pointer, layout code) of the key representation the dot should read for Q query rows:
     the packed planes while the call is bound by streaming them, the cached int8 image above."""
     if keys.ints8 is not None and core != _lib.CORE_VALU and Q > _FEW_ROWS_MAX_Q and 2 <= Sa <= 8:
-        return keys.ints8.data_ptr(), _lib.LAYOUT_INT8
+        return keys.ints8.data_ptr(), (_lib.LAYOUT_INT8_TILED if keys.ints8_tiled else _lib.LAYOUT_INT8)
     return keys.words.data_ptr(), keys.layout
 
 
+def _warm_region(next_keys, Q: int, Sa: int, core: int):
+    """(pointer, bytes) of what a dot of Q query rows would read of ``next_keys``, or (None, 0)."""
+    if next_keys is None or not next_keys.fixed:
+        return None, 0
+    if next_keys.ints8 is not None and core != _lib.CORE_VALU and Q > _FEW_ROWS_MAX_Q and 2 <= Sa <= 8:
+        return next_keys.ints8.data_ptr(), next_keys.ints8.numel()
+    return next_keys.words.data_ptr(), next_keys.words.numel() * 8
+
+
 def _dot(words, ints8, scales, scale_stride, Sa, W, keys: PrebuiltBSIKeysCUDA, Q, decimals_q, chunk_ints=None, core=None,
-         bias=None):
+         bias=None, warm_keys=None):
     f = _flags()
     dev = words.device
     R = keys.num_keys
@@ -720,7 +740,14 @@ def _dot(words, ints8, scales, scale_stride, Sa, W, keys: PrebuiltBSIKeysCUDA, Q
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
     kptr, klayout = key_operand(keys, Q, Sa, core)
-    if bias is not None and chunk_ints is None:
+    if warm_keys is not None and chunk_ints is None:
+        # the kernel also touches what the next layer's dot will read, so that it is cache-resident by then
+        wptr, wbytes = _warm_region(warm_keys, Q, Sa, core)
+        check(lib.bsi_hip_dot_bias_warm(words.data_ptr(), _ptr(ints8), scales.data_ptr(), scale_stride, Sa, W,
+                                        kptr, klayout, keys.slice_weights.data_ptr(), keys.Sb, R, Q,
+                                        _scale_inv(decimals_q, keys.decimals), R, _ptr(bias), out.data_ptr(), core,
+                                        _ptr(ws), ws_bytes, wptr, wbytes, _stream()), "bsi_hip_dot_bias_warm")
+    elif bias is not None and chunk_ints is None:
         check(lib.bsi_hip_dot_bias(words.data_ptr(), _ptr(ints8), scales.data_ptr(), scale_stride, Sa, W,
                                    kptr, klayout, keys.slice_weights.data_ptr(), keys.Sb, R, Q,
                                    _scale_inv(decimals_q, keys.decimals), R, bias.data_ptr(), out.data_ptr(), core,
@@ -755,11 +782,11 @@ def _dot_weighted(words, slice_weights, Sa, W, keys: PrebuiltBSIKeysCUDA, Q, dec
     R = keys.num_keys
     out = torch.empty((Q, R), dtype=torch.float32, device=words.device)
     Aw = slice_weights if slice_weights.is_contiguous() else slice_weights.contiguous()
-    k_digits, nk, preshift = None, 0, 0
+    k_digits, nk, preshift, k_tiled = None, 0, 0, 0
     if q_digits is None and q_image is not None and 2 <= Sa <= 8:
         q_digits, preshift = q_image.unsqueeze(0), 8 - int(Sa)
     if keys.fixed and keys.ints8 is not None:
-        k_digits, nk, preshift = keys.ints8, 1, preshift + 8 - keys.Sb
+        k_digits, nk, preshift, k_tiled = keys.ints8, 1, preshift + 8 - keys.Sb, int(keys.ints8_tiled)
     elif not keys.fixed and keys.digits8 is not None:
         k_digits, nk = keys.digits8, int(keys.digits8.shape[0])
     use_digits = (f["decimal_mfma"] and f["core"] != _lib.CORE_VALU and q_digits is not None and k_digits is not None
@@ -776,7 +803,7 @@ def _dot_weighted(words, slice_weights, Sa, W, keys: PrebuiltBSIKeysCUDA, Q, dec
         check(lib.bsi_hip_dot_digits(qd.data_ptr(), nq, Aw.data_ptr(), int(Sa), k_digits.data_ptr(), nk, preshift,
                                      keys.slice_weights.data_ptr(), keys.Sb, int(W), R, Q, None,
                                      _scale_inv(decimals_q, keys.decimals), R, _ptr(bias), out.data_ptr(),
-                                     ws.data_ptr(), ws_bytes, _stream()), "bsi_hip_dot_digits")
+                                     ws.data_ptr(), ws_bytes, k_tiled, _stream()), "bsi_hip_dot_digits")
     else:
         check(lib.bsi_hip_dot_weighted(words.data_ptr(), Aw.data_ptr(), int(Sa), int(W), keys.words.data_ptr(),
                                        keys.layout, keys.slice_weights.data_ptr(), keys.Sb, R, Q, None,
@@ -802,11 +829,12 @@ def _dot_result(out, ns, Q, R):
     return out, int(ns), per_q, per_s
 
 
-def batch_dot_product_multiquery_cuda_batch_caps(query_batch_cap, keyset_cuda_cap, bias=None):
+def batch_dot_product_multiquery_cuda_batch_caps(query_batch_cap, keyset_cuda_cap, bias=None, warm_keys=None):
     """bsi_cuda.cpp:658-815 -> (out[Q, R] float32 on the device, dot_ns_total, ns_per_query, ns_per_scalar).
     The times are zero unless BSI_PROFILE=1 (which synchronises), as in the reference.
     ``bias`` (not in the reference's signature): an optional float32 [R] device tensor added to every output
-    row in the same launch, rounded as ``out + bias`` would be."""
+    row in the same launch, rounded as ``out + bias`` would be.  ``warm_keys`` (not in the reference either): the
+    keyset the next dot will use; this launch also reads it once so that it is cache-resident by then."""
     keys = _capsule(keyset_cuda_cap, PrebuiltBSIKeysCUDA, "Invalid CUDA keys capsule")
     qb = _capsule(query_batch_cap, PrebuiltBSIQueryBatchCUDA, "Invalid CUDA query-batch capsule")
     _check(qb.words is not None and qb.slice_weights is not None, "Query batch tensors are not defined")
@@ -837,7 +865,10 @@ def batch_dot_product_multiquery_cuda_batch_caps(query_batch_cap, keyset_cuda_ca
         _check(bias.is_cuda and bias.dtype == torch.float32 and bias.dim() == 1 and bias.numel() == R and bias.is_contiguous(),
                "bias must be a contiguous float32 CUDA tensor of [R]")
     if qb.fixed and keys.fixed:
-        out, ns = _dot(qb.words, qb.ints8, scales, stride, int(Sa), int(W), keys, int(Q), qb.decimals, bias=bias)
+        if warm_keys is not None:
+            _capsule(warm_keys, PrebuiltBSIKeysCUDA, "Invalid CUDA keys capsule (warm_keys)")
+        out, ns = _dot(qb.words, qb.ints8, scales, stride, int(Sa), int(W), keys, int(Q), qb.decimals, bias=bias,
+                       warm_keys=warm_keys)
     else:
         # a decimal-mode operand on either side: its slice weights carry everything, per-chunk scales cannot apply
         _check(not have_chunk_scales, "chunk-scaled queries need fixed-bit keys (BSI_FIXED_BITS_KEYS > 0)")

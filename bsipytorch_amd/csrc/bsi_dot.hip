@@ -102,7 +102,7 @@ __device__ __forceinline__ void planes32_to_bytes(const uint32_t p[S], uint32_t 
 // ------------------------------------------------------------------ planes -> int8 pre-pass
 // One thread per (row, 32-bit column).
 __global__ void planes_to_int8_kernel(const uint32_t* __restrict__ words32, int64_t rows, int S, int W64, int chunks,
-                                      uint32_t* __restrict__ out32) {
+                                      uint32_t* __restrict__ out32, int tiled) {
     const int cols = chunks * 8;  // 32-bit columns per row, padded to whole chunks
     const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (idx >= rows * cols) return;
@@ -115,7 +115,12 @@ __global__ void planes_to_int8_kernel(const uint32_t* __restrict__ words32, int6
         y[s] = (j >= 0 && col < 2 * W64) ? words32[(static_cast<size_t>(row) * S + j) * (2 * W64) + col] : 0u;
     }
     transpose8x8(y);
-    uint4* dst = reinterpret_cast<uint4*>(out32 + (static_cast<size_t>(row) * cols + col) * 8);
+    // row-major [rows][chunks * 256], or tiled [rows / 64][2 chunks half-chunks][64 rows][128 bytes]: the 32 bytes
+    // of column `col` are bytes 32 (col % 4) .. of half-chunk col / 4 of the row
+    const size_t at = tiled ? ((static_cast<size_t>(row >> 6) * (2 * chunks) + (col >> 2)) * 8192 +
+                               static_cast<size_t>(row & 63) * 128 + static_cast<size_t>(col & 3) * 32) / 4
+                            : (static_cast<size_t>(row) * cols + col) * 8;
+    uint4* dst = reinterpret_cast<uint4*>(out32 + at);
     dst[0] = make_uint4(y[0], y[1], y[2], y[3]);
     dst[1] = make_uint4(y[4], y[5], y[6], y[7]);
 }
@@ -819,7 +824,14 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
     const int8_t* __restrict__ K8,  // int8 key image [R, chunks * 256]
     const float* __restrict__ Bw, int Sb, int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv,
     int64_t R_total, float* __restrict__ out, int* __restrict__ chunk_ints, const float* __restrict__ bias,
-    int ndig, long long dig_stride, const long long* __restrict__ key_indices) {
+    int ndig, long long dig_stride, const long long* __restrict__ key_indices, int key_tiled,
+    const unsigned char* __restrict__ warm, long long warm_lines) {
+    // warm / warm_lines: an optional region of 128-byte lines (the keys the NEXT dot will read) that the loader
+    // waves touch once they have issued their last stage, so that it sits in the memory-side cache by the time
+    // that dot runs.  (Issued any earlier, from any wave, these long misses hold up the stage loads queued behind
+    // them in the CU's vector memory path: measured 40 % slower.)
+    // key_tiled: K8 is the tiled image [ceil(R / 64)][2 chunks][64 rows][128 bytes] (a workgroup's key rows of one
+    // half-chunk are contiguous, so cold keys stream from HBM in whole pages) instead of row-major [R][chunks * 256].
     // kI8Sum only: A8 holds ndig digit images of the queries, dig_stride bytes apart, lowest digit first; the
     // chunk loop runs over them from the top digit down and the accumulators are shifted left by 7 between two
     // digits (Horner), so that they end as sum_d (sum_i digit_i[q, d] 128^i) K8[r, d].  With chunk_ints the int32
@@ -844,7 +856,13 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
         // ---- loader wave lw: 8 of the stage's groups of 8 rows (the TM key rows, then the TN query rows: a
         // load moves 1 KiB = 8 rows x 128 bytes), plus the chunk scales of 64 queries once per chunk.
         const int lw = wave - C::kConsumers;
-        const bsi_rsrc rk = make_rsrc(K8 + static_cast<size_t>(r0) * rowbytes, static_cast<size_t>(R - r0) * rowbytes);
+        // tiled keys: blocks of 64 rows x 128 bytes per half-chunk, 2 chunks of them per 64-row tile; rows past R
+        // are zero padding inside the last block, blocks past the last one read as zero (buffer bounds)
+        const size_t kblock = static_cast<size_t>(chunks) * 2 * 8192;  // bytes of a 64-row tile
+        const bsi_rsrc rk = key_tiled ? make_rsrc(K8 + static_cast<size_t>(r0 / 64) * kblock,
+                                                  static_cast<size_t>((R + 63) / 64 - r0 / 64) * kblock)
+                                      : make_rsrc(K8 + static_cast<size_t>(r0) * rowbytes,
+                                                  static_cast<size_t>(R - r0) * rowbytes);
         const bsi_rsrc rq = make_rsrc(A8 + static_cast<size_t>(q0) * rowbytes,
                                       static_cast<size_t>(Q - q0) * rowbytes +
                                           (kSum ? static_cast<size_t>(ndig - 1) * static_cast<size_t>(dig_stride) : 0));
@@ -864,7 +882,11 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
             const int64_t lim = is_key[i] ? (R - r0) : (Q - q0);              // past the end: clamp (never stored)
             const int64_t rr = (rowl < lim) ? rowl : (lim - 1);
             off[i] = static_cast<uint32_t>(rr * rowbytes) + col;
+            if (is_key[i] && key_tiled)
+                off[i] = static_cast<uint32_t>(rowl >> 6) * static_cast<uint32_t>(kblock) +
+                         static_cast<uint32_t>(rowl & 63) * 128 + col;
         }
+        const uint32_t kstep_bytes = key_tiled ? 8192u : 128u;  // from one half-chunk of a key row to the next
         // scales: loader wave lw fetches the 64 queries of group lw % (TN / 64) (waves fetching the same group
         // write their own regions, so that every loader wave has the same number of loads in flight)
         const int sq = (lw % (TN >= 64 ? TN / 64 : 1)) * 64 + lane;
@@ -878,8 +900,9 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
             const int hc = h < halves ? h : halves - 1;
             if (kSum) {
                 if (h < halves) {
-                    so_k = static_cast<uint32_t>(next_c) * 256 + static_cast<uint32_t>(h & 1) * 128;
-                    so_q = so_k + static_cast<uint32_t>(ndig - 1 - next_dg) * static_cast<uint32_t>(dig_stride);
+                    const uint32_t half = static_cast<uint32_t>(next_c) * 2 + static_cast<uint32_t>(h & 1);
+                    so_k = half * kstep_bytes;
+                    so_q = half * 128 + static_cast<uint32_t>(ndig - 1 - next_dg) * static_cast<uint32_t>(dig_stride);
                     if (h & 1) {
                         if (++next_c == chunks) {
                             next_c = 0;
@@ -888,7 +911,8 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
                     }
                 }
             } else {
-                so_k = so_q = static_cast<uint32_t>(hc) * 128;
+                so_q = static_cast<uint32_t>(hc) * 128;
+                so_k = static_cast<uint32_t>(hc) * kstep_bytes;
             }
 #pragma unroll
             for (int i = 0; i < NI; ++i)
@@ -913,6 +937,19 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
             // scale load, 2 NI + 1 instructions, may still be in flight
             asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NI + (kSum ? 0 : 1)) : "memory");
             lds_barrier();
+        }
+        if (warm_lines > 0) {
+            // one lane per 128-byte line, 64 lines per load; this loader wave's share of the region.  The values
+            // are summed only so that the loads stay; the store below never happens.
+            const long long waves = static_cast<long long>(gridDim.x) * gridDim.y * C::kLoaders;
+            const long long mine = (static_cast<long long>(blockIdx.y) * gridDim.x + blockIdx.x) * C::kLoaders + lw;
+            const long long per = (warm_lines + waves - 1) / waves;
+            const long long first = mine * per;
+            const long long last = (first + per < warm_lines) ? first + per : warm_lines;
+            unsigned sum = 0;
+            for (long long l = first + lane; l < last; l += 64)
+                sum += *reinterpret_cast<const volatile unsigned*>(warm + l * 128);
+            if (sum == 0x5ca1ab1eu && warm_lines < 0) scale_lds[lane] = 0;
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still be writing LDS when the workgroup ends
         return;
@@ -1642,13 +1679,25 @@ __global__ void add_bias_kernel(float* __restrict__ out, const float* __restrict
     out[q * R_total + r] = out[q * R_total + r] + bias[r];
 }
 
-static int launch_planes_to_int8(const uint64_t* words, int64_t rows, int S, int W64, int8_t* out, hipStream_t st) {
+__global__ void zero_uint4_kernel(uint4* __restrict__ p, size_t n) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = make_uint4(0u, 0u, 0u, 0u);
+}
+
+static int launch_planes_to_int8(const uint64_t* words, int64_t rows, int S, int W64, int8_t* out, hipStream_t st,
+                                 int tiled = 0) {
     const int chunks = (W64 + 3) / 4;
     const int64_t total = rows * chunks * 8;
     if (total == 0) return BSI_OK;
+    if (tiled && (rows & 63) != 0) {  // the rows that pad the last 64-row tile read as zeros
+        const size_t tile_bytes = static_cast<size_t>(chunks) * 2 * 8192;
+        hipLaunchKernelGGL(zero_uint4_kernel, dim3(static_cast<unsigned>((tile_bytes / 16 + 255) / 256)), dim3(256), 0, st,
+                           reinterpret_cast<uint4*>(out + static_cast<size_t>(rows >> 6) * tile_bytes), tile_bytes / 16);
+        BSI_LAUNCH_CHECK("zero_uint4_kernel");
+    }
     hipLaunchKernelGGL(planes_to_int8_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, st,
                        reinterpret_cast<const uint32_t*>(words), rows, S, W64, chunks,
-                       reinterpret_cast<uint32_t*>(out));
+                       reinterpret_cast<uint32_t*>(out), tiled);
     BSI_LAUNCH_CHECK("planes_to_int8_kernel");
     return BSI_OK;
 }
@@ -1701,11 +1750,15 @@ static void launch_mfma_ws(const int8_t* A8, const float* qscale, int stride, co
                            R_total, out, chunk_ints);
 }
 
+// Set by bsi_hip_dot_bias_warm around its launch: the region the int8-image kernel should touch for the next dot.
+static thread_local const void* g_warm_ptr = nullptr;
+static thread_local size_t g_warm_bytes = 0;
+
 template <int TM, int TN, int kMode>
 static void launch_mfma_i8_tm(const int8_t* A8, const float* qscale, int stride, const int8_t* K8, const float* Bw,
                               int Sb, int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv,
                               int64_t R_total, float* out, int32_t* chunk_ints, const float* bias, hipStream_t st,
-                              int ndig, long long dig_stride, const long long* key_indices) {
+                              int ndig, long long dig_stride, const long long* key_indices, int key_tiled) {
     using C = I8Cfg<TM, TN>;
     const dim3 grid(static_cast<unsigned>((R + TM - 1) / TM), static_cast<unsigned>((Q + TN - 1) / TN));
     static bool configured = false;
@@ -1716,25 +1769,26 @@ static void launch_mfma_i8_tm(const int8_t* A8, const float* qscale, int stride,
     }
     hipLaunchKernelGGL((dot_mfma_i8_kernel<TM, TN, kMode>), grid, dim3(C::kBlock), C::kLds, st, A8, qscale, stride, K8,
                        Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias, ndig, dig_stride,
-                       key_indices);
+                       key_indices, key_tiled, static_cast<const unsigned char*>(g_warm_ptr),
+                       static_cast<long long>(g_warm_bytes / 128));
 }
 
 // Sum mode (ndig >= 1 digit images of the queries; int32 sums into chunk_ints when given, else the float epilogue)
 // or, with ndig == 0, the chain with or without stored integers.
 template <int TM, int TN>
-static void launch_mfma_i8_t(int ndig, long long dig_stride, const long long* key_indices, const int8_t* A8,
+static void launch_mfma_i8_t(int ndig, long long dig_stride, const long long* key_indices, int key_tiled, const int8_t* A8,
                              const float* qscale, int stride, const int8_t* K8, const float* Bw, int Sb, int chunks,
                              int64_t R, int64_t Q, int down_shift, float scale_inv, int64_t R_total, float* out,
                              int32_t* chunk_ints, const float* bias, hipStream_t st) {
     if (ndig > 0)
         launch_mfma_i8_tm<TM, TN, kI8Sum>(A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total,
-                                          out, chunk_ints, bias, st, ndig, dig_stride, key_indices);
+                                          out, chunk_ints, bias, st, ndig, dig_stride, key_indices, key_tiled);
     else if (chunk_ints)
         launch_mfma_i8_tm<TM, TN, kI8Ints>(A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total,
-                                           out, chunk_ints, bias, st, 1, 0, nullptr);
+                                           out, chunk_ints, bias, st, 1, 0, nullptr, key_tiled);
     else
         launch_mfma_i8_tm<TM, TN, kI8Chain>(A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv,
-                                            R_total, out, chunk_ints, bias, st, 1, 0, nullptr);
+                                            R_total, out, chunk_ints, bias, st, 1, 0, nullptr, key_tiled);
 }
 
 // Tile choice.  The 128 x 128 tile moves the fewest operand bytes per MAC and is the fastest whenever its grid
@@ -1760,10 +1814,10 @@ static int choose_i8_tile(int64_t R, int64_t Q, int64_t* cost_out = nullptr) {
 
 static void launch_mfma_i8(const int8_t* A8, const float* qscale, int stride, const int8_t* K8, const float* Bw, int Sb,
                            int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv, int64_t R_total,
-                           float* out, int32_t* chunk_ints, const float* bias, hipStream_t st, int ndig = 0,
-                           long long dig_stride = 0, const long long* key_indices = nullptr) {
+                           float* out, int32_t* chunk_ints, const float* bias, hipStream_t st, int key_tiled = 0,
+                           int ndig = 0, long long dig_stride = 0, const long long* key_indices = nullptr) {
     const int tile = choose_i8_tile(R, Q);
-#define BSI_I8_ARGS ndig, dig_stride, key_indices, A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias, st
+#define BSI_I8_ARGS ndig, dig_stride, key_indices, key_tiled, A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias, st
     if (tile == 128) launch_mfma_i8_t<128, 128>(BSI_I8_ARGS);
     else if (tile == 12864) launch_mfma_i8_t<128, 64>(BSI_I8_ARGS);
     else if (tile == 64) launch_mfma_i8_t<64, 64>(BSI_I8_ARGS);
@@ -1837,6 +1891,20 @@ extern "C" int bsi_hip_planes_to_int8(const uint64_t* words, int64_t rows, int S
     return launch_planes_to_int8(words, rows, S, W64, out, as_stream(stream));
 }
 
+extern "C" size_t bsi_hip_int8_tiled_bytes(int64_t rows, int W64) {
+    if (rows <= 0 || W64 <= 0) return 0;
+    return static_cast<size_t>((rows + 63) / 64) * static_cast<size_t>((W64 + 3) / 4) * 2 * 8192;
+}
+
+extern "C" int bsi_hip_planes_to_int8_tiled(const uint64_t* words, int64_t rows, int S, int W64, int8_t* out,
+                                            void* stream) {
+    BSI_REQUIRE(rows >= 0 && W64 >= 1, "bad shape");
+    BSI_REQUIRE(S >= 1 && S <= 8, "S must be in [1, 8] (got %d)", S);
+    if (rows == 0) return BSI_OK;
+    BSI_REQUIRE(words && out, "null pointer");
+    return launch_planes_to_int8(words, rows, S, W64, out, as_stream(stream), /*tiled=*/1);
+}
+
 extern "C" int bsi_hip_set_option(int option, int value) {
     switch (option) {
         case BSI_OPT_DIGITS_ROUTE:
@@ -1869,7 +1937,8 @@ static int dot_launch(const uint64_t* A, const int8_t* A_ints8, const float* A_c
     BSI_REQUIRE(W64 >= 1, "W64 must be >= 1");
     BSI_REQUIRE(Sa >= 1 && Sa <= 16 && Sb >= 1 && Sb <= 16, "Sa and Sb must be in [1, 16]");
     BSI_REQUIRE(R_total >= R, "R_total must be >= R");
-    BSI_REQUIRE(b_layout == BSI_LAYOUT_CANONICAL || b_layout == BSI_LAYOUT_TILED16 || b_layout == BSI_LAYOUT_INT8,
+    BSI_REQUIRE(b_layout == BSI_LAYOUT_CANONICAL || b_layout == BSI_LAYOUT_TILED16 || b_layout == BSI_LAYOUT_INT8 ||
+                    b_layout == BSI_LAYOUT_INT8_TILED,
                 "unknown key layout %d", b_layout);
     if (Q == 0 || R == 0) return BSI_OK;
     const int chunks = (W64 + 3) / 4;
@@ -1896,10 +1965,11 @@ static int dot_launch(const uint64_t* A, const int8_t* A_ints8, const float* A_c
             A8 = static_cast<const int8_t*>(workspace);
         }
         const int down_shift = 16 - Sa - Sb;
-        if (b_layout == BSI_LAYOUT_INT8) {
+        if (b_layout == BSI_LAYOUT_INT8 || b_layout == BSI_LAYOUT_INT8_TILED) {
             BSI_REQUIRE((reinterpret_cast<uintptr_t>(B) & 15) == 0, "int8 key image must be 16-byte aligned");
             launch_mfma_i8(A8, A_chunk_scales, A_scale_stride, reinterpret_cast<const int8_t*>(B), Bw, Sb, chunks, R, Q,
-                           down_shift, scale_inv, R_total, out, chunk_ints, bias, st);
+                           down_shift, scale_inv, R_total, out, chunk_ints, bias, st,
+                           b_layout == BSI_LAYOUT_INT8_TILED ? 1 : 0);
             BSI_LAUNCH_CHECK("dot_mfma_i8_kernel");
             *bias_fused = true;
             return BSI_OK;
@@ -1933,7 +2003,8 @@ static int dot_launch(const uint64_t* A, const int8_t* A_ints8, const float* A_c
     }
 
     if (core != BSI_CORE_VALU) return fail(BSI_ERR_INVALID, "unknown core %d", core);
-    if (b_layout == BSI_LAYOUT_INT8) return fail(BSI_ERR_UNSUPPORTED, "the popcount core reads key planes, not the int8 image");
+    if (b_layout == BSI_LAYOUT_INT8 || b_layout == BSI_LAYOUT_INT8_TILED)
+        return fail(BSI_ERR_UNSUPPORTED, "the popcount core reads key planes, not the int8 image");
     BSI_REQUIRE(A != nullptr, "VALU core needs the query planes");
     if (Sa == 7 && Sb == 6) {
         if (b_layout == BSI_LAYOUT_TILED16)
@@ -1983,6 +2054,21 @@ extern "C" int bsi_hip_dot_bias(const uint64_t* A, const int8_t* A_ints8, const 
                                 float* out, int core, void* workspace, size_t workspace_bytes, void* stream) {
     return dot_with_bias(A, A_ints8, A_chunk_scales, A_scale_stride, Sa, W64, B, b_layout, Bw, Sb, R, Q, scale_inv,
                          R_total, out, nullptr, core, workspace, workspace_bytes, stream, bias);
+}
+
+extern "C" int bsi_hip_dot_bias_warm(const uint64_t* A, const int8_t* A_ints8, const float* A_chunk_scales,
+                                     int A_scale_stride, int Sa, int W64, const uint64_t* B, int b_layout, const float* Bw,
+                                     int Sb, int64_t R, int64_t Q, float scale_inv, int64_t R_total, const float* bias,
+                                     float* out, int core, void* workspace, size_t workspace_bytes, const void* warm,
+                                     size_t warm_bytes, void* stream) {
+    BSI_REQUIRE(warm != nullptr || warm_bytes == 0, "null warm-up region");
+    g_warm_ptr = warm;
+    g_warm_bytes = warm_bytes;
+    const int rc = dot_with_bias(A, A_ints8, A_chunk_scales, A_scale_stride, Sa, W64, B, b_layout, Bw, Sb, R, Q, scale_inv,
+                                 R_total, out, nullptr, core, workspace, workspace_bytes, stream, bias);
+    g_warm_ptr = nullptr;
+    g_warm_bytes = 0;
+    return rc;
 }
 
 extern "C" int bsi_hip_dot_ewah_query(const uint64_t* comp_words, const int64_t* comp_off, const int32_t* comp_len,
@@ -2101,9 +2187,10 @@ extern "C" size_t bsi_hip_dot_digits_workspace_bytes(int64_t Q, int nq, int64_t 
 extern "C" int bsi_hip_dot_digits(const int8_t* A_digits, int nq, const float* Aw, int Sa, const int8_t* K_digits, int nk,
                                   int preshift, const float* Bw, int Sb, int W64, int64_t R, int64_t Q,
                                   const int64_t* key_indices, float scale_inv, int64_t R_total, const float* bias,
-                                  float* out, void* workspace, size_t workspace_bytes, void* stream) {
+                                  float* out, void* workspace, size_t workspace_bytes, int k_tiled, void* stream) {
     BSI_REQUIRE(R >= 0 && Q >= 0 && W64 >= 1, "bad shape");
     BSI_REQUIRE(nq >= 1 && nq <= 10 && nk >= 1 && nk <= 10, "digit counts must be in [1, 10] (got %d, %d)", nq, nk);
+    BSI_REQUIRE(k_tiled == 0 || nk == 1, "a tiled key image is a single digit");
     BSI_REQUIRE(Sa >= 1 && Sb >= 1 && preshift >= 0 && preshift <= 14, "bad slice counts or preshift");
     BSI_REQUIRE(R_total >= R, "R_total (%lld) < R (%lld)", static_cast<long long>(R_total), static_cast<long long>(R));
     // |sum| <= 256 chunks' worth of 128 * 128 per element: int32 holds D up to 2^17 elements
@@ -2137,7 +2224,7 @@ extern "C" int bsi_hip_dot_digits(const int8_t* A_digits, int nq, const float* A
     const bool fold = g_digits_route == 2 || (g_digits_route == 0 && (nq == 1 || us_fold <= us_stack));
     if (can_fold && fold) {
         launch_mfma_i8(A_digits, Aw, Sa, K_digits, Bw, Sb, chunks, R, Q, preshift, scale_inv, R_total, out, nullptr, bias,
-                       st, nq, dig_stride, reinterpret_cast<const long long*>(key_indices));
+                       st, k_tiled, nq, dig_stride, reinterpret_cast<const long long*>(key_indices));
         BSI_LAUNCH_CHECK("dot_mfma_i8_kernel (int32 sum, digits recombined in the accumulator)");
         return BSI_OK;
     }
@@ -2146,7 +2233,7 @@ extern "C" int bsi_hip_dot_digits(const int8_t* A_digits, int nq, const float* A
                 need);
     // else one int8 GEMM over the stacked digits: I[i Q + q, j R + r] = sum_d A_i[q, d] K_j[r, d]
     launch_mfma_i8(A_digits, Bw, 1, K_digits, Bw, 1, chunks, Rd, Qd, 0, 1.0f, Rd, nullptr,
-                   reinterpret_cast<int32_t*>(workspace), nullptr, st, 1, 0, nullptr);
+                   reinterpret_cast<int32_t*>(workspace), nullptr, st, k_tiled, 1, 0, nullptr);
     BSI_LAUNCH_CHECK("dot_mfma_i8_kernel (int32 sum)");
     const int64_t total = Q * R;
     hipLaunchKernelGGL(digits_combine_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, st,

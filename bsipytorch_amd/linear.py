@@ -145,8 +145,12 @@ class BSIQuantizedLinear(nn.Module):
         fuse_bias = (use_packed and bias is not None and original_dtype == torch.float32 and bias.is_cuda
                      and bias.dtype == torch.float32 and bias.is_contiguous())
         if use_packed:
+            # the layer that runs next (set by quantize_model_bsi): its keys are touched by this dot's kernel so
+            # that they are cache-resident when their turn comes
+            nxt = c.get("_next_bsi_layer")
             scores, ns_total, ns_q, ns_s = bsi_ops.batch_dot_product_multiquery_cuda_batch_caps(
-                qcap, self._bsi_keys_cuda, bias if fuse_bias else None)
+                qcap, self._bsi_keys_cuda, bias if fuse_bias else None,
+                nxt._bsi_keys_cuda if nxt is not None else None)
         else:
             scores, ns_total, ns_q, ns_s = bsi_ops.batch_dot_product_multiquery_cuda_caps(qcap, self._bsi_keys_cuda)
         c["dot_kernel_ns_per_query_last"] = float(ns_q)
@@ -259,9 +263,22 @@ def quantize_model_bsi(model, decimalPlaces=2, skip_lm_head=True, scope="all", c
             module, decimalPlaces=_resolve_layer_value(decimalPlaces, kind, default_decimal),
             compress_threshold=_resolve_layer_value(compress_threshold, kind, default_threshold),
             prefer_cuda=prefer_cuda))
+    link_bsi_layers(model)
     if verbose:
         print(f"Quantized {len(targets)} linear layers to BSI with decimalPlaces={decimalPlaces} (scope={scope})")
     return model
+
+
+def link_bsi_layers(model: nn.Module) -> int:
+    """Tell every BSI layer which one runs after it (module order, the last one wrapping round to the first), so
+    that its dot can warm the cache with the next layer's keys: in a model every keyset has been evicted by the
+    time its layer comes round again, and the dot kernel runs 15-35 % slower on keys that come from HBM.
+    ``BSI_WARM_NEXT=0`` leaves the layers unlinked.  Returns the number of layers linked."""
+    layers = [m for m in model.modules() if isinstance(m, BSIQuantizedLinear)]
+    on = os.getenv("BSI_WARM_NEXT", "1") != "0" and len(layers) > 1
+    for i, m in enumerate(layers):
+        m.__dict__["_next_bsi_layer"] = layers[(i + 1) % len(layers)] if on else None
+    return len(layers) if on else 0
 
 
 def save_bsi_model(model: nn.Module, out_dir: str) -> List[Dict[str, Any]]:
@@ -310,6 +327,7 @@ def load_bsi_model(model: nn.Module, out_dir: str, verbose: bool = False) -> nn.
         setattr(parent, parts[-1], BSIQuantizedLinear(
             shell, decimalPlaces=entry["decimalPlaces"], compress_threshold=entry["compress_threshold"],
             prebuilt_keys=bsi_ops.load_keyset_cuda(layer_dir)))
+    link_bsi_layers(model)
     if verbose:
         print(f"Loaded {len(meta)} BSI layers from {out_dir}")
     return model

@@ -46,6 +46,7 @@ extern "C" {
 #define BSI_LAYOUT_CANONICAL 0 /* [R, Sb, W64] */
 #define BSI_LAYOUT_TILED16 1   /* [ceil(R/16), chunks, Sb, 64, 1] words: see bsi_hip_tile_key_planes */
 #define BSI_LAYOUT_INT8 2      /* int8 [R, chunks*256]: the recombined image bsi_hip_planes_to_int8 writes */
+#define BSI_LAYOUT_INT8_TILED 3 /* the same bytes tiled by 64 rows and half-chunks: bsi_hip_planes_to_int8_tiled */
 
 const char* bsi_hip_version(void);
 const char* bsi_hip_last_error(void);
@@ -159,6 +160,15 @@ int bsi_hip_tile_key_planes(const uint64_t* words_device, int64_t R, int Sb, int
 int bsi_hip_planes_to_int8(const uint64_t* words_device, int64_t rows, int S, int W64, int8_t* out_device,
                            void* stream);
 
+/* The same bytes in the tiled key image [ceil(rows / 64)][2 chunks half-chunks][64 rows][128 bytes] (layout
+ * BSI_LAYOUT_INT8_TILED, bsi_hip_int8_tiled_bytes bytes; rows padding the last tile are zero): the key rows a
+ * workgroup reads for one half-chunk are contiguous, so a keyset that is not cache-resident (every layer of a
+ * model but the last few) streams from HBM in whole pages instead of 128-byte pieces of 64 rows.
+ * No counterpart in the reference. */
+size_t bsi_hip_int8_tiled_bytes(int64_t rows, int W64);
+int bsi_hip_planes_to_int8_tiled(const uint64_t* words_device, int64_t rows, int S, int W64, int8_t* out_device,
+                                 void* stream);
+
 /* Tuning knobs (process-wide, not thread-safe; set before launching).  No counterpart in the reference,
  * whose kernel selection is read from environment variables on every call (bsi_cuda_kernels_dot.cuh:2642). */
 #define BSI_OPT_I8_TILE 1 /* tile of the int8-image kernel: 128 (128 keys x 128 queries), 12864 (128 x 64), 64 (64 x 64)
@@ -201,6 +211,18 @@ int bsi_hip_dot_bias(const uint64_t* A, const int8_t* A_ints8, const float* A_ch
                      float scale_inv, int64_t R_total, const float* bias, float* out, int core, void* workspace,
                      size_t workspace_bytes, void* stream);
 
+/* bsi_hip_dot_bias that also warms the memory-side cache for the NEXT dot: `warm` .. `warm + warm_bytes` (device
+ * memory, typically the key operand of the layer that runs next) is read once, one access per 128-byte line, by
+ * the int8-image kernel's loader waves after they have issued their last stage.  A keyset that is not cache-resident
+ * costs that kernel about 15 to 35 % more than a resident one (its loads wait on HBM latency), and in a model
+ * every keyset is cold by the time its layer comes round again; the hint turns those reads into cache hits.
+ * Results are those of bsi_hip_dot_bias; kernels other than the int8-image one ignore the hint.
+ * No counterpart in the reference. */
+int bsi_hip_dot_bias_warm(const uint64_t* A, const int8_t* A_ints8, const float* A_chunk_scales, int A_scale_stride,
+                          int Sa, int W64, const uint64_t* B, int b_layout, const float* Bw, int Sb, int64_t R, int64_t Q,
+                          float scale_inv, int64_t R_total, const float* bias, float* out, int core, void* workspace,
+                          size_t workspace_bytes, const void* warm, size_t warm_bytes, void* stream);
+
 /* The same dot for ONE query whose slices are EWAH streams (the hybrid query form of
  * build_bsi_query_cuda_hybrid, bsi_cuda.cpp:386-431): stream s at comp_words + comp_off[s], comp_len[s]
  * words, decoded to W64 words per slice inside the kernel's load stage with the semantics of
@@ -236,7 +258,8 @@ int bsi_hip_dot_weighted(const uint64_t* A, const float* Aw, int Sa, int W64, co
  * which is the weighted-slice dot of bsi_hip_dot_weighted whenever the slice weights are the builders' own
  * (w_s = 2^s times a per-row power of two, top slice negative for two's-complement rows).  A fixed-bit key image
  * from bsi_hip_planes_to_int8 is one digit pre-shifted by 8 - S bits; preshift is the sum of both operands'
- * pre-shifts (0 for digit images).  Rows of at most 2^17 elements.
+ * pre-shifts (0 for digit images).  k_tiled != 0: K_digits is one digit in the tiled layout of
+ * bsi_hip_planes_to_int8_tiled.  Rows of at most 2^17 elements.
  * No counterpart in the reference, whose decimal-mode dot is the popcount kernel cited at bsi_hip_dot_weighted. */
 int bsi_hip_planes_to_int8_digits(const uint64_t* words_device, int64_t rows, int S, int W64, int8_t* out_device,
                                   void* stream);
@@ -244,7 +267,7 @@ size_t bsi_hip_dot_digits_workspace_bytes(int64_t Q, int nq, int64_t R, int nk);
 int bsi_hip_dot_digits(const int8_t* A_digits, int nq, const float* Aw, int Sa, const int8_t* K_digits, int nk,
                        int preshift, const float* Bw, int Sb, int W64, int64_t R, int64_t Q,
                        const int64_t* key_indices, float scale_inv, int64_t R_total, const float* bias, float* out,
-                       void* workspace, size_t workspace_bytes, void* stream);
+                       void* workspace, size_t workspace_bytes, int k_tiled, void* stream);
 
 /* Runs fn-independent timing of `iters` back-to-back bsi_hip_dot launches between two HIP events
  * recorded on `stream`, synchronises, and returns the mean launch duration in microseconds.

@@ -311,6 +311,18 @@ _I8_TILES = {"int8": 0, "int8-128": 128, "int8-12864": 12864, "int8-64": 64, "in
 
 
 def _run_dot(hip, qb, kb, Q, R, W, Sa, Sb, core, tiled, with_ints8, want_ints=True, R_total=None):
+    """One bsi_hip_dot call.  With the int8 key image the call is made twice, on the row-major image and on the
+    image tiled by 64 rows and half-chunks, and both must give the same bits."""
+    if tiled in _I8_TILES:
+        ints_a, out_a = _run_dot_once(hip, qb, kb, Q, R, W, Sa, Sb, core, tiled, with_ints8, want_ints, R_total, False)
+        ints_b, out_b = _run_dot_once(hip, qb, kb, Q, R, W, Sa, Sb, core, tiled, with_ints8, want_ints, R_total, True)
+        assert np.array_equal(out_a, out_b, equal_nan=True)
+        assert ints_a is None or np.array_equal(ints_a, ints_b)
+        return ints_b, out_b
+    return _run_dot_once(hip, qb, kb, Q, R, W, Sa, Sb, core, tiled, with_ints8, want_ints, R_total, False)
+
+
+def _run_dot_once(hip, qb, kb, Q, R, W, Sa, Sb, core, tiled, with_ints8, want_ints, R_total, image_tiled):
     L = hip.lib
     chunks = (W + 3) // 4
     A = dev(qb["words"])
@@ -320,9 +332,14 @@ def _run_dot(hip, qb, kb, Q, R, W, Sa, Sb, core, tiled, with_ints8, want_ints=Tr
     layout = 0
     if tiled in _I8_TILES:   # the cached int8 image of the key integers; tile forced or automatic
         hip.check(L.bsi_hip_set_option(hip.OPT_I8_TILE, _I8_TILES[tiled]), "set_option")
-        Bi = torch.full((R, chunks * 256), 77, dtype=torch.int8, device="cuda")
-        hip.check(L.bsi_hip_planes_to_int8(B.data_ptr(), R, Sb, W, Bi.data_ptr(), st()), "key image")
-        B, layout = Bi, 2
+        if image_tiled:
+            Bi = torch.full((int(L.bsi_hip_int8_tiled_bytes(R, W)),), 77, dtype=torch.int8, device="cuda")
+            hip.check(L.bsi_hip_planes_to_int8_tiled(B.data_ptr(), R, Sb, W, Bi.data_ptr(), st()), "key image")
+            B, layout = Bi, 3
+        else:
+            Bi = torch.full((R, chunks * 256), 77, dtype=torch.int8, device="cuda")
+            hip.check(L.bsi_hip_planes_to_int8(B.data_ptr(), R, Sb, W, Bi.data_ptr(), st()), "key image")
+            B, layout = Bi, 2
     elif tiled:
         Bt = torch.full((((R + 15) // 16) * chunks * Sb * 64,), -1, dtype=torch.int64, device="cuda")
         hip.check(L.bsi_hip_tile_key_planes(B.data_ptr(), R, Sb, W, Bt.data_ptr(), st()), "tile")
@@ -1171,9 +1188,10 @@ def test_digit_images_match_oracle(hip, oracle, Q, d, scale):
     assert got.shape == want.shape and np.array_equal(got, want)
 
 
-def _run_digits(hip, a_dig, aw, Sa, k_dig, preshift, bw, Sb, W, Q, R, key_indices=None, R_total=None, bias=None):
+def _run_digits(hip, a_dig, aw, Sa, k_dig, preshift, bw, Sb, W, Q, R, key_indices=None, R_total=None, bias=None,
+                k_tiled=0):
     L = hip.lib
-    nq, nk = a_dig.shape[0], k_dig.shape[0]
+    nq, nk = a_dig.shape[0], (1 if k_tiled else k_dig.shape[0])
     R_total = R if R_total is None else R_total
     out = torch.full((Q, R_total), float("nan"), dtype=torch.float32, device="cuda")
     nbytes = int(L.bsi_hip_dot_digits_workspace_bytes(Q, nq, R, nk))
@@ -1184,7 +1202,7 @@ def _run_digits(hip, a_dig, aw, Sa, k_dig, preshift, bw, Sb, W, Q, R, key_indice
     hip.check(L.bsi_hip_dot_digits(a_dig.data_ptr(), nq, Aw.data_ptr(), Sa, k_dig.data_ptr(), nk, preshift, Bw.data_ptr(),
                                    Sb, W, R, Q, idx.data_ptr() if idx is not None else None, float(np.float32(1e-4)),
                                    R_total, bias.data_ptr() if bias is not None else None, out.data_ptr(), ws.data_ptr(),
-                                   nbytes, st()), "digit dot")
+                                   nbytes, k_tiled, st()), "digit dot")
     torch.cuda.synchronize()
     return out.cpu().numpy()
 
@@ -1226,9 +1244,13 @@ def test_dot_digits_fixed_images_indices_bias_and_stride(hip, oracle):
     a_dig = _digits_dev(hip, a["words"])
     perm = np.random.default_rng(3).permutation(60)[:R]
     bias = torch.randn(R, device="cuda")
+    k8t = torch.full((int(hip.lib.bsi_hip_int8_tiled_bytes(R, W)),), 77, dtype=torch.int8, device="cuda")
+    hip.check(hip.lib.bsi_hip_planes_to_int8_tiled(dev(b["words"]).data_ptr(), R, 6, W, k8t.data_ptr(), st()), "image")
     for route in (1, 2):
         hip.check(hip.lib.bsi_hip_set_option(hip.OPT_DIGITS_ROUTE, route), "opt")
         got = _run_digits(hip, a_dig, a["slice_weights"], a["S"], k8, 2, b["slice_weights"], 6, W, Q, R)
+        assert np.array_equal(got, want), route
+        got = _run_digits(hip, a_dig, a["slice_weights"], a["S"], k8t, 2, b["slice_weights"], 6, W, Q, R, k_tiled=1)
         assert np.array_equal(got, want), route
         got = _run_digits(hip, a_dig, a["slice_weights"], a["S"], k8, 2, b["slice_weights"], 6, W, Q, R, key_indices=perm,
                           R_total=60, bias=bias)
@@ -1265,3 +1287,72 @@ def test_ops_decimal_mfma_and_popcount_routes_agree(ops, monkeypatch):
     assert torch.equal(outs["0"], outs["1"])
     dense = (X.double() @ K.double().T).float().cuda()
     assert (outs["1"] - dense).abs().max().item() < 2048 * 0.005 * 4.0
+
+
+@pytest.mark.parametrize("R,d", [(64, 256), (150, 2048), (1, 64), (200, 700)])
+def test_tiled_key_image_holds_the_row_major_bytes(hip, oracle, R, d):
+    """[ceil(R/64)][2 chunks][64][128]: half-chunk h of row r sits at tile r // 64, block h, row r % 64; padding rows
+    are zero."""
+    rng = np.random.default_rng(R)
+    k = (rng.standard_normal((R, d)) * 0.02).astype(np.float32)
+    kb = oracle.build_keys(k, 2, 6)
+    W = (d + 63) // 64
+    chunks = (W + 3) // 4
+    words = dev(kb["words"])
+    rows = torch.empty((R, chunks * 256), dtype=torch.int8, device="cuda")
+    hip.check(hip.lib.bsi_hip_planes_to_int8(words.data_ptr(), R, 6, W, rows.data_ptr(), st()), "rows")
+    nbytes = int(hip.lib.bsi_hip_int8_tiled_bytes(R, W))
+    tiles = (R + 63) // 64
+    assert nbytes == tiles * chunks * 2 * 8192
+    tiled = torch.full((nbytes,), 77, dtype=torch.int8, device="cuda")
+    hip.check(hip.lib.bsi_hip_planes_to_int8_tiled(words.data_ptr(), R, 6, W, tiled.data_ptr(), st()), "tiled")
+    t = tiled.view(tiles, chunks * 2, 64, 128).permute(0, 2, 1, 3).reshape(tiles * 64, chunks * 256)
+    assert torch.equal(t[:R], rows) and not t[R:].any()
+
+
+def test_warm_hint_changes_nothing_but_the_cache(ops, oracle):
+    """bsi_hip_dot_bias_warm: same bits as without the hint, for every tile, with and without a bias; the warmed
+    region is only read."""
+    rng = np.random.default_rng(12)
+    Q, R, d = 70, 150, 2048
+    x = rng.standard_normal((Q, d)).astype(np.float32)
+    k = (rng.standard_normal((R, d)) * 0.02).astype(np.float32)
+    kcap, *_ = ops.build_bsi_keys_cuda(torch.from_numpy(k), 2, 0.5)
+    other, *_ = ops.build_bsi_keys_cuda(torch.from_numpy(k[::-1].copy()), 2, 0.5)
+    before = other.ints8.clone()
+    qcap = ops.build_bsi_queries_cuda_batch_packed(torch.from_numpy(x).cuda(), 2, 0.5)
+    bias = torch.randn(R, device="cuda")
+    from bsipytorch_amd import _lib
+    for tile in (0, 128, 12864, 64, 6432):
+        _lib.check(_lib.lib.bsi_hip_set_option(_lib.OPT_I8_TILE, tile), "opt")
+        for b in (None, bias):
+            plain, *_ = ops.batch_dot_product_multiquery_cuda_batch_caps(qcap, kcap, b)
+            warm, *_ = ops.batch_dot_product_multiquery_cuda_batch_caps(qcap, kcap, b, other)
+            assert torch.equal(plain, warm), (tile, b is not None)
+    _lib.check(_lib.lib.bsi_hip_set_option(_lib.OPT_I8_TILE, 0), "opt")
+    assert torch.equal(other.ints8, before)
+    # few query rows stream the planes; the hint is accepted there too
+    q1 = ops.build_bsi_queries_cuda_batch_packed(torch.from_numpy(x[:3]).cuda(), 2, 0.5)
+    a, *_ = ops.batch_dot_product_multiquery_cuda_batch_caps(q1, kcap)
+    b2, *_ = ops.batch_dot_product_multiquery_cuda_batch_caps(q1, kcap, None, other)
+    assert torch.equal(a, b2)
+
+
+def test_quantized_model_links_layers_for_the_warm_hint(ops, monkeypatch):
+    from bsipytorch_amd import linear
+
+    torch.manual_seed(3)
+    model = torch.nn.Sequential(torch.nn.Linear(256, 128), torch.nn.ReLU(), torch.nn.Linear(128, 256),
+                                torch.nn.ReLU(), torch.nn.Linear(256, 64)).cuda()
+    x = torch.randn(40, 256, device="cuda")
+    monkeypatch.setenv("BSI_WARM_NEXT", "0")
+    linear.quantize_model_bsi(model, decimalPlaces=2, compress_threshold=0.5, verbose=False)
+    assert all(m.__dict__["_next_bsi_layer"] is None for m in model if isinstance(m, linear.BSIQuantizedLinear))
+    with torch.no_grad():
+        want = model(x)
+    monkeypatch.setenv("BSI_WARM_NEXT", "1")
+    assert linear.link_bsi_layers(model) == 3
+    assert model[0].__dict__["_next_bsi_layer"] is model[2] and model[4].__dict__["_next_bsi_layer"] is model[0]
+    with torch.no_grad():
+        got = model(x)
+    assert torch.equal(got, want)
