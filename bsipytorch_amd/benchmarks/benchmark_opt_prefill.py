@@ -119,7 +119,7 @@ def time_forward(model, input_ids, iters: int, warmup: int):
 
 
 def run(model_name="opt-1.3b", seq_len=512, batch=1, iters=5, warmup=2, decimal_places=2, compress_threshold=0.5,
-        seed=123, dense=True, graph=True):
+        seed=123, dense=True, graph=True, fuse_qkv=False):
     from bsipytorch_amd import bsi_ops, linear
 
     assert torch.cuda.is_available(), "needs the GPU"
@@ -138,7 +138,9 @@ def run(model_name="opt-1.3b", seq_len=512, batch=1, iters=5, warmup=2, decimal_
         res["dense_fp32_tokens_per_s"] = tokens / (med * 1e-3)
 
     t0 = time.perf_counter()
-    linear.quantize_model_bsi(model, decimalPlaces=decimal_places, compress_threshold=compress_threshold, verbose=False)
+    linear.quantize_model_bsi(model, decimalPlaces=decimal_places, compress_threshold=compress_threshold, verbose=False,
+                              fuse_qkv=fuse_qkv)
+    res["fuse_qkv"] = bool(fuse_qkv)
     torch.cuda.synchronize()
     res["key_build_s"] = time.perf_counter() - t0
     summary = linear.summarize_bsi_model(model)
@@ -223,9 +225,10 @@ def main():
     ap.add_argument("--seed", type=int, default=123)
     ap.add_argument("--no_dense", action="store_true")
     ap.add_argument("--no_graph", action="store_true", help="skip the HIP-graph replay leg")
+    ap.add_argument("--fuse_qkv", action="store_true", help="one dot for q_proj, k_proj and v_proj of a layer")
     a = ap.parse_args()
     print(json.dumps(run(a.model, a.seq_len, a.batch, a.iters, a.warmup, a.decimal_places, a.compress_threshold,
-                         a.seed, not a.no_dense, not a.no_graph)))
+                         a.seed, not a.no_dense, not a.no_graph, a.fuse_qkv)))
 
 
 if __name__ == "__main__":

@@ -599,6 +599,47 @@ def build_bsi_keys_cuda(K: torch.Tensor, decimal_places: int, compress_threshold
     return h, int(total_bytes), int(R), int(d), int(h.W)
 
 
+def concat_keysets(keysets: List["PrebuiltBSIKeysCUDA"]) -> "PrebuiltBSIKeysCUDA":
+    """One fixed-bit keyset holding the rows of several (same width, slice count and decimals), in order: the
+    planes, slice weights and shifts are concatenated on the device and the dot's representations derived anew,
+    so every row keeps exactly the bits it had.  No counterpart in the reference."""
+    _check(len(keysets) > 0, "no keysets to concatenate")
+    k0 = keysets[0]
+    for k in keysets:
+        _capsule(k, PrebuiltBSIKeysCUDA, "Invalid CUDA keys capsule")
+        _check(k.fixed and k.shifts is not None, "only fixed-bit keysets can be concatenated")
+        _check((k.W, k.d, k.Sb, k.decimals) == (k0.W, k0.d, k0.Sb, k0.decimals), "keysets differ in shape or precision")
+    h = PrebuiltBSIKeysCUDA()
+    h.num_keys, h.d, h.W, h.Sb = sum(k.num_keys for k in keysets), k0.d, k0.W, k0.Sb
+    h.decimals, h.threshold = k0.decimals, k0.threshold
+    h.slice_weights = torch.cat([k.slice_weights for k in keysets]).contiguous()
+    h.shifts = torch.cat([k.shifts for k in keysets]).contiguous()
+    _install_fixed_key_planes(h, torch.cat([canonical_key_planes(k) for k in keysets]).contiguous())
+    return h
+
+
+def keyset_rows(keys: "PrebuiltBSIKeysCUDA", start: int, stop: int) -> "PrebuiltBSIKeysCUDA":
+    """Rows start .. stop of a fixed-bit keyset as a keyset of their own that shares its memory (views); both
+    bounds must be multiples of 64 or the end of the keyset, so that tiles are not split."""
+    _capsule(keys, PrebuiltBSIKeysCUDA, "Invalid CUDA keys capsule")
+    _check(keys.fixed, "only fixed-bit keysets can be viewed by rows")
+    _check(0 <= start < stop <= keys.num_keys and start % 64 == 0 and (stop % 64 == 0 or stop == keys.num_keys),
+           "row bounds must be multiples of 64 within the keyset")
+    h = PrebuiltBSIKeysCUDA()
+    h.num_keys, h.d, h.W, h.Sb = stop - start, keys.d, keys.W, keys.Sb
+    h.decimals, h.threshold, h.layout = keys.decimals, keys.threshold, keys.layout
+    h.slice_weights, h.shifts = keys.slice_weights[start:stop], keys.shifts[start:stop]
+    h.words = keys.words[start // 16:(stop + 15) // 16] if keys.layout == _lib.LAYOUT_TILED16 else keys.words[start:stop]
+    if keys.ints8 is not None:
+        h.ints8_tiled = keys.ints8_tiled
+        if keys.ints8_tiled:
+            tile = ((keys.W + 3) // 4) * 2 * 8192
+            h.ints8 = keys.ints8[(start // 64) * tile:((stop + 63) // 64) * tile]
+        else:
+            h.ints8 = keys.ints8[start:stop]
+    return h
+
+
 # --------------------------------------------------------------------------- keyset files
 
 _KEYSET_MAGIC = b"BSIKEYS1"

@@ -144,13 +144,19 @@ class BSIQuantizedLinear(nn.Module):
         # precision the reference adds it after the cast, so it stays a separate addition there
         fuse_bias = (use_packed and bias is not None and original_dtype == torch.float32 and bias.is_cuda
                      and bias.dtype == torch.float32 and bias.is_contiguous())
-        if use_packed:
+        fused = c.get("_fused") if use_packed else None
+        if fused is not None:
+            # this layer shares its input with siblings (q/k/v): one dot over their stacked keys serves all of them
+            group, start, stop = fused
+            all_scores, ns_total, ns_q, ns_s, bias_done = group.scores(qcap, fuse_bias)
+            scores = all_scores[:, start:stop]
+            fuse_bias = fuse_bias and bias_done
+        elif use_packed:
             # the layer that runs next (set by quantize_model_bsi): its keys are touched by this dot's kernel so
             # that they are cache-resident when their turn comes
             nxt = c.get("_next_bsi_layer")
             scores, ns_total, ns_q, ns_s = bsi_ops.batch_dot_product_multiquery_cuda_batch_caps(
-                qcap, self._bsi_keys_cuda, bias if fuse_bias else None,
-                nxt._bsi_keys_cuda if nxt is not None else None)
+                qcap, self._bsi_keys_cuda, bias if fuse_bias else None, _keys_to_warm(nxt))
         else:
             scores, ns_total, ns_q, ns_s = bsi_ops.batch_dot_product_multiquery_cuda_caps(qcap, self._bsi_keys_cuda)
         c["dot_kernel_ns_per_query_last"] = float(ns_q)
@@ -169,6 +175,65 @@ class BSIQuantizedLinear(nn.Module):
         if len(original_shape) != 2:
             scores = scores.view(*original_shape[:-1], -1)
         return scores
+
+
+def _keys_to_warm(layer):
+    """The keyset a dot should warm for `layer` (the whole stacked keyset when that layer is part of a fused group)."""
+    if layer is None:
+        return None
+    fused = layer.__dict__.get("_fused")
+    return fused[0].keys if fused is not None else layer._bsi_keys_cuda
+
+
+class _FusedSiblings:
+    """Layers fed by the same activation tensor (q_proj / k_proj / v_proj), served by ONE dot over their stacked
+    keys; each member takes its columns of the result.  The result is kept for the query build it was computed
+    from (the members share one build per input), so the first member called does the work."""
+
+    def __init__(self, members):
+        self.members = list(members)
+        self.keys = bsi_ops.concat_keysets([m._bsi_keys_cuda for m in self.members])
+        biases = [m.bias for m in self.members]
+        self.bias = torch.cat([b.to(torch.float32) for b in biases]).contiguous() if all(b is not None for b in biases) else None
+        self.next_layer = None
+        self._last = None
+
+    def scores(self, qcap, want_bias):
+        """(scores of all members [Q, sum of out_features], dot times, whether the bias is already added)."""
+        last = self._last
+        if last is not None and last[0] is qcap:  # siblings share one query build: the same handle means the same input
+            return last[1], 0, 0.0, 0.0, last[2]
+        bias_done = bool(want_bias and self.bias is not None)
+        out, ns_total, ns_q, ns_s = bsi_ops.batch_dot_product_multiquery_cuda_batch_caps(
+            qcap, self.keys, self.bias if bias_done else None, _keys_to_warm(self.next_layer))
+        self._last = (qcap, out, bias_done)
+        return out, ns_total, ns_q, ns_s, bias_done
+
+
+def fuse_sibling_layers(model: nn.Module, names=("q_proj", "k_proj", "v_proj")) -> int:
+    """Stack the keys of BSI layers that are children of one module under the given names (the attention
+    projections, which read the same activations) so that one dot serves them all: three launches over 2048 key
+    rows each become one over 6144, which fills the GPU with the large tile.  Every output element is computed
+    from the same query row and key row as before, so the results are bit-identical.  The members' own keysets
+    become views into the stacked one.  Returns the number of groups formed.  Not in the reference."""
+    groups = 0
+    for parent in model.modules():
+        kids = [getattr(parent, n, None) for n in names]
+        if not all(isinstance(k, BSIQuantizedLinear) for k in kids) or any(k.__dict__.get("_fused") for k in kids):
+            continue
+        k0 = kids[0]
+        if any((k.in_features, k.decimalPlaces) != (k0.in_features, k0.decimalPlaces) or not k._bsi_keys_cuda.fixed
+               or k.out_features % 64 != 0 for k in kids):
+            continue
+        group = _FusedSiblings(kids)
+        start = 0
+        for k in kids:
+            k.__dict__["_fused"] = (group, start, start + k.out_features)
+            k._bsi_keys_cuda = bsi_ops.keyset_rows(group.keys, start, start + k.out_features)
+            start += k.out_features
+        groups += 1
+    link_bsi_layers(model)
+    return groups
 
 
 _COUNTERS = ("dot_ns_total", "dot_calls", "build_ns_total", "build_quantize_ns_total", "build_pack_ns_total",
@@ -233,7 +298,7 @@ _MLP_TOKENS = ("mlp", "ff", "ffn", "fc1", "fc2")
 
 
 def quantize_model_bsi(model, decimalPlaces=2, skip_lm_head=True, scope="all", compress_threshold=0.2,
-                       prefer_cuda: bool = True, verbose: bool = True):
+                       prefer_cuda: bool = True, verbose: bool = True, fuse_qkv: bool = False):
     """Replace every ``nn.Linear`` (except ``lm_head``) by ``BSIQuantizedLinear``; ``scope`` is
     'all' | 'attention' | 'mlp', chosen by name tokens (verify_accuracy_bsi.py:444-486)."""
     default_decimal = float(decimalPlaces if isinstance(decimalPlaces, (int, float)) else decimalPlaces.get("default", 2))
@@ -264,6 +329,8 @@ def quantize_model_bsi(model, decimalPlaces=2, skip_lm_head=True, scope="all", c
             compress_threshold=_resolve_layer_value(compress_threshold, kind, default_threshold),
             prefer_cuda=prefer_cuda))
     link_bsi_layers(model)
+    if fuse_qkv:  # not in the reference's signature: see fuse_sibling_layers
+        fuse_sibling_layers(model)
     if verbose:
         print(f"Quantized {len(targets)} linear layers to BSI with decimalPlaces={decimalPlaces} (scope={scope})")
     return model
@@ -278,6 +345,11 @@ def link_bsi_layers(model: nn.Module) -> int:
     on = os.getenv("BSI_WARM_NEXT", "1") != "0" and len(layers) > 1
     for i, m in enumerate(layers):
         m.__dict__["_next_bsi_layer"] = layers[(i + 1) % len(layers)] if on else None
+    for i, m in enumerate(layers):  # a fused group warms the first layer after its last member
+        fused = m.__dict__.get("_fused")
+        if fused is not None and m is fused[0].members[-1]:
+            nxt = m.__dict__["_next_bsi_layer"]
+            fused[0].next_layer = nxt if (nxt is not None and nxt.__dict__.get("_fused", (None,))[0] is not fused[0]) else None
     return len(layers) if on else 0
 
 

@@ -827,8 +827,8 @@ def test_linear_drop_in(ops, oracle):
     assert isinstance(m.q_proj, BSIQuantizedLinear) and isinstance(m.fc1, BSIQuantizedLinear)
     assert isinstance(m.lm_head, torch.nn.Linear)
     m.cuda()
-    got = m(inp.cuda()).cpu()
-    cos = float((got * dense).sum() / (torch.linalg.norm(got) * torch.linalg.norm(dense)))
+    got = m(inp.cuda()).detach().cpu()
+    cos = float((got * dense.detach()).sum() / (torch.linalg.norm(got) * torch.linalg.norm(dense.detach())))
     assert cos > 0.9, cos
     assert sum_bsi_dot_query_vectors(m) == 6
     m2 = Tiny()
@@ -1356,3 +1356,64 @@ def test_quantized_model_links_layers_for_the_warm_hint(ops, monkeypatch):
     with torch.no_grad():
         got = model(x)
     assert torch.equal(got, want)
+
+
+def test_fused_sibling_layers_are_bit_identical(ops, oracle):
+    """q_proj / k_proj / v_proj served by one dot over their stacked keys: same bits as three dots; keyset
+    concatenation and row views keep every row's planes, weights and shifts."""
+    from bsipytorch_amd import linear
+
+    class Attn(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.q_proj = torch.nn.Linear(512, 128)
+            self.k_proj = torch.nn.Linear(512, 128)
+            self.v_proj = torch.nn.Linear(512, 192, bias=False)   # not all biased: members add their own
+            self.out_proj = torch.nn.Linear(128, 512)
+
+        def forward(self, x):
+            return self.out_proj(self.q_proj(x) * self.k_proj(x)) + self.v_proj(x).sum(-1, keepdim=True)
+
+    class Block(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.a, self.b = Attn(), Attn()
+
+        def forward(self, x):
+            return self.b(self.a(x))
+
+    torch.manual_seed(5)
+    model = Block().cuda()
+    with torch.no_grad():
+        model.b.v_proj.weight.mul_(3.0)
+    x = torch.randn(2, 40, 512, device="cuda")
+    linear.quantize_model_bsi(model, decimalPlaces=2, compress_threshold=0.5, verbose=False)
+    with torch.no_grad():
+        want = model(x)
+        want_q = model.a.q_proj(x)
+    planes_before = [ops.canonical_key_planes(m._bsi_keys_cuda).clone() for m in (model.a.q_proj, model.a.k_proj, model.a.v_proj)]
+    assert linear.fuse_sibling_layers(model) == 2
+    g = model.a.q_proj.__dict__["_fused"][0]
+    assert g.keys.num_keys == 128 + 128 + 192 and g.bias is None and g.next_layer is model.a.out_proj
+    assert model.a.out_proj.__dict__["_next_bsi_layer"] is model.b.q_proj
+    for m, before in zip((model.a.q_proj, model.a.k_proj, model.a.v_proj), planes_before):
+        assert torch.equal(ops.canonical_key_planes(m._bsi_keys_cuda), before)
+    with torch.no_grad():
+        got = model(x)
+        got_q = model.a.q_proj(x)
+    assert torch.equal(got, want) and torch.equal(got_q, want_q) and got_q.shape == (2, 40, 128)
+    # all members biased: the stacked bias goes into the dot
+    torch.manual_seed(6)
+    m2 = Attn().cuda()
+    m2.v_proj = torch.nn.Linear(512, 192).cuda()
+    linear.quantize_model_bsi(m2, decimalPlaces=2, compress_threshold=0.5, verbose=False)
+    with torch.no_grad():
+        want2 = m2(x)
+    linear.fuse_sibling_layers(m2)
+    assert m2.q_proj.__dict__["_fused"][0].bias is not None
+    with torch.no_grad():
+        assert torch.equal(m2(x), want2)
+    # a second, different input must not be served from the first one's result
+    with torch.no_grad():
+        y = m2(x * 2.0)
+    assert not torch.equal(y, want2)
