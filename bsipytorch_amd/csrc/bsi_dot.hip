@@ -17,6 +17,11 @@
 //           dot_mfma_ws_kernel       many rows on tiled planes (producer waves recombine the planes)
 //           dot_mfma_kernel          canonical planes or slice counts other than 6
 //
+// Operands whose slice count follows the data (decimal mode) carry float slice weights instead of scales:
+//   dot_weighted_kernel      popcounts per slice pair, summed exactly in float64 (any Sa, Sb <= 64)
+//   dot_mfma_i8_kernel in its int32-sum mode on int8 digit images (planes_to_digits_kernel), the digits put back
+//   together in the accumulator or by digits_combine_kernel: the same sum on the matrix cores
+//
 // Both feed the same fp32 epilogue, in chunk order:  acc = fmaf((float)I, qscale[q,c], acc), then
 // out = (acc * bscale[r]) * scale_inv.  bscale is a power of two, so hoisting it out of the chain is
 // exact and the result is bit-identical to fmaf((float)I, qscale*bscale, acc) of the reference
@@ -1991,9 +1996,8 @@ static int dot_launch(const uint64_t* A, const int8_t* A_ints8, const float* A_c
             BSI_LAUNCH_CHECK("dot_mfma_ws_kernel");
             return BSI_OK;
         }
-        if (Sb == 6) {
-            if (tiled) launch_mfma<6, true>(A8, A_chunk_scales, A_scale_stride, B, Bw, Sb, W64, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, st);
-            else launch_mfma<6, false>(A8, A_chunk_scales, A_scale_stride, B, Bw, Sb, W64, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, st);
+        if (Sb == 6) {  // canonical planes (the tiled ones went to the kernels above)
+            launch_mfma<6, false>(A8, A_chunk_scales, A_scale_stride, B, Bw, Sb, W64, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, st);
         } else {
             if (tiled) launch_mfma<0, true>(A8, A_chunk_scales, A_scale_stride, B, Bw, Sb, W64, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, st);
             else launch_mfma<0, false>(A8, A_chunk_scales, A_scale_stride, B, Bw, Sb, W64, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, st);
