@@ -172,9 +172,30 @@ class BSIQuantizedLinear(nn.Module):
             if bias.dtype != original_dtype or bias.device != scores.device:
                 bias = bias.to(device=scores.device, dtype=original_dtype)
             scores = scores + bias
+        if c.get("collect_stats") and self.weight_fp32 is not None:
+            self._track_error(batch_inputs, scores)
         if len(original_shape) != 2:
             scores = scores.view(*original_shape[:-1], -1)
         return scores
+
+    @torch.no_grad()
+    def _track_error(self, batch_inputs, scores):
+        """Error of this forward against the dense fp32 layer, accumulated per sample (row)."""
+        w = self.weight_fp32.to(batch_inputs.device)
+        ref = batch_inputs.to(torch.float32) @ w.t()
+        if self.bias is not None:
+            ref = ref + self.bias.to(torch.float32)
+        got = scores.to(torch.float32)
+        err = got - ref
+        n = int(ref.shape[0])
+        c = self.__dict__
+        if "samples_tracked" not in c:
+            self.reset_error_stats()
+        c["mse_sum"] += float(err.pow(2).mean(dim=1).sum())
+        c["mae_sum"] += float(err.abs().mean(dim=1).sum())
+        c["cosine_sum"] += float(torch.nn.functional.cosine_similarity(got, ref, dim=1).sum())
+        c["max_abs_error"] = max(c["max_abs_error"], float(err.abs().max()))
+        c["samples_tracked"] += n
 
 
 def _keys_to_warm(layer):
@@ -273,6 +294,16 @@ def summarize_bsi_model(model: nn.Module) -> Dict[str, Any]:
                                 decimalPlaces=m.decimalPlaces, compress_threshold=m.compress_threshold,
                                 weight_bsi_bytes=m.weight_bsi_memory_bytes, weight_dense_bytes=m.weight_dense_memory_bytes,
                                 bias_bytes=m.bias_memory_bytes, weight_fp16_bytes=fp16_bytes))
+        # device keysets hold every slice verbatim (EWAH is applied to hybrid queries only)
+        keys = m._bsi_keys_cuda
+        slices = int(keys.num_keys * keys.Sb)
+        disk = int(bsi_ops.keyset_size_on_disk_cuda(keys)[1])
+        s["layers"][-1].update(weight_total_slices=slices, weight_verbatim_slices=slices, weight_compressed_slices=0,
+                               weight_compressed_pct=0.0, weight_verbatim_pct=100.0 if slices else 0.0,
+                               weight_bsi_disk_bytes=disk)
+        s["total_slices"] += slices
+        s["verbatim_slices"] += slices
+        s["total_bsi_disk_bytes"] = s.get("total_bsi_disk_bytes", 0) + disk
         s["total_bsi_bytes"] += m.weight_bsi_memory_bytes
         s["total_dense_bytes"] += m.weight_dense_memory_bytes
         s["total_bias_bytes"] += m.bias_memory_bytes
@@ -281,8 +312,83 @@ def summarize_bsi_model(model: nn.Module) -> Dict[str, Any]:
     s["total_static_bytes"] = s["total_bsi_bytes"] + s["total_bias_bytes"]
     s["total_dense_with_bias_bytes"] = s["total_dense_bytes"] + s["total_bias_bytes"]
     s["compressed_pct"] = 0.0
-    s["verbatim_pct"] = 0.0
+    s["verbatim_pct"] = 100.0 if s["total_slices"] else 0.0
     return s
+
+
+def enable_bsi_error_stats(model: nn.Module, enabled: bool) -> None:
+    """Toggle per-layer error tracking (verify_accuracy_bsi.py:282-290).  While it is on, every forward of a BSI
+    layer also computes the dense fp32 result from the kept weights and accumulates MSE, MAE, cosine similarity
+    and the largest absolute error (a debugging mode: it costs a dense matmul per layer)."""
+    for module in model.modules():
+        if isinstance(module, BSIQuantizedLinear):
+            if enabled and not module.collect_stats:
+                module.collect_stats = True
+                module.reset_error_stats()
+            elif not enabled:
+                module.collect_stats = False
+
+
+def collect_bsi_error_stats(model: nn.Module) -> List[Dict[str, float]]:
+    """Accumulated per-layer error metrics, worst MSE first (verify_accuracy_bsi.py:293-310)."""
+    out: List[Dict[str, float]] = []
+    for name, m in model.named_modules():
+        if isinstance(m, BSIQuantizedLinear) and getattr(m, "samples_tracked", 0) > 0:
+            n = float(m.samples_tracked)
+            out.append({"name": name, "decimalPlaces": m.decimalPlaces, "compress_threshold": m.compress_threshold,
+                        "samples_tracked": n, "mse": m.mse_sum / n, "mae": m.mae_sum / n, "cosine": m.cosine_sum / n,
+                        "max_abs": m.max_abs_error})
+    out.sort(key=lambda item: item["mse"], reverse=True)
+    return out
+
+
+def get_model_static_bytes(model: nn.Module) -> int:
+    """Parameters plus buffers, in bytes (benchmark_performance_bsi.py:488-492)."""
+    return int(sum(p.nelement() * p.element_size() for p in model.parameters())
+               + sum(b.nelement() * b.element_size() for b in model.buffers()))
+
+
+def bsi_full_model_static_bytes(model: nn.Module, summary: Dict[str, Any]) -> int:
+    """Static size of a BSI-quantised model: parameters and buffers (the non-BSI modules and the BSI biases) plus
+    the BSI key bytes, which are not parameters (verify_accuracy_bsi.py:389-402)."""
+    return get_model_static_bytes(model) + int(summary.get("total_bsi_bytes", 0))
+
+
+def compression_summary_lines(summary: Dict[str, Any]):
+    """(one line per layer, (compressed slices, all slices, percentage)) -- verify_accuracy_bsi.py:405-418."""
+    lines = []
+    for idx, layer in enumerate(summary.get("layers", []), start=1):
+        total = int(layer.get("weight_total_slices", 0) or 0)
+        compressed = int(layer.get("weight_compressed_slices", 0) or 0)
+        pct = (compressed * 100.0 / total) if total else 0.0
+        lines.append(f"Layer {idx} ({layer.get('name', f'Layer {idx}')}): {compressed}/{total} ({pct:.2f}%)")
+    total = int(summary.get("total_slices", 0) or 0)
+    compressed = int(summary.get("compressed_slices", 0) or 0)
+    return lines, (compressed, total, (compressed * 100.0 / total) if total else 0.0)
+
+
+def print_compression_summary(summary: Dict[str, Any], heading: str = "Compression Summary") -> None:
+    """verify_accuracy_bsi.py:421-432."""
+    lines, (compressed, total, pct) = compression_summary_lines(summary)
+    print(f"\n=== {heading} ===")
+    if not lines and total == 0:
+        print("No compression statistics available.")
+        return
+    for line in lines:
+        print(line)
+    print(f"Overall compressed slices: {compressed}/{total} ({pct:.2f}%)")
+
+
+def build_layer_config(default_value, attention_value, mlp_value):
+    """Per-scope configuration for quantize_model_bsi (benchmark_performance_bsi.py:494-503)."""
+    if attention_value is None and mlp_value is None:
+        return default_value
+    config = {"default": default_value}
+    if attention_value is not None:
+        config["attention"] = attention_value
+    if mlp_value is not None:
+        config["mlp"] = mlp_value
+    return config
 
 
 def _resolve_layer_value(config: Union[float, Dict[str, float]], layer_kind: str, fallback: float) -> float:

@@ -1417,3 +1417,38 @@ def test_fused_sibling_layers_are_bit_identical(ops, oracle):
     with torch.no_grad():
         y = m2(x * 2.0)
     assert not torch.equal(y, want2)
+
+
+def test_model_harness_helpers(ops, capsys):
+    """Error statistics, byte accounting and compression summary of a quantised model (the reference's harness
+    helpers, verify_accuracy_bsi.py:282-432 and benchmark_performance_bsi.py:488-503)."""
+    from bsipytorch_amd import linear
+
+    torch.manual_seed(9)
+    model = torch.nn.Sequential(torch.nn.Linear(256, 128), torch.nn.ReLU(), torch.nn.Linear(128, 64, bias=False)).cuda()
+    dense_bytes = linear.get_model_static_bytes(model)
+    assert dense_bytes == (256 * 128 + 128 + 128 * 64) * 4
+    cfg = linear.build_layer_config(2, None, 3)
+    assert cfg == {"default": 2, "mlp": 3} and linear.build_layer_config(2, None, None) == 2
+    linear.quantize_model_bsi(model, decimalPlaces=2, compress_threshold=0.5, verbose=False)
+    summary = linear.summarize_bsi_model(model)
+    assert summary["num_quantized_layers"] == 2 and summary["total_slices"] == (128 + 64) * 6
+    assert summary["layers"][0]["weight_bsi_disk_bytes"] > 128 * 6 * 4 * 8
+    assert linear.bsi_full_model_static_bytes(model, summary) == 128 * 4 + summary["total_bsi_bytes"]
+    lines, overall = linear.compression_summary_lines(summary)
+    assert len(lines) == 2 and overall == (0, (128 + 64) * 6, 0.0)
+    linear.print_compression_summary(summary)
+    assert "Overall compressed slices: 0/1152" in capsys.readouterr().out
+    x = torch.randn(10, 256, device="cuda")
+    linear.enable_bsi_error_stats(model, True)
+    with torch.no_grad():
+        model(x)
+        model(x)
+    stats = linear.collect_bsi_error_stats(model)
+    assert len(stats) == 2 and all(s["samples_tracked"] == 20 for s in stats)
+    assert all(s["cosine"] > 0.9 and s["mse"] >= 0 and s["max_abs"] > 0 for s in stats)
+    assert stats[0]["mse"] >= stats[1]["mse"]
+    linear.enable_bsi_error_stats(model, False)
+    with torch.no_grad():
+        model(x)
+    assert linear.collect_bsi_error_stats(model)[0]["samples_tracked"] == 20
