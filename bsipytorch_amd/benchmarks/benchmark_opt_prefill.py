@@ -119,7 +119,7 @@ def time_forward(model, input_ids, iters: int, warmup: int):
 
 
 def run(model_name="opt-1.3b", seq_len=512, batch=1, iters=5, warmup=2, decimal_places=2, compress_threshold=0.5,
-        seed=123, dense=True, graph=True, fuse_qkv=False):
+        seed=123, dense=True, graph=True, fuse_qkv=False, quantize_lm_head=False):
     from bsipytorch_amd import bsi_ops, linear
 
     assert torch.cuda.is_available(), "needs the GPU"
@@ -139,8 +139,9 @@ def run(model_name="opt-1.3b", seq_len=512, batch=1, iters=5, warmup=2, decimal_
 
     t0 = time.perf_counter()
     linear.quantize_model_bsi(model, decimalPlaces=decimal_places, compress_threshold=compress_threshold, verbose=False,
-                              fuse_qkv=fuse_qkv)
+                              fuse_qkv=fuse_qkv, skip_lm_head=not quantize_lm_head)
     res["fuse_qkv"] = bool(fuse_qkv)
+    res["lm_head"] = "bsi" if quantize_lm_head else "dense"
     torch.cuda.synchronize()
     res["key_build_s"] = time.perf_counter() - t0
     summary = linear.summarize_bsi_model(model)
@@ -226,9 +227,11 @@ def main():
     ap.add_argument("--no_dense", action="store_true")
     ap.add_argument("--no_graph", action="store_true", help="skip the HIP-graph replay leg")
     ap.add_argument("--fuse_qkv", action="store_true", help="one dot for q_proj, k_proj and v_proj of a layer")
+    ap.add_argument("--quantize_lm_head", action="store_true",
+                    help="also replace lm_head (the reference's harness keeps it dense; this is an extra figure)")
     a = ap.parse_args()
     print(json.dumps(run(a.model, a.seq_len, a.batch, a.iters, a.warmup, a.decimal_places, a.compress_threshold,
-                         a.seed, not a.no_dense, not a.no_graph, a.fuse_qkv)))
+                         a.seed, not a.no_dense, not a.no_graph, a.fuse_qkv, a.quantize_lm_head)))
 
 
 if __name__ == "__main__":
