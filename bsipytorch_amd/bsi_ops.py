@@ -864,6 +864,39 @@ def _dot_weighted(words, slice_weights, Sa, W, keys: PrebuiltBSIKeysCUDA, Q, dec
     return out, ns
 
 
+FUSED_LINEAR_MAX_ROWS = 4
+
+
+def can_fuse_linear_few_rows(x2d: torch.Tensor, keys: "PrebuiltBSIKeysCUDA") -> bool:
+    """Whether linear_few_rows_cuda serves this call: a few rows, 7-or-so-bit chunk-scaled queries without
+    clipping, fixed 6-plane tiled keys, the matrix-core route not switched off."""
+    f = _flags()
+    d = int(x2d.shape[1])
+    return (0 < x2d.shape[0] <= FUSED_LINEAR_MAX_ROWS and x2d.is_cuda and x2d.is_contiguous()
+            and x2d.dtype in (torch.float32, torch.float16, torch.bfloat16)
+            and keys.fixed and keys.Sb == 6 and keys.layout == _lib.LAYOUT_TILED16 and keys.d == d
+            and 2 <= f["bits_q"] <= 8 and f["chunk_scale"] and f["clip_k"] == 0.0 and ((d + 63) // 64) % 4 == 0
+            and d <= 8192 * 256 and f["core"] != _lib.CORE_VALU and not f["profile"]
+            and os.environ.get("BSI_TC_DOT", "1").strip() != "0" and os.environ.get("BSI_FUSED_LINEAR", "1").strip() != "0")
+
+
+def linear_few_rows_cuda(x2d: torch.Tensor, keyset_cuda_cap, decimal_places: int, bias=None) -> torch.Tensor:
+    """out[Q, R] float32 = BSI dot of the rows of ``x2d`` (Q <= 4) with the keyset, query build included, in one
+    launch (bsi_hip_linear_few_rows): what build_bsi_queries_cuda_batch_packed followed by
+    batch_dot_product_multiquery_cuda_batch_caps returns, bit for bit.  Not in the reference."""
+    keys = _capsule(keyset_cuda_cap, PrebuiltBSIKeysCUDA, "Invalid CUDA keys capsule")
+    _check(x2d.dim() == 2 and can_fuse_linear_few_rows(x2d, keys), "linear_few_rows_cuda: call not served by the fused kernel")
+    _check(int(decimal_places) == keys.decimals,
+           f"Decimal mismatch between queries and keys: q={int(decimal_places)} k={keys.decimals}")
+    Q, R = int(x2d.shape[0]), keys.num_keys
+    out = torch.empty((Q, R), dtype=torch.float32, device=x2d.device)
+    check(lib.bsi_hip_linear_few_rows(x2d.data_ptr(), _dtype_code(x2d), Q, int(x2d.shape[1]), int(decimal_places),
+                                      _flags()["bits_q"], keys.words.data_ptr(), keys.slice_weights.data_ptr(), keys.Sb,
+                                      R, _scale_inv(int(decimal_places), keys.decimals), R, _ptr(bias), out.data_ptr(),
+                                      _stream()), "bsi_hip_linear_few_rows")
+    return out
+
+
 def _dot_result(out, ns, Q, R):
     per_q = float(ns) / float(Q) if Q > 0 else 0.0
     per_s = float(ns) / (float(Q) * float(R)) if (Q > 0 and R > 0) else 0.0

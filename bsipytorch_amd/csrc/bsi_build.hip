@@ -17,14 +17,6 @@ namespace bsi {
 constexpr int kBlock = 256;
 constexpr int kWavesPerBlock = kBlock / BSI_WAVE;
 
-// Position of element e (0..255) of a chunk inside the chunk's 256 int8 bytes in the MFMA core's
-// order: element 32w + 8m + t sits at byte 32w + 4t + m (see planes_to_int8 in bsi_dot.hip).
-__device__ __forceinline__ int mfma_byte_pos(int e) {
-    const int w = e >> 5, r = e & 31;
-    const int m = r >> 3, t = r & 7;
-    return (w << 5) + (t << 2) + m;
-}
-
 // ---------------------------------------------------------------- elementwise
 
 template <typename T>

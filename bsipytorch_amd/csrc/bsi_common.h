@@ -108,6 +108,14 @@ __device__ __forceinline__ long long shift_clamp(long long v, int shift, long lo
     return out;
 }
 
+// Position of element e (0..255) of a chunk inside the chunk's 256 int8 bytes in the MFMA core's
+// order: element 32w + 8m + t sits at byte 32w + 4t + m (see planes_to_int8 in bsi_dot.hip).
+__device__ __forceinline__ int mfma_byte_pos(int e) {
+    const int w = e >> 5, r = e & 31;
+    const int m = r >> 3, t = r & 7;
+    return (w << 5) + (t << 2) + m;
+}
+
 // wave64 butterfly reductions (every lane ends with the result)
 __device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long v) {
 #pragma unroll

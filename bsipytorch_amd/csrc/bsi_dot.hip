@@ -1303,6 +1303,175 @@ __global__ __launch_bounds__(1024) void dot_mfma_stream_kernel(
     }
 }
 
+// The few-rows kernel with the query build inside (at most kFusedMaxQ rows: a decode step).  The wave that takes
+// chunk c quantises that chunk of every query row itself -- round half away of x * 10^dec, the chunk's shift
+// from its largest magnitude, rounded shift and clamp, exactly the builder's per-chunk routine -- into its own
+// LDS image, takes the MFMA operand from there and leaves the chunk scale in LDS for the chain.  Every workgroup
+// repeats that small amount of arithmetic (the kernel waits on the key planes, the VALU is idle), and a BSI-linear
+// layer becomes ONE launch instead of a build and a dot.  Same integers, scales and fp32 chain as
+// bsi_hip_build_fixed + bsi_hip_dot, so the same bits.
+constexpr int kFusedMaxQ = 4;
+
+template <typename T, int KT>
+__global__ __launch_bounds__(1024) void dot_mfma_stream_fused_kernel(
+    const T* __restrict__ x, int64_t d, double dec_scale, int slices,
+    const unsigned long long* __restrict__ B64,  // tiled key planes, Sb = 6
+    const float* __restrict__ Bw, int chunks, int pass_chunks, int64_t R, int Q, float scale_inv, int64_t R_total,
+    float* __restrict__ out, const float* __restrict__ bias) {
+    // [pass_chunks][KT][16 queries][16 keys] ints | [waves][kFusedMaxQ][256] image bytes | [chunks][kFusedMaxQ] scales
+    extern __shared__ __attribute__((aligned(16))) int ints[];
+    constexpr int kSlot = KT * 256;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nwaves = static_cast<int>(blockDim.x >> 6);
+    const int ln = lane & 15, lg = lane >> 4;
+    unsigned char* const qimg = reinterpret_cast<unsigned char*>(ints + static_cast<size_t>(pass_chunks) * kSlot) +
+                                static_cast<size_t>(wave) * (kFusedMaxQ * 256);
+    float* const qsc = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(ints + static_cast<size_t>(pass_chunks) * kSlot) +
+                                                static_cast<size_t>(nwaves) * (kFusedMaxQ * 256));
+    const int64_t ntiles = (R + 15) / 16;
+    const int64_t tile0 = static_cast<int64_t>(blockIdx.x) * KT;
+    const size_t ktile = static_cast<size_t>(chunks) * (6 * 64);  // words per key tile
+    const unsigned long long* ksrc[KT];
+#pragma unroll
+    for (int k = 0; k < KT; ++k) {
+        const int64_t t = (tile0 + k < ntiles) ? tile0 + k : ntiles - 1;  // clamped: its outputs are never stored
+        ksrc[k] = B64 + static_cast<size_t>(t) * ktile + lane;
+    }
+    const int down_shift = 16 - slices - 6;
+    const long long qmax = (1LL << (slices - 1)) - 1LL, qmin = -(1LL << (slices - 1));
+
+    // the chain lanes: tid <-> (key tile, query, key), keys fastest so output stores are contiguous
+    float accf = 0.0f;
+    const int ck = tid >> 8, cn = (tid >> 4) & 15, ckey = tid & 15;
+    const int64_t cr = (tile0 + ck) * 16 + ckey;
+    const bool cvalid = tid < kSlot && cn < Q && cr < R;
+    const float down = __uint_as_float(static_cast<uint32_t>(127 - down_shift) << 23);
+
+    for (int p0 = 0; p0 < chunks; p0 += pass_chunks) {
+        const int pend = (p0 + pass_chunks < chunks) ? p0 + pass_chunks : chunks;
+        int c = p0 + wave;
+        uint2 kc[KT][6];
+        float xc[kFusedMaxQ][4];  // the wave's chunk of the activations, element k * 64 + lane (0 past the end)
+        auto load_x = [&](int chunk, float (&dst)[kFusedMaxQ][4]) {
+            const int64_t s0 = static_cast<int64_t>(chunk) * BSI_CHUNK_ELEMS;
+#pragma unroll
+            for (int q = 0; q < kFusedMaxQ; ++q)
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const int64_t e = s0 + k * BSI_WAVE + lane;
+                    dst[q][k] = (q < Q && e < d) ? load_as_float<T>(x, static_cast<int64_t>(q) * d + e) : 0.0f;
+                }
+        };
+        if (c < pend) {
+#pragma unroll
+            for (int k = 0; k < KT; ++k)
+#pragma unroll
+                for (int j = 0; j < 6; ++j) {
+                    const unsigned long long w = ksrc[k][(static_cast<size_t>(c) * 6 + j) * 64];
+                    kc[k][j] = make_uint2(static_cast<uint32_t>(w), static_cast<uint32_t>(w >> 32));
+                }
+            load_x(c, xc);
+        }
+        for (; c < pend; c += nwaves) {
+            // the key planes and the activations of the wave's next chunk first, then this chunk's query build
+            uint2 kn[KT][6];
+            float xn[kFusedMaxQ][4];
+            const int cnext = c + nwaves;
+            if (cnext < pend) {
+#pragma unroll
+                for (int k = 0; k < KT; ++k)
+#pragma unroll
+                    for (int j = 0; j < 6; ++j) {
+                        const unsigned long long w = ksrc[k][(static_cast<size_t>(cnext) * 6 + j) * 64];
+                        kn[k][j] = make_uint2(static_cast<uint32_t>(w), static_cast<uint32_t>(w >> 32));
+                    }
+                load_x(cnext, xn);
+            }
+            const int64_t start = static_cast<int64_t>(c) * BSI_CHUNK_ELEMS;
+            const int valid = static_cast<int>((d - start) < BSI_CHUNK_ELEMS ? (d - start) : BSI_CHUNK_ELEMS);
+#pragma unroll
+            for (int q = 0; q < kFusedMaxQ; ++q) {
+                if (q >= Q) break;  // uniform
+                long long r[4];
+                unsigned long long mx = 0ULL;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const int e = k * BSI_WAVE + lane;
+                    r[k] = 0;
+                    if (e < valid) {
+                        r[k] = round_scaled(xc[q][k], dec_scale);
+                        const unsigned long long av = uabs_ll(r[k]);
+                        if (av > mx) mx = av;
+                    }
+                }
+                mx = wave_max_u64(mx);
+                const int shift = (valid > 0) ? compute_shift(mx, 0.0, valid, slices, 0.0f) : 0;
+                if (lane == 0) qsc[c * kFusedMaxQ + q] = static_cast<float>(1ULL << shift);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const int e = k * BSI_WAVE + lane;
+                    const long long v = (e < valid) ? shift_clamp(r[k], shift, qmin, qmax) : 0;
+                    qimg[q * 256 + mfma_byte_pos(e)] = static_cast<unsigned char>(static_cast<int>(v) << (8 - slices));
+                }
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            v4i qb[4];
+            if (ln < Q) {
+                const v4i* src = reinterpret_cast<const v4i*>(qimg + ln * 256 + lg * 64);
+#pragma unroll
+                for (int m = 0; m < 4; ++m) qb[m] = src[m];
+            } else {
+#pragma unroll
+                for (int m = 0; m < 4; ++m) qb[m] = (v4i){0, 0, 0, 0};
+            }
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            __builtin_amdgcn_wave_barrier();  // the image is rewritten for the wave's next chunk
+#pragma unroll
+            for (int k = 0; k < KT; ++k) {
+                uint32_t lo[8], hi[8];
+                transpose_6planes(kc[k][0].x, kc[k][1].x, kc[k][2].x, kc[k][3].x, kc[k][4].x, kc[k][5].x, lo);
+                transpose_6planes(kc[k][0].y, kc[k][1].y, kc[k][2].y, kc[k][3].y, kc[k][4].y, kc[k][5].y, hi);
+                v4i ka[4];
+                ka[0] = (v4i){static_cast<int>(lo[0]), static_cast<int>(lo[1]), static_cast<int>(lo[2]), static_cast<int>(lo[3])};
+                ka[1] = (v4i){static_cast<int>(lo[4]), static_cast<int>(lo[5]), static_cast<int>(lo[6]), static_cast<int>(lo[7])};
+                ka[2] = (v4i){static_cast<int>(hi[0]), static_cast<int>(hi[1]), static_cast<int>(hi[2]), static_cast<int>(hi[3])};
+                ka[3] = (v4i){static_cast<int>(hi[4]), static_cast<int>(hi[5]), static_cast<int>(hi[6]), static_cast<int>(hi[7])};
+                v4i acc = {0, 0, 0, 0};
+#pragma unroll
+                for (int m = 0; m < 4; ++m) acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(ka[m], qb[m], acc, 0, 0, 0);
+                // the lane holds keys 4*lg .. 4*lg+3 of query ln
+                *reinterpret_cast<v4i*>(&ints[(c - p0) * kSlot + k * 256 + ln * 16 + lg * 4]) = acc;
+            }
+            if (cnext < pend) {
+#pragma unroll
+                for (int k = 0; k < KT; ++k)
+#pragma unroll
+                    for (int j = 0; j < 6; ++j) kc[k][j] = kn[k][j];
+#pragma unroll
+                for (int q = 0; q < kFusedMaxQ; ++q)
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) xc[q][k] = xn[q][k];
+            }
+        }
+        __syncthreads();
+        if (cvalid) {
+            for (int cc = p0; cc < pend; ++cc) {
+                const int v = ints[(cc - p0) * kSlot + tid];
+                accf = fmaf(static_cast<float>(v), qsc[cc * kFusedMaxQ + cn] * down, accf);
+            }
+        }
+        if (pend < chunks) __syncthreads();
+    }
+    if (cvalid) {
+        float v = (accf * Bw[cr * 6]) * scale_inv;
+        if (bias != nullptr) v = v + bias[cr];
+        out[static_cast<size_t>(cn) * R_total + cr] = v;
+    }
+}
+
 // ------------------------------------------------------------------ one EWAH-compressed query, decode inline
 //
 // The hybrid query form keeps each of its Sa slices as an EWAH stream ([marker][literals...],
@@ -2073,6 +2242,65 @@ extern "C" int bsi_hip_dot_bias_warm(const uint64_t* A, const int8_t* A_ints8, c
     g_warm_ptr = nullptr;
     g_warm_bytes = 0;
     return rc;
+}
+
+template <typename T, int KT>
+static void launch_stream_fused(const T* x, int64_t d, double dec_scale, int slices, const uint64_t* B, const float* Bw,
+                                int chunks, int64_t R, int Q, float scale_inv, int64_t R_total, float* out,
+                                const float* bias, hipStream_t st) {
+    constexpr int kSlot = KT * 256;
+    const int64_t ntiles = (R + 15) / 16;
+    const dim3 grid(static_cast<unsigned>((ntiles + KT - 1) / KT));
+    int waves = (grid.x <= 256) ? 16 : 8;  // as the few-rows kernel: one workgroup per CU gets more waves
+    if (waves > chunks) waves = chunks;
+    if (waves < kSlot / 64) waves = kSlot / 64;
+    int pass_chunks = kStreamLdsInts / kSlot;
+    if (pass_chunks > chunks) pass_chunks = chunks;
+    const size_t lds = static_cast<size_t>(pass_chunks) * kSlot * sizeof(int) +
+                       static_cast<size_t>(waves) * kFusedMaxQ * 256 + static_cast<size_t>(chunks) * kFusedMaxQ * sizeof(float);
+    static bool configured = false;
+    if (!configured) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dot_mfma_stream_fused_kernel<T, KT>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        configured = true;
+    }
+    hipLaunchKernelGGL((dot_mfma_stream_fused_kernel<T, KT>), grid, dim3(waves * 64), lds, st, x, d, dec_scale, slices,
+                       reinterpret_cast<const unsigned long long*>(B), Bw, chunks, pass_chunks, R, Q, scale_inv, R_total,
+                       out, bias);
+}
+
+extern "C" int bsi_hip_linear_few_rows(const void* x, int dtype, int64_t Q, int64_t d, int decimal_places, int fixed_bits,
+                                       const uint64_t* B_tiled, const float* Bw, int Sb, int64_t R, float scale_inv,
+                                       int64_t R_total, const float* bias, float* out, void* stream) {
+    BSI_REQUIRE(Q >= 0 && R >= 0 && d >= 1, "bad shape");
+    BSI_REQUIRE(Q <= kFusedMaxQ, "the fused few-rows kernel takes at most %d query rows (got %lld)", kFusedMaxQ,
+                static_cast<long long>(Q));
+    BSI_REQUIRE(fixed_bits >= 2 && fixed_bits <= 8, "fixed_bits must be in [2, 8] (got %d)", fixed_bits);
+    BSI_REQUIRE(R_total >= R, "R_total must be >= R");
+    if (Sb != 6) return fail(BSI_ERR_UNSUPPORTED, "the fused few-rows kernel reads 6-plane tiled keys (got Sb = %d)", Sb);
+    const int W64 = static_cast<int>((d + 63) / 64);
+    if (W64 % 4 != 0)
+        return fail(BSI_ERR_UNSUPPORTED, "chunk scales need a multiple of 4 words per slice (d = %lld)", static_cast<long long>(d));
+    if (Q == 0 || R == 0) return BSI_OK;
+    BSI_REQUIRE(x && B_tiled && Bw && out, "null pointer");
+    const int chunks = W64 / 4;
+    if (static_cast<size_t>(chunks) * kFusedMaxQ * sizeof(float) > 32 * 1024)
+        return fail(BSI_ERR_UNSUPPORTED, "rows of %lld elements do not fit the scale buffer", static_cast<long long>(d));
+    const double dec_scale = pow(10.0, static_cast<double>(decimal_places));
+    hipStream_t st = as_stream(stream);
+    const bool two = (R + 15) / 16 >= 1024;  // as bsi_hip_dot: two key tiles per workgroup once the GPU is full
+#define BSI_FUSED(T)                                                                                              \
+    if (two) launch_stream_fused<T, 2>(static_cast<const T*>(x), d, dec_scale, fixed_bits, B_tiled, Bw, chunks, R,    \
+                                       static_cast<int>(Q), scale_inv, R_total, out, bias, st);                       \
+    else launch_stream_fused<T, 1>(static_cast<const T*>(x), d, dec_scale, fixed_bits, B_tiled, Bw, chunks, R,        \
+                                   static_cast<int>(Q), scale_inv, R_total, out, bias, st);
+    if (dtype == BSI_DTYPE_F32) { BSI_FUSED(float) }
+    else if (dtype == BSI_DTYPE_F16) { BSI_FUSED(__half) }
+    else if (dtype == BSI_DTYPE_BF16) { BSI_FUSED(__hip_bfloat16) }
+    else return fail(BSI_ERR_INVALID, "unknown dtype %d", dtype);
+#undef BSI_FUSED
+    BSI_LAUNCH_CHECK("dot_mfma_stream_fused_kernel");
+    return BSI_OK;
 }
 
 extern "C" int bsi_hip_dot_ewah_query(const uint64_t* comp_words, const int64_t* comp_off, const int32_t* comp_len,

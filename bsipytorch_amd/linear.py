@@ -127,6 +127,10 @@ class BSIQuantizedLinear(nn.Module):
 
         # the counters live in the instance dict: nn.Module.__setattr__ costs more than the rest of this method
         c = self.__dict__
+        if q_rows <= bsi_ops.FUSED_LINEAR_MAX_ROWS:
+            scores = self._forward_few_rows(batch_inputs, original_dtype)
+            if scores is not None:
+                return scores.view(*original_shape[:-1], -1) if len(original_shape) != 2 else scores
         t0 = time.perf_counter_ns()
         use_packed = os.getenv("BSI_QUERY_PACKED", "1") != "0"
         qcap, reused = _cached_query_build(batch_inputs, self.decimalPlaces, float(self.query_compress_threshold),
@@ -176,6 +180,45 @@ class BSIQuantizedLinear(nn.Module):
             self._track_error(batch_inputs, scores)
         if len(original_shape) != 2:
             scores = scores.view(*original_shape[:-1], -1)
+        return scores
+
+    def _forward_few_rows(self, batch_inputs, original_dtype):
+        """A decode step (at most 4 rows): query build and dot in one launch, or None when that kernel does not
+        serve the call.  Siblings that share their input (fused q/k/v) share the launch."""
+        c = self.__dict__
+        fused = c.get("_fused")
+        keys = fused[0].keys if fused is not None else self._bsi_keys_cuda
+        if c.get("collect_stats") or not bsi_ops.can_fuse_linear_few_rows(batch_inputs, keys):
+            return None
+        # The fused kernel saves the host a launch and the handles of a query build, which is what an eager decode
+        # step is bound by; on the GPU it costs what it saves (every workgroup repeats the quantisation), so a
+        # forward that is being captured into a graph, where host time does not count, keeps the two launches.
+        if torch.cuda.is_current_stream_capturing():
+            return None
+        fp32 = original_dtype == torch.float32
+        if fused is not None:
+            group, start, stop = fused
+            key = (batch_inputs.data_ptr(), tuple(batch_inputs.shape), batch_inputs.dtype, batch_inputs._version)
+            last = group.__dict__.get("_last_few")
+            if last is not None and last[0] == key:
+                scores, bias_done = last[2][:, start:stop], last[3]
+            else:
+                gb = group.bias if (fp32 and group.bias is not None) else None
+                all_scores = bsi_ops.linear_few_rows_cuda(batch_inputs, keys, self.decimalPlaces, gb)
+                group.__dict__["_last_few"] = (key, batch_inputs, all_scores, gb is not None)  # holds the input's storage
+                scores, bias_done = all_scores[:, start:stop], gb is not None
+                c["dot_calls"] += 1
+        else:
+            b = self.bias if (fp32 and self.bias is not None and self.bias.dtype == torch.float32) else None
+            scores, bias_done = bsi_ops.linear_few_rows_cuda(batch_inputs, keys, self.decimalPlaces, b), b is not None
+            c["dot_calls"] += 1
+        q_rows = int(batch_inputs.shape[0])
+        c["dot_query_vectors_total"] += q_rows
+        c["dot_output_elements_total"] += q_rows * int(self.out_features)
+        if scores.dtype != original_dtype:
+            scores = scores.to(dtype=original_dtype)
+        if self.bias is not None and not bias_done:
+            scores = scores + self.bias.to(device=scores.device, dtype=original_dtype)
         return scores
 
     @torch.no_grad()

@@ -223,6 +223,17 @@ int bsi_hip_dot_bias_warm(const uint64_t* A, const int8_t* A_ints8, const float*
                           float scale_inv, int64_t R_total, const float* bias, float* out, int core, void* workspace,
                           size_t workspace_bytes, const void* warm, size_t warm_bytes, void* stream);
 
+/* A whole BSI-linear layer for at most 4 activation rows (a decode step) in ONE launch: the chunk-scale query
+ * build of bsi_hip_build_fixed (x [Q, d] of dtype, decimal_places, fixed_bits in [2, 8], no clipping) is done
+ * inside the few-rows dot kernel, by the wave that takes each chunk, and the result is that of
+ * bsi_hip_build_fixed followed by bsi_hip_dot_bias on the tiled planes, bit for bit.  d must give a multiple of
+ * 4 words per slice (chunk scales), Sb must be 6.  Replaces, for such calls, the sequence
+ * build_bsi_queries_cuda_batch_packed + batch_dot_product_multiquery_cuda_batch_caps of a layer forward
+ * (verify_accuracy_bsi.py:143-178). */
+int bsi_hip_linear_few_rows(const void* x_device, int dtype, int64_t Q, int64_t d, int decimal_places, int fixed_bits,
+                            const uint64_t* B_tiled, const float* Bw, int Sb, int64_t R, float scale_inv, int64_t R_total,
+                            const float* bias, float* out, void* stream);
+
 /* The same dot for ONE query whose slices are EWAH streams (the hybrid query form of
  * build_bsi_query_cuda_hybrid, bsi_cuda.cpp:386-431): stream s at comp_words + comp_off[s], comp_len[s]
  * words, decoded to W64 words per slice inside the kernel's load stage with the semantics of

@@ -1462,3 +1462,96 @@ def test_collect_bsi_shape_stats(ops):
     linear.quantize_model_bsi(model, decimalPlaces=2, compress_threshold=0.5, verbose=False)
     res = cs.collect(model)
     assert res["W"] == {4: 1, 2: 1} and res["Sb"] == {6: 192} and [r[0] for r in res["layers"]] == ["0", "2"]
+
+
+# ------------------------------------------------------------------ fused build + dot for a few rows
+
+
+@pytest.mark.parametrize("Q", [1, 2, 3, 4])
+@pytest.mark.parametrize("R,d,kind", [(200, 2048, "randn"), (33, 4096, "outliers"), (16400, 1024, "relu"), (75, 700 + 68, "ties")])
+def test_linear_few_rows_matches_build_plus_dot(hip, oracle, Q, R, d, kind):
+    """bsi_hip_linear_few_rows against the oracle's build + dot (so also against the two-launch path, which the
+    other tests hold to the same oracle): one or two key tiles per workgroup, ragged D (768 = 3 chunks), a chunk of
+    zeros, an outlier."""
+    L = hip.lib
+    x = _inputs(max(Q, 3), d, seed=Q * 13 + R, kind=kind)[:Q]
+    rng = np.random.default_rng(R)
+    k = (rng.standard_normal((R, d)) * 0.02).astype(np.float32)
+    qb, kb = oracle.build_queries(x, 2, 7), oracle.build_keys(k, 2, 6)
+    assert qb["chunk_scale"]
+    _, want = oracle.dot_fixed(qb["words"], qb["scales"], kb["words"], kb["scales"], oracle.scale_inv(2, 2), want_ints=False)
+    W = (d + 63) // 64
+    chunks = W // 4
+    B = dev(kb["words"])
+    Bt = torch.full((((R + 15) // 16) * chunks * 6 * 64,), -1, dtype=torch.int64, device="cuda")
+    hip.check(L.bsi_hip_tile_key_planes(B.data_ptr(), R, 6, W, Bt.data_ptr(), st()), "tile")
+    Bw = dev(kb["slice_weights"])
+    xd = torch.from_numpy(x).cuda()
+    bias = torch.randn(R, device="cuda")
+    for b in (None, bias):
+        out = torch.full((Q, R + 3), float("nan"), dtype=torch.float32, device="cuda")
+        hip.check(L.bsi_hip_linear_few_rows(xd.data_ptr(), hip.DTYPE_F32, Q, d, 2, 7, Bt.data_ptr(), Bw.data_ptr(), 6, R,
+                                            float(oracle.scale_inv(2, 2)), R + 3, b.data_ptr() if b is not None else None,
+                                            out.data_ptr(), st()), "fused")
+        got = out.cpu().numpy()
+        expect = want if b is None else want + b.cpu().numpy()[None, :]
+        assert np.array_equal(got[:, :R], expect.astype(np.float32))
+        assert np.isnan(got[:, R:]).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_linear_few_rows_half_inputs_and_limits(hip, oracle, dtype):
+    L = hip.lib
+    torch.manual_seed(3)
+    xh = (torch.randn(2, 1024) * 3).to(dtype)
+    x = xh.to(torch.float32).numpy()
+    k = (np.random.default_rng(1).standard_normal((40, 1024)) * 0.02).astype(np.float32)
+    qb, kb = oracle.build_queries(x, 2, 7), oracle.build_keys(k, 2, 6)
+    _, want = oracle.dot_fixed(qb["words"], qb["scales"], kb["words"], kb["scales"], oracle.scale_inv(2, 2), want_ints=False)
+    Bt = torch.empty((3 * 4 * 6 * 64,), dtype=torch.int64, device="cuda")
+    hip.check(L.bsi_hip_tile_key_planes(dev(kb["words"]).data_ptr(), 40, 6, 16, Bt.data_ptr(), st()), "tile")
+    Bw = dev(kb["slice_weights"])
+    out = torch.empty((2, 40), dtype=torch.float32, device="cuda")
+    xd = xh.cuda()
+    code = hip.DTYPE_F16 if dtype == torch.float16 else hip.DTYPE_BF16
+    hip.check(L.bsi_hip_linear_few_rows(xd.data_ptr(), code, 2, 1024, 2, 7, Bt.data_ptr(), Bw.data_ptr(), 6, 40,
+                                        float(oracle.scale_inv(2, 2)), 40, None, out.data_ptr(), st()), "fused")
+    assert np.array_equal(out.cpu().numpy(), want)
+    # limits are refused on the host
+    assert L.bsi_hip_linear_few_rows(xd.data_ptr(), code, 5, 1024, 2, 7, Bt.data_ptr(), Bw.data_ptr(), 6, 40, 1e-4, 40,
+                                     None, out.data_ptr(), st()) != 0
+    assert b"at most 4 query rows" in L.bsi_hip_last_error()
+    assert L.bsi_hip_linear_few_rows(xd.data_ptr(), code, 2, 960, 2, 7, Bt.data_ptr(), Bw.data_ptr(), 6, 40, 1e-4, 40,
+                                     None, out.data_ptr(), st()) != 0   # 15 words per slice: no chunk scales
+    assert L.bsi_hip_linear_few_rows(xd.data_ptr(), code, 2, 1024, 2, 7, Bt.data_ptr(), Bw.data_ptr(), 5, 40, 1e-4, 40,
+                                     None, out.data_ptr(), st()) != 0
+
+
+def test_layer_forward_uses_the_fused_few_rows_kernel(ops, monkeypatch):
+    """A decode-sized call through BSIQuantizedLinear (alone and as fused q/k/v siblings) gives the bits of the
+    build + dot path, for fp32 and fp16 activations."""
+    from bsipytorch_amd import linear
+
+    class Attn(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.q_proj, self.k_proj = torch.nn.Linear(1024, 256), torch.nn.Linear(1024, 256)
+            self.v_proj, self.out_proj = torch.nn.Linear(1024, 256), torch.nn.Linear(256, 1024)
+
+        def forward(self, x):
+            return self.out_proj(self.q_proj(x) + self.k_proj(x) * self.v_proj(x))
+
+    torch.manual_seed(8)
+    model = Attn().cuda()
+    linear.quantize_model_bsi(model, decimalPlaces=2, compress_threshold=0.5, verbose=False, fuse_qkv=True)
+    for dtype in (torch.float32, torch.float16):
+        x = torch.randn(1, 3, 1024, device="cuda").to(dtype)
+        monkeypatch.setenv("BSI_FUSED_LINEAR", "0")
+        with torch.no_grad():
+            want = model(x)
+        calls = linear._sum(model, "build_calls")
+        monkeypatch.setenv("BSI_FUSED_LINEAR", "1")
+        with torch.no_grad():
+            got = model(x)
+        assert torch.equal(got, want) and got.dtype == dtype and got.shape == (1, 3, 1024)
+        assert linear._sum(model, "build_calls") == calls  # no separate query build ran
