@@ -202,10 +202,14 @@ class BSIQuantizedLinear(nn.Module):
             last = group.__dict__.get("_last_few")
             if last is not None and last[0] == key:
                 scores, bias_done = last[2][:, start:stop], last[3]
+                last[4] -= 1
+                if last[4] <= 0:
+                    group.__dict__["_last_few"] = None
             else:
                 gb = group.bias if (fp32 and group.bias is not None) else None
                 all_scores = bsi_ops.linear_few_rows_cuda(batch_inputs, keys, self.decimalPlaces, gb)
-                group.__dict__["_last_few"] = (key, batch_inputs, all_scores, gb is not None)  # holds the input's storage
+                # holds the input's storage (so that its address is not reused) until every member has been served
+                group.__dict__["_last_few"] = [key, batch_inputs, all_scores, gb is not None, len(group.members) - 1]
                 scores, bias_done = all_scores[:, start:stop], gb is not None
                 c["dot_calls"] += 1
         else:
@@ -266,11 +270,15 @@ class _FusedSiblings:
         """(scores of all members [Q, sum of out_features], dot times, whether the bias is already added)."""
         last = self._last
         if last is not None and last[0] is qcap:  # siblings share one query build: the same handle means the same input
-            return last[1], 0, 0.0, 0.0, last[2]
+            out, bias_done = last[1], last[2]
+            last[3] -= 1
+            if last[3] <= 0:  # every member has had its columns: nothing is held until the next forward
+                self._last = None
+            return out, 0, 0.0, 0.0, bias_done
         bias_done = bool(want_bias and self.bias is not None)
         out, ns_total, ns_q, ns_s = bsi_ops.batch_dot_product_multiquery_cuda_batch_caps(
             qcap, self.keys, self.bias if bias_done else None, _keys_to_warm(self.next_layer))
-        self._last = (qcap, out, bias_done)
+        self._last = [qcap, out, bias_done, len(self.members) - 1]
         return out, ns_total, ns_q, ns_s, bias_done
 
 
