@@ -54,6 +54,7 @@ PROTOTYPES = {
     "bsi_hip_dot_bias": [_vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _i, _i64, _i64, _f, _i64, _vp, _vp, _i, _vp, _sz, _vp],
     "bsi_hip_dot_bias_warm": [_vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _i, _i64, _i64, _f, _i64, _vp, _vp, _i, _vp, _sz, _vp, _sz, _vp],
     "bsi_hip_linear_few_rows": [_vp, _i, _i64, _i64, _i, _i, _vp, _vp, _i, _i64, _f, _i64, _vp, _vp, _vp],
+    "bsi_hip_linear_few_rows_upfront": [_i64, _i64, _i64],
     "bsi_hip_dot_ewah_query": [_vp, _vp, _vp, _i, _i, _vp, _i, _vp, _vp, _i, _i64, _f, _vp, _vp, _vp],
     "bsi_hip_planes_to_int8_digits": [_vp, _i64, _i, _i, _vp, _vp],
     "bsi_hip_dot_digits_workspace_bytes": [_i64, _i, _i64, _i],

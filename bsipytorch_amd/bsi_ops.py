@@ -237,12 +237,28 @@ CUDA_BUILDER_VERSION = cuda_builder_version()
 _slice_weight_cache: dict = {}
 
 
+def _capturing() -> bool:
+    return torch.cuda.is_available() and torch.cuda.is_current_stream_capturing()
+
+
 def _slice_weights(S: int, offset: int, twos: bool, device) -> torch.Tensor:
     # bsi_cuda.cpp:217-236; cached per device like make_slice_weights_cuda_cached (bsi_vector_cuda.cpp:48-88).
     # Callers must not modify the returned tensor.
     key = (int(S), int(offset), bool(twos), str(device))
     t = _slice_weight_cache.get(key)
     if t is None:
+        if _capturing():
+            # A host-to-device copy is not allowed while the stream records a graph, and a tensor made here only gets
+            # its values when the graph runs: computed on the device (powers of two as integer shifts, exact) and
+            # kept out of the cache, which eager callers read.
+            e = torch.arange(int(S), device=device, dtype=torch.int64) + int(offset)
+            t = torch.ones(int(S), device=device, dtype=torch.float32)
+            for lo in (0, 62, 124):
+                t = t * torch.bitwise_left_shift(torch.ones_like(e), (e - lo).clamp(0, 62)).to(torch.float32)
+            t = torch.where(e < 0, torch.zeros_like(t), t)
+            if twos and S > 0:
+                t[S - 1] = -t[S - 1]
+            return t
         w = [float(2.0 ** (offset + i)) if offset + i >= 0 else 0.0 for i in range(S)]
         if twos and S > 0:
             w[S - 1] = -w[S - 1]
@@ -344,8 +360,21 @@ def _expanded_slice_weights(base: torch.Tensor, Q: int, bits: int, dev) -> torch
         if len(_expanded_cache) > 64:
             _expanded_cache.clear()
         t = base.unsqueeze(0).expand(Q, -1).contiguous()
+        if _capturing():
+            return t  # filled when the graph runs: not for the cache
         _expanded_cache[key] = t
     return t
+
+
+def warm_query_build_caches(Q: int) -> None:
+    """Creates the constant tensors a fixed-bit query build of Q rows reads (slice weights and their per-row copies),
+    so that a build recorded into a HIP graph later finds them.  A forward that skips the builder when run eagerly
+    (the fused few-rows kernel) calls this for the graph capture that does not skip it."""
+    f = _flags()
+    if f["bits_q"] == 0 or _capturing():
+        return
+    dev = _device()
+    _expanded_slice_weights(_slice_weights(f["bits_q"], 0, True, dev), int(Q), f["bits_q"], dev)
 
 
 def _build_query_batch(q2d: torch.Tensor, decimal_places: int) -> PrebuiltBSIQueryBatchCUDA:
@@ -865,6 +894,7 @@ def _dot_weighted(words, slice_weights, Sa, W, keys: PrebuiltBSIKeysCUDA, Q, dec
 
 
 FUSED_LINEAR_MAX_ROWS = 4
+FUSED_LINEAR_QUERY_LDS_BYTES = 96 * 1024  # the kernel keeps the rows' int8 image and chunk scales in LDS
 
 
 def can_fuse_linear_few_rows(x2d: torch.Tensor, keys: "PrebuiltBSIKeysCUDA") -> bool:
@@ -876,8 +906,14 @@ def can_fuse_linear_few_rows(x2d: torch.Tensor, keys: "PrebuiltBSIKeysCUDA") -> 
             and x2d.dtype in (torch.float32, torch.float16, torch.bfloat16)
             and keys.fixed and keys.Sb == 6 and keys.layout == _lib.LAYOUT_TILED16 and keys.d == d
             and 2 <= f["bits_q"] <= 8 and f["chunk_scale"] and f["clip_k"] == 0.0 and ((d + 63) // 64) % 4 == 0
-            and d <= 8192 * 256 and f["core"] != _lib.CORE_VALU and not f["profile"]
+            and ((d + 255) // 256) * int(x2d.shape[0]) * 260 <= FUSED_LINEAR_QUERY_LDS_BYTES and f["core"] != _lib.CORE_VALU and not f["profile"]
             and os.environ.get("BSI_TC_DOT", "1").strip() != "0" and os.environ.get("BSI_FUSED_LINEAR", "1").strip() != "0")
+
+
+def linear_few_rows_is_free(x2d: torch.Tensor, keys: "PrebuiltBSIKeysCUDA") -> bool:
+    """Whether the fused kernel's query build hides entirely behind its key traffic for this shape
+    (bsi_hip_linear_few_rows_upfront): then the one launch costs the GPU what the dot alone costs."""
+    return bool(lib.bsi_hip_linear_few_rows_upfront(int(x2d.shape[0]), int(x2d.shape[1]), int(keys.num_keys)))
 
 
 def linear_few_rows_cuda(x2d: torch.Tensor, keyset_cuda_cap, decimal_places: int, bias=None) -> torch.Tensor:

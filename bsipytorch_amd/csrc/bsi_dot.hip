@@ -1303,22 +1303,146 @@ __global__ __launch_bounds__(1024) void dot_mfma_stream_kernel(
     }
 }
 
-// The few-rows kernel with the query build inside (at most kFusedMaxQ rows: a decode step).  The wave that takes
-// chunk c quantises that chunk of every query row itself -- round half away of x * 10^dec, the chunk's shift
-// from its largest magnitude, rounded shift and clamp, exactly the builder's per-chunk routine -- into its own
-// LDS image, takes the MFMA operand from there and leaves the chunk scale in LDS for the chain.  Every workgroup
-// repeats that small amount of arithmetic (the kernel waits on the key planes, the VALU is idle), and a BSI-linear
-// layer becomes ONE launch instead of a build and a dot.  Same integers, scales and fp32 chain as
-// bsi_hip_build_fixed + bsi_hip_dot, so the same bits.
+// The few-rows kernel with the query build inside (at most kFusedMaxQ rows: a decode step).  Every workgroup first
+// issues the loads of its first key planes, then quantises the activations itself while those are in flight: the
+// (chunk, row) items go round-robin over the waves, each one the builder's per-chunk routine -- round half away of
+// x * 10^dec, the chunk's shift from its largest magnitude, rounded shift and clamp -- and leave the int8 MFMA
+// operand and the chunk scale in LDS.  After a barrier the kernel is the few-rows kernel above with its query
+// operand in LDS.  Every workgroup repeats that small amount of arithmetic (a few hundred VALU cycles per wave
+// against microseconds of key traffic), and a BSI-linear layer becomes ONE launch instead of a build and a dot.
+// Same integers, scales and fp32 chain as bsi_hip_build_fixed + bsi_hip_dot, so the same bits.
 constexpr int kFusedMaxQ = 4;
+constexpr size_t kFusedQueryLdsBytes = 96 * 1024;  // int8 image + chunk scales of all rows: chunks * Q * 260 bytes
 
-template <typename T, int KT>
+// Element i of a buffer of T as float; 0 past the descriptor's range.
+template <typename T>
+__device__ __forceinline__ float buffer_load_as_float(bsi_rsrc r, int i);
+template <>
+__device__ __forceinline__ float buffer_load_as_float<float>(bsi_rsrc r, int i) {
+    return __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, i * 4, 0, 0));
+}
+template <>
+__device__ __forceinline__ float buffer_load_as_float<__half>(bsi_rsrc r, int i) {
+    const unsigned short h = static_cast<unsigned short>(__builtin_amdgcn_raw_buffer_load_b16(r, i * 2, 0, 0));
+    return __half2float(__ushort_as_half(h));
+}
+template <>
+__device__ __forceinline__ float buffer_load_as_float<__hip_bfloat16>(bsi_rsrc r, int i) {
+    const unsigned short h = static_cast<unsigned short>(__builtin_amdgcn_raw_buffer_load_b16(r, i * 2, 0, 0));
+    return __uint_as_float(static_cast<uint32_t>(h) << 16);
+}
+
+// |round half away from zero of x * scale| for an integer scale of at most 127 and |x| < 2^23, in a dozen 32-bit
+// integer instructions.  With |x| = m * 2^(ex - 150) (24-bit m, hidden bit included) the product M = m * scale is
+// exact in 31 bits, and the float64 route (exact product, + 0.5, floor) equals (M + half) >> s with s = 150 - ex;
+// s >= 32 gives 0 (denormals land there too, so their missing hidden bit does not matter).  Checked against the
+// float64 route on every float.  |x| >= 2^23, infinities and NaNs set `big` and are left to the 64-bit routine.
+__device__ __forceinline__ unsigned scaled_magnitude_u32(float x, unsigned scale, bool& big) {
+    const unsigned bits = __float_as_uint(x) & 0x7fffffffu;
+    const unsigned ex = bits >> 23;
+    const unsigned M = __umul24((bits & 0x7fffffu) | 0x800000u, scale);
+    big = big || ex >= 150u;
+    const unsigned s = 150u - ex;
+    const unsigned r = (M + (1u << ((s - 1u) & 31u))) >> (s & 31u);
+    return (s >= 32u) ? 0u : r;
+}
+
+// Largest v of the wave in every lane's return value (all 64 lanes active): four DPP steps inside each row of 16
+// lanes, then the four rows through scalar registers.
+__device__ __forceinline__ unsigned wave_max_u32(unsigned v) {
+#define BSI_DPP_MAX(ctrl)                                                                                      \
+    {                                                                                                          \
+        const unsigned o = static_cast<unsigned>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), ctrl, 0xF, 0xF, false)); \
+        v = o > v ? o : v;                                                                                     \
+    }
+    BSI_DPP_MAX(0xB1)   // quad_perm [1,0,3,2]
+    BSI_DPP_MAX(0x4E)   // quad_perm [2,3,0,1]
+    BSI_DPP_MAX(0x141)  // row_half_mirror
+    BSI_DPP_MAX(0x140)  // row_mirror
+#undef BSI_DPP_MAX
+    const unsigned a = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(v), 0));
+    const unsigned b = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(v), 16));
+    const unsigned c = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(v), 32));
+    const unsigned d = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(v), 48));
+    const unsigned ab = a > b ? a : b, cd = c > d ? c : d;
+    return ab > cd ? ab : cd;
+}
+
+// One (chunk, row) item: the wave's 256 activations xv[k] = element k * 64 + lane (0 past the row's end) become 256
+// image bytes at img and one scale.  scale_int is 10^dec when that is at most 127 (else 0: float64 arithmetic).
+// Magnitudes below 2^31 (all but pathological inputs) go through 32-bit integer arithmetic; an item with a larger
+// one is left untouched and reported (true, for the whole wave) for fused_quantize_item_wide -- the same two routes,
+// with the same results, as the builder's fast kernel.
+__device__ __forceinline__ bool fused_quantize_item(const float (&xv)[4], double dec_scale, unsigned scale_int, int slices,
+                                                    int valid, int lane, unsigned char* img, float* scale_out) {
+    unsigned mag[4];
+    bool big = false;
+    if (scale_int != 0u) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) mag[k] = scaled_magnitude_u32(xv[k], scale_int, big);
+    } else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const double xs = __dmul_rn(static_cast<double>(xv[k]), dec_scale);
+            const bool b = !(fabs(xs) < 2147483000.0);
+            big = big || b;
+            mag[k] = b ? 0u : static_cast<unsigned>(static_cast<int>(floor(__dadd_rn(fabs(xs), 0.5))));
+        }
+    }
+    if (__any(big)) return true;
+    unsigned mx = 0u;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) mx = mag[k] > mx ? mag[k] : mx;
+    mx = wave_max_u32(mx);
+    // compute_shift without clipping: the bits of the largest magnitude beyond the slices' magnitude bits
+    int shift = (32 - __clz(static_cast<int>(mx))) - (slices - 1);  // mx < 2^31; __clz(0) = 32
+    shift = (shift < 0 || valid <= 0) ? 0 : shift;
+    if (lane == 0) *scale_out = static_cast<float>(1ULL << shift);
+    const unsigned round_add = (shift > 0) ? (1u << (shift - 1)) : 0u;
+    const int qmax32 = (1 << (slices - 1)) - 1, qmin32 = -(1 << (slices - 1));
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int qa = static_cast<int>((mag[k] + round_add) >> shift);
+        int v = (xv[k] < 0.0f) ? -qa : qa;
+        v = v < qmin32 ? qmin32 : (v > qmax32 ? qmax32 : v);
+        img[mfma_byte_pos(k * BSI_WAVE + lane)] = static_cast<unsigned char>(v << (8 - slices));
+    }
+    return false;
+}
+
+// The rare item (a magnitude of 2^31 or more, an infinity, a NaN): the builder's 64-bit routine, reading the chunk
+// from memory (xsrc = its first element) in rolled loops, so that it costs the kernel no registers.
+template <typename T>
+__device__ __forceinline__ void fused_quantize_item_wide(const T* xsrc, double dec_scale, int slices, int valid, int lane,
+                                                         unsigned char* img, float* scale_out) {
+    const long long qmax = (1LL << (slices - 1)) - 1LL, qmin = -(1LL << (slices - 1));
+    unsigned long long mx = 0ULL;
+#pragma unroll 1
+    for (int k = 0; k < 4; ++k) {
+        const int e = k * BSI_WAVE + lane;
+        if (e < valid) {
+            const unsigned long long av = uabs_ll(round_scaled(load_as_float<T>(xsrc, e), dec_scale));
+            if (av > mx) mx = av;
+        }
+    }
+    mx = wave_max_u64(mx);
+    const int shift = (valid > 0) ? compute_shift(mx, 0.0, valid, slices, 0.0f) : 0;
+    if (lane == 0) *scale_out = static_cast<float>(1ULL << shift);
+#pragma unroll 1
+    for (int k = 0; k < 4; ++k) {
+        const int e = k * BSI_WAVE + lane;
+        const long long v = (e < valid) ? shift_clamp(round_scaled(load_as_float<T>(xsrc, e), dec_scale), shift, qmin, qmax) : 0;
+        img[mfma_byte_pos(e)] = static_cast<unsigned char>(static_cast<int>(v) << (8 - slices));
+    }
+}
+
+template <typename T, int KT, int NI>
 __global__ __launch_bounds__(1024) void dot_mfma_stream_fused_kernel(
-    const T* __restrict__ x, int64_t d, double dec_scale, int slices,
+    const T* __restrict__ x, int64_t d, double dec_scale, unsigned scale_int, int slices,
     const unsigned long long* __restrict__ B64,  // tiled key planes, Sb = 6
     const float* __restrict__ Bw, int chunks, int pass_chunks, int64_t R, int Q, float scale_inv, int64_t R_total,
     float* __restrict__ out, const float* __restrict__ bias) {
-    // [pass_chunks][KT][16 queries][16 keys] ints | [waves][kFusedMaxQ][256] image bytes | [chunks][kFusedMaxQ] scales
+    // [pass_chunks][KT][16 queries][16 keys] ints | [chunks][Q][256] image bytes | [chunks][Q] scales
     extern __shared__ __attribute__((aligned(16))) int ints[];
     constexpr int kSlot = KT * 256;
     const int tid = threadIdx.x;
@@ -1326,10 +1450,8 @@ __global__ __launch_bounds__(1024) void dot_mfma_stream_fused_kernel(
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nwaves = static_cast<int>(blockDim.x >> 6);
     const int ln = lane & 15, lg = lane >> 4;
-    unsigned char* const qimg = reinterpret_cast<unsigned char*>(ints + static_cast<size_t>(pass_chunks) * kSlot) +
-                                static_cast<size_t>(wave) * (kFusedMaxQ * 256);
-    float* const qsc = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(ints + static_cast<size_t>(pass_chunks) * kSlot) +
-                                                static_cast<size_t>(nwaves) * (kFusedMaxQ * 256));
+    unsigned char* const qimg = reinterpret_cast<unsigned char*>(ints + static_cast<size_t>(pass_chunks) * kSlot);
+    float* const qsc = reinterpret_cast<float*>(qimg + static_cast<size_t>(chunks) * Q * 256);
     const int64_t ntiles = (R + 15) / 16;
     const int64_t tile0 = static_cast<int64_t>(blockIdx.x) * KT;
     const size_t ktile = static_cast<size_t>(chunks) * (6 * 64);  // words per key tile
@@ -1340,7 +1462,6 @@ __global__ __launch_bounds__(1024) void dot_mfma_stream_fused_kernel(
         ksrc[k] = B64 + static_cast<size_t>(t) * ktile + lane;
     }
     const int down_shift = 16 - slices - 6;
-    const long long qmax = (1LL << (slices - 1)) - 1LL, qmin = -(1LL << (slices - 1));
 
     // the chain lanes: tid <-> (key tile, query, key), keys fastest so output stores are contiguous
     float accf = 0.0f;
@@ -1349,35 +1470,107 @@ __global__ __launch_bounds__(1024) void dot_mfma_stream_fused_kernel(
     const bool cvalid = tid < kSlot && cn < Q && cr < R;
     const float down = __uint_as_float(static_cast<uint32_t>(127 - down_shift) << 23);
 
+    // The wave's share of the query build: (chunk, row) items wave, wave + nwaves, ...  The loads of a CU return in
+    // order, so the activations are requested BEFORE the first key planes (they would otherwise wait behind that
+    // traffic, one round trip per item) and all at once: up to kFusedItems items per wave sit in registers while
+    // the key loads are issued, then they are quantised under the latency of those.
+    constexpr int kFusedItems = NI;  // 1, 2 or (one key tile only) 4: what the registers hold beside the key planes
+    const int items = chunks * Q;
+    // Buffer loads, one descriptor per row: past the row's end they return 0 without a branch (with loads in
+    // conditional blocks the compiler waits for every outstanding load, the key planes included, before a use).
+    auto load_item = [&](int item, float (&dst)[4]) {
+        const int ic = item / Q, iq = item - ic * Q;
+        const bsi_rsrc row = make_rsrc(x + static_cast<int64_t>(iq) * d, static_cast<size_t>(d) * sizeof(T));
+        const int e0 = ic * BSI_CHUNK_ELEMS + lane;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) dst[k] = buffer_load_as_float<T>(row, e0 + k * BSI_WAVE);
+    };
+    auto quantize = [&](int item, const float (&xv)[4]) -> bool {
+        const int ic = item / Q;
+        const int64_t left = d - static_cast<int64_t>(ic) * BSI_CHUNK_ELEMS;
+        const int valid = static_cast<int>(left < BSI_CHUNK_ELEMS ? left : BSI_CHUNK_ELEMS);
+        return fused_quantize_item(xv, dec_scale, scale_int, slices, valid, lane, qimg + static_cast<size_t>(item) * 256,
+                                   qsc + item);
+    };
+    auto quantize_wide = [&](int item) {
+        const int ic = item / Q, iq = item - ic * Q;
+        const int64_t s0 = static_cast<int64_t>(ic) * BSI_CHUNK_ELEMS, left = d - s0;
+        const int valid = static_cast<int>(left < BSI_CHUNK_ELEMS ? left : BSI_CHUNK_ELEMS);
+        fused_quantize_item_wide<T>(x + static_cast<int64_t>(iq) * d + s0, dec_scale, slices, valid, lane,
+                                    qimg + static_cast<size_t>(item) * 256, qsc + item);
+    };
+    float xr[kFusedItems][4];
+#pragma unroll
+    for (int i = 0; i < kFusedItems; ++i) {
+        const int item = wave + i * nwaves;
+        load_item(item < items ? item : items - 1, xr[i]);
+    }
+
+    uint2 kc[KT][6];
+    auto load_keys = [&](int chunk, uint2 (&dst)[KT][6]) {
+#pragma unroll
+        for (int k = 0; k < KT; ++k)
+#pragma unroll
+            for (int j = 0; j < 6; ++j) {
+                const unsigned long long w = ksrc[k][(static_cast<size_t>(chunk) * 6 + j) * 64];
+                dst[k][j] = make_uint2(static_cast<uint32_t>(w), static_cast<uint32_t>(w >> 32));
+            }
+    };
+    // the first pass's first chunk; a wave without one loads the last chunk's planes for nothing, because a branch
+    // here would make the compiler's load counting assume the worst and wait for these loads in the query build
+    load_keys(wave < pass_chunks ? wave : pass_chunks - 1, kc);
+    __builtin_amdgcn_sched_barrier(0);
+    {
+        unsigned wide = 0u;  // items left to the 64-bit routine
+#pragma unroll
+        for (int i = 0; i < kFusedItems; ++i) {
+            // no branch here either (the compiler would sink the item's loads into it, behind the key loads): a wave
+            // with fewer items repeats the last one, and writes the bytes its owner writes
+            const int item = wave + i * nwaves;
+            const bool w = quantize(item < items ? item : items - 1, xr[i]);
+            wide |= (w && item < items) ? 1u << i : 0u;
+            __builtin_amdgcn_sched_barrier(0);  // one item at a time: interleaving them costs registers, gains nothing
+        }
+        // longer rows: the rest one item at a time (each waits for its own loads)
+#pragma unroll 1
+        for (int item = wave + kFusedItems * nwaves; item < items; item += nwaves) {
+            float xa[4];
+            load_item(item, xa);
+            if (quantize(item, xa)) wide |= 1u << 31;
+        }
+#pragma unroll 1
+        for (int i = 0; wide != 0u && i < kFusedItems; ++i)
+            if (wide & (1u << i)) quantize_wide(wave + i * nwaves);
+        if (wide >> 31) {  // some item past the first ones: find it again (rare twice over)
+#pragma unroll 1
+            for (int item = wave + kFusedItems * nwaves; item < items; item += nwaves) {
+                float xa[4];
+                load_item(item, xa);
+                bool big = false;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) big = big || !(fabs(__dmul_rn(static_cast<double>(xa[k]), dec_scale)) < 2147483000.0);
+                if (__any(big)) quantize_wide(item);
+            }
+        }
+        __syncthreads();
+    }
+
     for (int p0 = 0; p0 < chunks; p0 += pass_chunks) {
         const int pend = (p0 + pass_chunks < chunks) ? p0 + pass_chunks : chunks;
         int c = p0 + wave;
-        uint2 kc[KT][6];
-        float xc[kFusedMaxQ][4];  // the wave's chunk of the activations, element k * 64 + lane (0 past the end)
-        auto load_x = [&](int chunk, float (&dst)[kFusedMaxQ][4]) {
-            const int64_t s0 = static_cast<int64_t>(chunk) * BSI_CHUNK_ELEMS;
-#pragma unroll
-            for (int q = 0; q < kFusedMaxQ; ++q)
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    const int64_t e = s0 + k * BSI_WAVE + lane;
-                    dst[q][k] = (q < Q && e < d) ? load_as_float<T>(x, static_cast<int64_t>(q) * d + e) : 0.0f;
-                }
-        };
-        if (c < pend) {
-#pragma unroll
-            for (int k = 0; k < KT; ++k)
-#pragma unroll
-                for (int j = 0; j < 6; ++j) {
-                    const unsigned long long w = ksrc[k][(static_cast<size_t>(c) * 6 + j) * 64];
-                    kc[k][j] = make_uint2(static_cast<uint32_t>(w), static_cast<uint32_t>(w >> 32));
-                }
-            load_x(c, xc);
-        }
+        if (p0 > 0 && c < pend) load_keys(c, kc);
         for (; c < pend; c += nwaves) {
-            // the key planes and the activations of the wave's next chunk first, then this chunk's query build
+            // query operand of this chunk from LDS, then the key planes of the wave's next chunk
+            v4i qb[4];
+            if (ln < Q) {
+                const v4i* src = reinterpret_cast<const v4i*>(qimg + (static_cast<size_t>(c) * Q + ln) * 256 + lg * 64);
+#pragma unroll
+                for (int m = 0; m < 4; ++m) qb[m] = src[m];
+            } else {
+#pragma unroll
+                for (int m = 0; m < 4; ++m) qb[m] = (v4i){0, 0, 0, 0};
+            }
             uint2 kn[KT][6];
-            float xn[kFusedMaxQ][4];
             const int cnext = c + nwaves;
             if (cnext < pend) {
 #pragma unroll
@@ -1387,48 +1580,7 @@ __global__ __launch_bounds__(1024) void dot_mfma_stream_fused_kernel(
                         const unsigned long long w = ksrc[k][(static_cast<size_t>(cnext) * 6 + j) * 64];
                         kn[k][j] = make_uint2(static_cast<uint32_t>(w), static_cast<uint32_t>(w >> 32));
                     }
-                load_x(cnext, xn);
             }
-            const int64_t start = static_cast<int64_t>(c) * BSI_CHUNK_ELEMS;
-            const int valid = static_cast<int>((d - start) < BSI_CHUNK_ELEMS ? (d - start) : BSI_CHUNK_ELEMS);
-#pragma unroll
-            for (int q = 0; q < kFusedMaxQ; ++q) {
-                if (q >= Q) break;  // uniform
-                long long r[4];
-                unsigned long long mx = 0ULL;
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    const int e = k * BSI_WAVE + lane;
-                    r[k] = 0;
-                    if (e < valid) {
-                        r[k] = round_scaled(xc[q][k], dec_scale);
-                        const unsigned long long av = uabs_ll(r[k]);
-                        if (av > mx) mx = av;
-                    }
-                }
-                mx = wave_max_u64(mx);
-                const int shift = (valid > 0) ? compute_shift(mx, 0.0, valid, slices, 0.0f) : 0;
-                if (lane == 0) qsc[c * kFusedMaxQ + q] = static_cast<float>(1ULL << shift);
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    const int e = k * BSI_WAVE + lane;
-                    const long long v = (e < valid) ? shift_clamp(r[k], shift, qmin, qmax) : 0;
-                    qimg[q * 256 + mfma_byte_pos(e)] = static_cast<unsigned char>(static_cast<int>(v) << (8 - slices));
-                }
-            }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            v4i qb[4];
-            if (ln < Q) {
-                const v4i* src = reinterpret_cast<const v4i*>(qimg + ln * 256 + lg * 64);
-#pragma unroll
-                for (int m = 0; m < 4; ++m) qb[m] = src[m];
-            } else {
-#pragma unroll
-                for (int m = 0; m < 4; ++m) qb[m] = (v4i){0, 0, 0, 0};
-            }
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-            __builtin_amdgcn_wave_barrier();  // the image is rewritten for the wave's next chunk
 #pragma unroll
             for (int k = 0; k < KT; ++k) {
                 uint32_t lo[8], hi[8];
@@ -1450,17 +1602,13 @@ __global__ __launch_bounds__(1024) void dot_mfma_stream_fused_kernel(
                 for (int k = 0; k < KT; ++k)
 #pragma unroll
                     for (int j = 0; j < 6; ++j) kc[k][j] = kn[k][j];
-#pragma unroll
-                for (int q = 0; q < kFusedMaxQ; ++q)
-#pragma unroll
-                    for (int k = 0; k < 4; ++k) xc[q][k] = xn[q][k];
             }
         }
         __syncthreads();
         if (cvalid) {
             for (int cc = p0; cc < pend; ++cc) {
                 const int v = ints[(cc - p0) * kSlot + tid];
-                accf = fmaf(static_cast<float>(v), qsc[cc * kFusedMaxQ + cn] * down, accf);
+                accf = fmaf(static_cast<float>(v), qsc[cc * Q + cn] * down, accf);
             }
         }
         if (pend < chunks) __syncthreads();
@@ -2244,29 +2392,74 @@ extern "C" int bsi_hip_dot_bias_warm(const uint64_t* A, const int8_t* A_ints8, c
     return rc;
 }
 
-template <typename T, int KT>
-static void launch_stream_fused(const T* x, int64_t d, double dec_scale, int slices, const uint64_t* B, const float* Bw,
-                                int chunks, int64_t R, int Q, float scale_inv, int64_t R_total, float* out,
+// Launch shape of the fused few-rows kernel: key tiles per workgroup, waves, and how many (chunk, row) items of the
+// query build a wave takes up front (loads issued before the key loads; the rest go one at a time, each waiting for
+// its own loads).
+struct FusedPlan {
+    int key_tiles, waves, upfront, per_wave;
+    unsigned grid;
+};
+static FusedPlan fused_plan(int64_t Q, int chunks, int64_t R) {
+    FusedPlan p;
+    const int64_t ntiles = (R + 15) / 16;
+    p.key_tiles = ntiles >= 1024 ? 2 : 1;  // as bsi_hip_dot: two key tiles per workgroup once the GPU is full
+    p.grid = static_cast<unsigned>((ntiles + p.key_tiles - 1) / p.key_tiles);
+    p.waves = (p.grid <= 256) ? 16 : 8;  // as the few-rows kernel: one workgroup per CU gets more waves
+    if (p.waves > chunks) p.waves = chunks;
+    if (p.waves < p.key_tiles * 4) p.waves = p.key_tiles * 4;
+    p.per_wave = static_cast<int>((static_cast<int64_t>(chunks) * Q + p.waves - 1) / p.waves);
+    const int cap = p.key_tiles == 1 ? 4 : 2;
+    p.upfront = p.per_wave <= 1 ? 1 : (p.per_wave <= 2 ? 2 : cap);
+    return p;
+}
+
+template <typename T, int KT, int NI>
+static void launch_stream_fused(const FusedPlan& plan, const T* x, int64_t d, double dec_scale, int slices, const uint64_t* B,
+                                const float* Bw, int chunks, int64_t R, int Q, float scale_inv, int64_t R_total, float* out,
                                 const float* bias, hipStream_t st) {
     constexpr int kSlot = KT * 256;
-    const int64_t ntiles = (R + 15) / 16;
-    const dim3 grid(static_cast<unsigned>((ntiles + KT - 1) / KT));
-    int waves = (grid.x <= 256) ? 16 : 8;  // as the few-rows kernel: one workgroup per CU gets more waves
-    if (waves > chunks) waves = chunks;
-    if (waves < kSlot / 64) waves = kSlot / 64;
+    // LDS: the query image and scales of all chunks, then as many chunk accumulators as fit beside them
+    const size_t query_bytes = static_cast<size_t>(chunks) * Q * (256 + sizeof(float));
     int pass_chunks = kStreamLdsInts / kSlot;
+    const int fit = static_cast<int>((150 * 1024 - query_bytes) / (kSlot * sizeof(int)));
+    if (pass_chunks > fit) pass_chunks = fit;
     if (pass_chunks > chunks) pass_chunks = chunks;
-    const size_t lds = static_cast<size_t>(pass_chunks) * kSlot * sizeof(int) +
-                       static_cast<size_t>(waves) * kFusedMaxQ * 256 + static_cast<size_t>(chunks) * kFusedMaxQ * sizeof(float);
+    const size_t lds = static_cast<size_t>(pass_chunks) * kSlot * sizeof(int) + query_bytes;
     static bool configured = false;
     if (!configured) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dot_mfma_stream_fused_kernel<T, KT>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dot_mfma_stream_fused_kernel<T, KT, NI>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         configured = true;
     }
-    hipLaunchKernelGGL((dot_mfma_stream_fused_kernel<T, KT>), grid, dim3(waves * 64), lds, st, x, d, dec_scale, slices,
-                       reinterpret_cast<const unsigned long long*>(B), Bw, chunks, pass_chunks, R, Q, scale_inv, R_total,
-                       out, bias);
+    const unsigned scale_int = (dec_scale >= 1.0 && dec_scale <= 127.0 && dec_scale == floor(dec_scale))
+                                   ? static_cast<unsigned>(dec_scale) : 0u;
+    hipLaunchKernelGGL((dot_mfma_stream_fused_kernel<T, KT, NI>), dim3(plan.grid), dim3(plan.waves * 64), lds, st, x, d,
+                       dec_scale, scale_int, slices, reinterpret_cast<const unsigned long long*>(B), Bw, chunks, pass_chunks,
+                       R, Q, scale_inv, R_total, out, bias);
+}
+
+template <typename T>
+static void launch_stream_fused_t(const T* x, int64_t d, double dec_scale, int slices, const uint64_t* B, const float* Bw,
+                                  int chunks, int64_t R, int Q, float scale_inv, int64_t R_total, float* out,
+                                  const float* bias, hipStream_t st) {
+    const FusedPlan p = fused_plan(Q, chunks, R);
+#define BSI_FUSED_GO(KT, NI) \
+    launch_stream_fused<T, KT, NI>(p, x, d, dec_scale, slices, B, Bw, chunks, R, Q, scale_inv, R_total, out, bias, st)
+    if (p.key_tiles == 2) {
+        if (p.upfront == 1) BSI_FUSED_GO(2, 1);
+        else BSI_FUSED_GO(2, 2);
+    } else {
+        if (p.upfront == 1) BSI_FUSED_GO(1, 1);
+        else if (p.upfront == 2) BSI_FUSED_GO(1, 2);
+        else BSI_FUSED_GO(1, 4);
+    }
+#undef BSI_FUSED_GO
+}
+
+extern "C" int bsi_hip_linear_few_rows_upfront(int64_t Q, int64_t d, int64_t R) {
+    if (Q < 1 || Q > kFusedMaxQ || d < 1 || R < 1) return 0;
+    const FusedPlan p = fused_plan(Q, static_cast<int>((d + 255) / 256), R);
+    return p.per_wave <= p.upfront ? 1 : 0;
 }
 
 extern "C" int bsi_hip_linear_few_rows(const void* x, int dtype, int64_t Q, int64_t d, int decimal_places, int fixed_bits,
@@ -2284,16 +2477,14 @@ extern "C" int bsi_hip_linear_few_rows(const void* x, int dtype, int64_t Q, int6
     if (Q == 0 || R == 0) return BSI_OK;
     BSI_REQUIRE(x && B_tiled && Bw && out, "null pointer");
     const int chunks = W64 / 4;
-    if (static_cast<size_t>(chunks) * kFusedMaxQ * sizeof(float) > 32 * 1024)
-        return fail(BSI_ERR_UNSUPPORTED, "rows of %lld elements do not fit the scale buffer", static_cast<long long>(d));
+    if (static_cast<size_t>(chunks) * Q * (256 + sizeof(float)) > kFusedQueryLdsBytes)
+        return fail(BSI_ERR_UNSUPPORTED, "%lld rows of %lld elements do not fit the kernel's LDS query buffer (%zu bytes)",
+                    static_cast<long long>(Q), static_cast<long long>(d), kFusedQueryLdsBytes);
     const double dec_scale = pow(10.0, static_cast<double>(decimal_places));
     hipStream_t st = as_stream(stream);
-    const bool two = (R + 15) / 16 >= 1024;  // as bsi_hip_dot: two key tiles per workgroup once the GPU is full
-#define BSI_FUSED(T)                                                                                              \
-    if (two) launch_stream_fused<T, 2>(static_cast<const T*>(x), d, dec_scale, fixed_bits, B_tiled, Bw, chunks, R,    \
-                                       static_cast<int>(Q), scale_inv, R_total, out, bias, st);                       \
-    else launch_stream_fused<T, 1>(static_cast<const T*>(x), d, dec_scale, fixed_bits, B_tiled, Bw, chunks, R,        \
-                                   static_cast<int>(Q), scale_inv, R_total, out, bias, st);
+#define BSI_FUSED(T)                                                                                                \
+    launch_stream_fused_t<T>(static_cast<const T*>(x), d, dec_scale, fixed_bits, B_tiled, Bw, chunks, R, static_cast<int>(Q), \
+                             scale_inv, R_total, out, bias, st);
     if (dtype == BSI_DTYPE_F32) { BSI_FUSED(float) }
     else if (dtype == BSI_DTYPE_F16) { BSI_FUSED(__half) }
     else if (dtype == BSI_DTYPE_BF16) { BSI_FUSED(__hip_bfloat16) }

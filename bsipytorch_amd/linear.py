@@ -191,11 +191,15 @@ class BSIQuantizedLinear(nn.Module):
         if c.get("collect_stats") or not bsi_ops.can_fuse_linear_few_rows(batch_inputs, keys):
             return None
         # The fused kernel saves the host a launch and the handles of a query build, which is what an eager decode
-        # step is bound by; on the GPU it costs what it saves (every workgroup repeats the quantisation), so a
-        # forward that is being captured into a graph, where host time does not count, keeps the two launches.
-        if torch.cuda.is_current_stream_capturing():
+        # step is bound by.  On the GPU it costs no more than the dot alone as long as every workgroup can request
+        # its share of the activations before its key planes; past that (more rows, longer rows) it repeats too much
+        # arithmetic, so a forward that is being captured into a graph, where host time does not count, then keeps
+        # the two launches.  BSI_FUSED_LINEAR=2 forces the fused kernel in both cases.
+        if (torch.cuda.is_current_stream_capturing() and os.getenv("BSI_FUSED_LINEAR", "1") != "2"
+                and not bsi_ops.linear_few_rows_is_free(batch_inputs, keys)):
             return None
         fp32 = original_dtype == torch.float32
+        bsi_ops.warm_query_build_caches(int(batch_inputs.shape[0]))
         if fused is not None:
             group, start, stop = fused
             key = (batch_inputs.data_ptr(), tuple(batch_inputs.shape), batch_inputs.dtype, batch_inputs._version)

@@ -225,14 +225,21 @@ int bsi_hip_dot_bias_warm(const uint64_t* A, const int8_t* A_ints8, const float*
 
 /* A whole BSI-linear layer for at most 4 activation rows (a decode step) in ONE launch: the chunk-scale query
  * build of bsi_hip_build_fixed (x [Q, d] of dtype, decimal_places, fixed_bits in [2, 8], no clipping) is done
- * inside the few-rows dot kernel, by the wave that takes each chunk, and the result is that of
- * bsi_hip_build_fixed followed by bsi_hip_dot_bias on the tiled planes, bit for bit.  d must give a multiple of
- * 4 words per slice (chunk scales), Sb must be 6.  Replaces, for such calls, the sequence
+ * inside the few-rows dot kernel -- every workgroup quantises the rows into LDS while its first key planes are
+ * on their way -- and the result is that of bsi_hip_build_fixed followed by bsi_hip_dot_bias on the tiled planes,
+ * bit for bit.  d must give a multiple of 4 words per slice (chunk scales), Sb must be 6, and the rows' int8
+ * image and scales (260 bytes per row and 256 elements) must fit 96 KiB of LDS.  Replaces, for such calls, the sequence
  * build_bsi_queries_cuda_batch_packed + batch_dot_product_multiquery_cuda_batch_caps of a layer forward
  * (verify_accuracy_bsi.py:143-178). */
 int bsi_hip_linear_few_rows(const void* x_device, int dtype, int64_t Q, int64_t d, int decimal_places, int fixed_bits,
                             const uint64_t* B_tiled, const float* Bw, int Sb, int64_t R, float scale_inv, int64_t R_total,
                             const float* bias, float* out, void* stream);
+
+/* 1 when bsi_hip_linear_few_rows, for this shape, issues the loads of the whole query build before its first key
+ * loads (the case in which the launch costs the GPU no more than the dot alone), 0 when some of the build waits
+ * behind the key traffic (then the one launch still saves host time, but build + dot is the faster pair on the
+ * GPU).  A host-side query: no GPU work.  No counterpart in the reference. */
+int bsi_hip_linear_few_rows_upfront(int64_t Q, int64_t d, int64_t R);
 
 /* The same dot for ONE query whose slices are EWAH streams (the hybrid query form of
  * build_bsi_query_cuda_hybrid, bsi_cuda.cpp:386-431): stream s at comp_words + comp_off[s], comp_len[s]

@@ -203,3 +203,16 @@ def test_load_keyset_refuses_foreign_files_before_touching_the_device(tmp_path):
     (tmp_path / "keyset.bsik").write_bytes(b"BSIKEYS1" + (1 << 40).to_bytes(8, "little"))
     with pytest.raises(RuntimeError, match="bad header length"):
         bsi_ops.load_keyset_cuda(str(tmp_path))
+
+
+def test_linear_few_rows_upfront_is_a_host_side_query():
+    """bsi_hip_linear_few_rows_upfront needs no GPU: decode shapes of an OPT-6.7B layer at one row are served
+    entirely up front, four rows of 16384 elements are not, bad shapes say no."""
+    from bsipytorch_amd import _lib
+
+    f = _lib.lib.bsi_hip_linear_few_rows_upfront
+    assert f(1, 4096, 16384) == 1 and f(1, 16384, 4096) == 1 and f(1, 4096, 4096) == 1 and f(1, 4096, 12288) == 1
+    assert f(4, 16384, 4096) == 0 and f(4, 4096, 16384) == 0
+    assert f(2, 4096, 4096) == 1
+    assert f(0, 4096, 4096) == 0 and f(5, 4096, 4096) == 0 and f(1, 0, 4096) == 0
+

@@ -1499,6 +1499,51 @@ def test_linear_few_rows_matches_build_plus_dot(hip, oracle, Q, R, d, kind):
         assert np.isnan(got[:, R:]).all()
 
 
+@pytest.mark.parametrize("dec", [0, 1, 3])
+def test_linear_few_rows_other_decimal_places(hip, oracle, dec):
+    """10^dec of 1 and 10 take the kernel's integer rounding route (as 100 does), 1000 its float64 route."""
+    L = hip.lib
+    Q, R, d = 3, 50, 1024
+    x = _inputs(Q, d, seed=dec, kind="ties") * np.float32(10.0 ** (2 - dec))
+    k = (np.random.default_rng(dec).standard_normal((R, d)) * (0.02 * 10.0 ** (2 - dec))).astype(np.float32)
+    qb, kb = oracle.build_queries(x, dec, 7), oracle.build_keys(k, dec, 6)
+    _, want = oracle.dot_fixed(qb["words"], qb["scales"], kb["words"], kb["scales"], oracle.scale_inv(dec, dec), want_ints=False)
+    Bt = torch.empty((4 * 4 * 6 * 64,), dtype=torch.int64, device="cuda")
+    hip.check(L.bsi_hip_tile_key_planes(dev(kb["words"]).data_ptr(), R, 6, 16, Bt.data_ptr(), st()), "tile")
+    Bw = dev(kb["slice_weights"])
+    out = torch.empty((Q, R), dtype=torch.float32, device="cuda")
+    hip.check(L.bsi_hip_linear_few_rows(torch.from_numpy(x).cuda().data_ptr(), hip.DTYPE_F32, Q, d, dec, 7, Bt.data_ptr(),
+                                        Bw.data_ptr(), 6, R, float(oracle.scale_inv(dec, dec)), R, None, out.data_ptr(),
+                                        st()), "fused")
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy(), want)
+
+
+def test_linear_few_rows_long_rows_and_lds_limit(hip, oracle):
+    """Rows of 96 chunks: three of them fit the kernel's LDS query buffer and run in two passes over the chunk
+    accumulators; four do not and are refused on the host."""
+    L = hip.lib
+    R, d = 20, 24576
+    x = _inputs(4, d, seed=5, kind="outliers")
+    x[0, 7] = 3.0e7   # x * 100 beyond 32 bits: that chunk takes the kernel's 64-bit route
+    x[2, 20000] = -4.0e7  # and one among a wave's later items
+    k = (np.random.default_rng(2).standard_normal((R, d)) * 0.02).astype(np.float32)
+    qb, kb = oracle.build_queries(x[:3], 2, 7), oracle.build_keys(k, 2, 6)
+    _, want = oracle.dot_fixed(qb["words"], qb["scales"], kb["words"], kb["scales"], oracle.scale_inv(2, 2), want_ints=False)
+    W = d // 64
+    Bt = torch.empty((2 * (W // 4) * 6 * 64,), dtype=torch.int64, device="cuda")
+    hip.check(L.bsi_hip_tile_key_planes(dev(kb["words"]).data_ptr(), R, 6, W, Bt.data_ptr(), st()), "tile")
+    Bw = dev(kb["slice_weights"])
+    xd = torch.from_numpy(x).cuda()
+    out = torch.empty((4, R), dtype=torch.float32, device="cuda")
+    hip.check(L.bsi_hip_linear_few_rows(xd.data_ptr(), hip.DTYPE_F32, 3, d, 2, 7, Bt.data_ptr(), Bw.data_ptr(), 6, R,
+                                        float(oracle.scale_inv(2, 2)), R, None, out.data_ptr(), st()), "fused")
+    assert np.array_equal(out[:3].cpu().numpy(), want)
+    assert L.bsi_hip_linear_few_rows(xd.data_ptr(), hip.DTYPE_F32, 4, d, 2, 7, Bt.data_ptr(), Bw.data_ptr(), 6, R,
+                                     float(oracle.scale_inv(2, 2)), R, None, out.data_ptr(), st()) != 0
+    assert b"LDS query buffer" in L.bsi_hip_last_error()
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_linear_few_rows_half_inputs_and_limits(hip, oracle, dtype):
     L = hip.lib
