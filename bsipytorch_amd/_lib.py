@@ -17,6 +17,7 @@ CORE_AUTO, CORE_VALU, CORE_MFMA = 0, 1, 2
 LAYOUT_CANONICAL, LAYOUT_TILED16, LAYOUT_INT8, LAYOUT_INT8_TILED = 0, 1, 2, 3
 OPT_I8_TILE = 1
 OPT_DIGITS_ROUTE = 2
+OPT_BUILD_ITEMS = 3
 
 _vp = ctypes.c_void_p
 _i = ctypes.c_int

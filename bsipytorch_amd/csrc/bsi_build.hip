@@ -252,9 +252,11 @@ __global__ void build_fixed_chunk_kernel(const T* __restrict__ x, int64_t Q, int
 
 // The same build for the common case (at most 8 slices, no clipping, whole chunks of words), about
 // seven times fewer instructions per element.  One wave takes 8 consecutive (row, chunk) items:
-//   * rounding stays in fp64 (the product (double)(float)v * 10^dec must be exact), but everything
-//     after it is 32-bit integer work; an item holding a magnitude of 2^31 or more (or a NaN) is
-//     handed to the 64-bit routine above, so results never differ;
+//   * round-half-away(v * 10^dec) comes from the float's mantissa in 32-bit integer arithmetic when 10^dec is
+//     an integer of at most 127 (the same integer as the exact float64 product + 0.5 and floor, checked on every
+//     float), else from that float64 sequence; everything after it is 32-bit integer work; an item holding a
+//     magnitude the 32-bit route does not cover (2^31 or more after scaling, a NaN) is handed to the 64-bit
+//     routine above, so results never differ;
 //   * the quantised values go to LDS as the int8 image (value << (8 - slices), the MFMA core's
 //     in-chunk order); the image is the bit-transpose of the planes, 32 elements at a time, so
 //     lane (item j, unit w) reads its 8 dwords, transposes the 8x8 bit blocks in registers and
@@ -264,7 +266,7 @@ __global__ void build_fixed_chunk_kernel(const T* __restrict__ x, int64_t Q, int
 template <typename T, int kFastItems>
 __global__ __launch_bounds__(kBlock) void build_fixed_chunk_fast_kernel(
     const T* __restrict__ x, int64_t Q, int64_t d, int chunks, int slices, int words_per_slice, double dec_scale,
-    unsigned long long* __restrict__ words, int* __restrict__ shifts, float* __restrict__ scales,
+    unsigned scale_int, unsigned long long* __restrict__ words, int* __restrict__ shifts, float* __restrict__ scales,
     int8_t* __restrict__ ints8) {
     __shared__ uint32_t image[kWavesPerBlock][kFastItems][BSI_CHUNK_ELEMS / 4];
     const int lane = threadIdx.x & (BSI_WAVE - 1);
@@ -302,29 +304,29 @@ __global__ __launch_bounds__(kBlock) void build_fixed_chunk_fast_kernel(
             (void)row;
             const int64_t start = static_cast<int64_t>(c) * BSI_CHUNK_ELEMS;
             const int valid = static_cast<int>((d - start) < BSI_CHUNK_ELEMS ? (d - start) : BSI_CHUNK_ELEMS);
-            double xs[4];
+            // magnitudes of round-half-away(x * 10^dec): from the float's mantissa when 10^dec is a small integer
+            // (scaled_magnitude_u32), else in float64; elements past the end were loaded as 0
+            unsigned mag[4];
             bool big = false;
+            if (scale_int != 0u) {
 #pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                xs[k] = __dmul_rn(static_cast<double>(raw[j][k]), dec_scale);  // elements past the end were loaded as 0
-                big = big || !(fabs(xs[k]) < 2147483000.0);
+                for (int k = 0; k < 4; ++k) mag[k] = scaled_magnitude_u32(raw[j][k], scale_int, big);
+            } else {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const double xs = __dmul_rn(static_cast<double>(raw[j][k]), dec_scale);
+                    const bool b = !(fabs(xs) < 2147483000.0);
+                    big = big || b;
+                    mag[k] = b ? 0u : static_cast<unsigned>(static_cast<int>(floor(__dadd_rn(fabs(xs), 0.5))));
+                }
             }
             if (__any(big)) {
                 slow |= 1u << j;  // done below by the 64-bit routine
             } else {
-                int r[4];
                 unsigned mx = 0u;
 #pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    const int mag = static_cast<int>(floor(__dadd_rn(fabs(xs[k]), 0.5)));  // round half away from zero
-                    r[k] = (xs[k] < 0.0) ? -mag : mag;
-                    mx = (static_cast<unsigned>(mag) > mx) ? static_cast<unsigned>(mag) : mx;
-                }
-#pragma unroll
-                for (int off = 32; off > 0; off >>= 1) {
-                    const unsigned o = __shfl_xor(mx, off, BSI_WAVE);
-                    mx = o > mx ? o : mx;
-                }
+                for (int k = 0; k < 4; ++k) mx = mag[k] > mx ? mag[k] : mx;
+                mx = wave_max_u32(mx);
                 const int shift = compute_shift(static_cast<unsigned long long>(mx), 0.0, valid, slices, 0.0f);
                 if (lane == 0) {
                     shifts[item] = shift;
@@ -334,9 +336,8 @@ __global__ __launch_bounds__(kBlock) void build_fixed_chunk_fast_kernel(
                 unsigned char* img = reinterpret_cast<unsigned char*>(image[wib][j]);
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
-                    const unsigned av = static_cast<unsigned>(r[k] < 0 ? -r[k] : r[k]);
-                    const int qa = static_cast<int>((av + round_add) >> shift);
-                    int q = (r[k] < 0) ? -qa : qa;
+                    const int qa = static_cast<int>((mag[k] + round_add) >> shift);
+                    int q = (raw[j][k] < 0.0f) ? -qa : qa;
                     q = q < qmin ? qmin : (q > qmax ? qmax : q);
                     img[mfma_byte_pos(k * BSI_WAVE + lane)] = static_cast<unsigned char>(q << (8 - slices));
                 }
@@ -702,6 +703,8 @@ extern "C" int bsi_hip_decimal_stats(const int64_t* ints, int64_t Q, int64_t d, 
     return BSI_OK;
 }
 
+int bsi::g_build_items = 0;
+
 extern "C" int bsi_hip_build_fixed(const void* x, int dtype, int64_t Q, int64_t d, int decimal_places, int fixed_bits,
                                    int chunk_scale, float clip_k, uint64_t* words, int32_t* shifts, float* scales,
                                    int8_t* ints8, void* stream) {
@@ -721,13 +724,17 @@ extern "C" int bsi_hip_build_fixed(const void* x, int dtype, int64_t Q, int64_t 
         BSI_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((build_fixed_chunk_fast_kernel<T, N>), dim3(grid_for(waves)),   \
                                                      dim3(kBlock), 0, as_stream(stream), static_cast<const T*>(x), Q, \
                                                      d, chunks, fixed_bits, W, dec_scale,                            \
+                                                     integer_decimal_scale(dec_scale),                               \
                                                      reinterpret_cast<unsigned long long*>(words), shifts, scales,   \
                                                      ints8));                                                        \
     }
-        // a wave gets more items only once there are more than about 16 waves per SIMD (16384 in all)
-        if (items > 8 * 16384) BSI_LAUNCH_FAST(8)
-        else if (items > 4 * 16384) BSI_LAUNCH_FAST(4)
-        else if (items > 16384) BSI_LAUNCH_FAST(2)
+        // a wave gets more items only once there are about 8 waves per SIMD (8192 in all); measured on
+        // 4096 ... 131072 items, every other choice is within a few percent or slower
+        int per_wave = g_build_items;
+        if (per_wave == 0) per_wave = items > 8 * 16384 ? 8 : (items >= 16384 ? 4 : (items >= 8192 ? 2 : 1));
+        if (per_wave == 8) BSI_LAUNCH_FAST(8)
+        else if (per_wave == 4) BSI_LAUNCH_FAST(4)
+        else if (per_wave == 2) BSI_LAUNCH_FAST(2)
         else BSI_LAUNCH_FAST(1)
 #undef BSI_LAUNCH_FAST
         BSI_LAUNCH_CHECK("build_fixed_chunk_fast_kernel");

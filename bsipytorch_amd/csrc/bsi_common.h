@@ -108,6 +108,50 @@ __device__ __forceinline__ long long shift_clamp(long long v, int shift, long lo
     return out;
 }
 
+// |round half away from zero of x * scale| for an integer scale of at most 127 and |x| < 2^23, in a dozen 32-bit
+// integer instructions.  With |x| = m * 2^(ex - 150) (24-bit m, hidden bit included) the product M = m * scale is
+// exact in 31 bits, and the float64 route (exact product, + 0.5, floor) equals (M + half) >> s with s = 150 - ex;
+// s >= 32 gives 0 (denormals land there too, so their missing hidden bit does not matter).  Checked against the
+// float64 route on every float.  |x| >= 2^23, infinities and NaNs set `big` and are left to the 64-bit routine.
+__device__ __forceinline__ unsigned scaled_magnitude_u32(float x, unsigned scale, bool& big) {
+    const unsigned bits = __float_as_uint(x) & 0x7fffffffu;
+    const unsigned ex = bits >> 23;
+    const unsigned M = __umul24((bits & 0x7fffffu) | 0x800000u, scale);
+    big = big || ex >= 150u;
+    const unsigned s = 150u - ex;
+    const unsigned r = (M + (1u << ((s - 1u) & 31u))) >> (s & 31u);
+    return (s >= 32u) ? 0u : r;
+}
+
+// Largest v of the wave in every lane's return value (all 64 lanes active): four DPP steps inside each row of 16
+// lanes, then the four rows through scalar registers.
+__device__ __forceinline__ unsigned wave_max_u32(unsigned v) {
+#define BSI_DPP_MAX(ctrl)                                                                                      \
+    {                                                                                                          \
+        const unsigned o = static_cast<unsigned>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), ctrl, 0xF, 0xF, false)); \
+        v = o > v ? o : v;                                                                                     \
+    }
+    BSI_DPP_MAX(0xB1)   // quad_perm [1,0,3,2]
+    BSI_DPP_MAX(0x4E)   // quad_perm [2,3,0,1]
+    BSI_DPP_MAX(0x141)  // row_half_mirror
+    BSI_DPP_MAX(0x140)  // row_mirror
+#undef BSI_DPP_MAX
+    const unsigned a = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(v), 0));
+    const unsigned b = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(v), 16));
+    const unsigned c = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(v), 32));
+    const unsigned d = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(v), 48));
+    const unsigned ab = a > b ? a : b, cd = c > d ? c : d;
+    return ab > cd ? ab : cd;
+}
+
+extern int g_build_items;  // BSI_OPT_BUILD_ITEMS (bsi_build.hip)
+
+// 10^dec as an integer when scaled_magnitude_u32 can take it (at most 127), else 0: float64 arithmetic then.
+static inline unsigned integer_decimal_scale(double dec_scale) {
+    return (dec_scale >= 1.0 && dec_scale <= 127.0 && dec_scale == static_cast<double>(static_cast<unsigned>(dec_scale)))
+               ? static_cast<unsigned>(dec_scale) : 0u;
+}
+
 // Position of element e (0..255) of a chunk inside the chunk's 256 int8 bytes in the MFMA core's
 // order: element 32w + 8m + t sits at byte 32w + 4t + m (see planes_to_int8 in bsi_dot.hip).
 __device__ __forceinline__ int mfma_byte_pos(int e) {

@@ -1332,42 +1332,6 @@ __device__ __forceinline__ float buffer_load_as_float<__hip_bfloat16>(bsi_rsrc r
     return __uint_as_float(static_cast<uint32_t>(h) << 16);
 }
 
-// |round half away from zero of x * scale| for an integer scale of at most 127 and |x| < 2^23, in a dozen 32-bit
-// integer instructions.  With |x| = m * 2^(ex - 150) (24-bit m, hidden bit included) the product M = m * scale is
-// exact in 31 bits, and the float64 route (exact product, + 0.5, floor) equals (M + half) >> s with s = 150 - ex;
-// s >= 32 gives 0 (denormals land there too, so their missing hidden bit does not matter).  Checked against the
-// float64 route on every float.  |x| >= 2^23, infinities and NaNs set `big` and are left to the 64-bit routine.
-__device__ __forceinline__ unsigned scaled_magnitude_u32(float x, unsigned scale, bool& big) {
-    const unsigned bits = __float_as_uint(x) & 0x7fffffffu;
-    const unsigned ex = bits >> 23;
-    const unsigned M = __umul24((bits & 0x7fffffu) | 0x800000u, scale);
-    big = big || ex >= 150u;
-    const unsigned s = 150u - ex;
-    const unsigned r = (M + (1u << ((s - 1u) & 31u))) >> (s & 31u);
-    return (s >= 32u) ? 0u : r;
-}
-
-// Largest v of the wave in every lane's return value (all 64 lanes active): four DPP steps inside each row of 16
-// lanes, then the four rows through scalar registers.
-__device__ __forceinline__ unsigned wave_max_u32(unsigned v) {
-#define BSI_DPP_MAX(ctrl)                                                                                      \
-    {                                                                                                          \
-        const unsigned o = static_cast<unsigned>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), ctrl, 0xF, 0xF, false)); \
-        v = o > v ? o : v;                                                                                     \
-    }
-    BSI_DPP_MAX(0xB1)   // quad_perm [1,0,3,2]
-    BSI_DPP_MAX(0x4E)   // quad_perm [2,3,0,1]
-    BSI_DPP_MAX(0x141)  // row_half_mirror
-    BSI_DPP_MAX(0x140)  // row_mirror
-#undef BSI_DPP_MAX
-    const unsigned a = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(v), 0));
-    const unsigned b = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(v), 16));
-    const unsigned c = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(v), 32));
-    const unsigned d = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(v), 48));
-    const unsigned ab = a > b ? a : b, cd = c > d ? c : d;
-    return ab > cd ? ab : cd;
-}
-
 // One (chunk, row) item: the wave's 256 activations xv[k] = element k * 64 + lane (0 past the row's end) become 256
 // image bytes at img and one scale.  scale_int is 10^dec when that is at most 127 (else 0: float64 arithmetic).
 // Magnitudes below 2^31 (all but pathological inputs) go through 32-bit integer arithmetic; an item with a larger
@@ -2238,6 +2202,10 @@ extern "C" int bsi_hip_set_option(int option, int value) {
                         "tile must be 0, 128, 12864, 64 or 6432");
             g_i8_tile = value;
             return BSI_OK;
+        case BSI_OPT_BUILD_ITEMS:
+            BSI_REQUIRE(value == 0 || value == 1 || value == 2 || value == 4 || value == 8, "items must be 0, 1, 2, 4 or 8");
+            g_build_items = value;
+            return BSI_OK;
         default:
             return fail(BSI_ERR_INVALID, "unknown option %d", option);
     }
@@ -2431,8 +2399,7 @@ static void launch_stream_fused(const FusedPlan& plan, const T* x, int64_t d, do
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         configured = true;
     }
-    const unsigned scale_int = (dec_scale >= 1.0 && dec_scale <= 127.0 && dec_scale == floor(dec_scale))
-                                   ? static_cast<unsigned>(dec_scale) : 0u;
+    const unsigned scale_int = integer_decimal_scale(dec_scale);
     hipLaunchKernelGGL((dot_mfma_stream_fused_kernel<T, KT, NI>), dim3(plan.grid), dim3(plan.waves * 64), lds, st, x, d,
                        dec_scale, scale_int, slices, reinterpret_cast<const unsigned long long*>(B), Bw, chunks, pass_chunks,
                        R, Q, scale_inv, R_total, out, bias);

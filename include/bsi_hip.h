@@ -176,6 +176,8 @@ int bsi_hip_planes_to_int8_tiled(const uint64_t* words_device, int64_t rows, int
                              the 256 CUs */
 #define BSI_OPT_DIGITS_ROUTE 2 /* bsi_hip_dot_digits: 1 = stacked digits and a combine pass, 2 = digits recombined in the
                                   accumulator where the int32 bound allows; 0 (default) = the cheaper by a cost estimate */
+#define BSI_OPT_BUILD_ITEMS 3 /* (row, chunk) items per wave of the fused chunk-scale builder: 1, 2, 4 or 8; 0 (default)
+                                 = chosen per call from the number of items */
 int bsi_hip_set_option(int option, int value);
 
 /* Bytes of device workspace bsi_hip_dot needs for this shape and core (0 when none). */

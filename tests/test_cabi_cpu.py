@@ -190,6 +190,9 @@ def test_set_option_validates_on_host():
     assert _lib.lib.bsi_hip_set_option(_lib.OPT_DIGITS_ROUTE, 2) == 0
     assert _lib.lib.bsi_hip_set_option(_lib.OPT_DIGITS_ROUTE, 3) == 1
     assert _lib.lib.bsi_hip_set_option(_lib.OPT_DIGITS_ROUTE, 0) == 0
+    assert _lib.lib.bsi_hip_set_option(_lib.OPT_BUILD_ITEMS, 4) == 0
+    assert _lib.lib.bsi_hip_set_option(_lib.OPT_BUILD_ITEMS, 3) == 1
+    assert _lib.lib.bsi_hip_set_option(_lib.OPT_BUILD_ITEMS, 0) == 0
     assert _lib.lib.bsi_hip_set_option(999, 1) == 1
     assert b"unknown option" in _lib.lib.bsi_hip_last_error()
 

@@ -133,6 +133,43 @@ def test_build_huge_magnitudes_take_the_wide_path(hip, oracle):
     assert shifts.max() >= 30
 
 
+@pytest.mark.parametrize("dec", [0, 1, 2, 3])
+@pytest.mark.parametrize("per_wave", [0, 1, 2, 4, 8])
+def test_build_rounding_routes_and_items_per_wave(hip, oracle, dec, per_wave):
+    """10^dec of 1, 10 and 100 round from the float's mantissa, 1000 in float64; values around the limits of the
+    integer route (2^23, ties, denormals, signed zeros) and every items-per-wave variant of the kernel."""
+    Q, d = 37, 1024
+    rng = np.random.default_rng(dec * 10 + per_wave)
+    x = (rng.standard_normal((Q, d)) * 10.0 ** (2 - dec)).astype(np.float32)
+    special = np.array([0.125, -0.125, 0.375, 2.5, -2.5, 0.5, -0.5, 1.5, 0.005, -0.005, 0.015, 0.045, 1e-40, -1e-40, 0.0, -0.0,
+                        1.17549435e-38, 8388607.5, 8388608.0, -8388607.5, 4194304.25, 4194303.75, 1048576.125, 16777216.0,
+                        21474836.0, 21474838.0, 0.49999997, 0.004999999888241291, 0.5000001], dtype=np.float32)
+    x[3, :special.size] = special
+    x[7, 300:300 + special.size] = -special
+    x[11, 512:768] = 0.0
+    ints, shifts, scales = oracle.quantize_fixed(x, dec, 7, True)
+    xd = dev(x)
+    words = torch.full((Q, 7, d // 64), -1, dtype=torch.int64, device="cuda")
+    sh = torch.full(shifts.shape, -1, dtype=torch.int32, device="cuda")
+    sc = torch.zeros(scales.shape, dtype=torch.float32, device="cuda")
+    i8 = torch.full((Q, d), 77, dtype=torch.int8, device="cuda")
+    hip.check(hip.lib.bsi_hip_set_option(hip.OPT_BUILD_ITEMS, per_wave), "opt")
+    try:
+        hip.check(hip.lib.bsi_hip_build_fixed(xd.data_ptr(), 0, Q, d, dec, 7, 1, 0.0, words.data_ptr(), sh.data_ptr(),
+                                              sc.data_ptr(), i8.data_ptr(), st()), "build")
+        torch.cuda.synchronize()
+    finally:
+        hip.check(hip.lib.bsi_hip_set_option(hip.OPT_BUILD_ITEMS, 0), "opt")
+    np.testing.assert_array_equal(sh.cpu().numpy(), shifts)
+    np.testing.assert_array_equal(sc.cpu().numpy(), scales)
+    np.testing.assert_array_equal(host_u64(words), oracle.pack(ints, 7))
+    e = np.arange(d)
+    pos = (e // 32) * 32 + ((e % 32) % 8) * 4 + (e % 32) // 8
+    want8 = np.zeros((Q, d), dtype=np.int64)
+    want8[:, pos] = ints << 1
+    np.testing.assert_array_equal(i8.cpu().numpy().astype(np.int64), want8)
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_build_half_inputs(hip, oracle, dtype):
     x = torch.from_numpy(_inputs(12, 1024, 5)).to(dtype)
