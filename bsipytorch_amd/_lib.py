@@ -64,6 +64,8 @@ PROTOTYPES = {
     "bsi_hip_int8_tiled_bytes": [_i64, _i],
     "bsi_hip_planes_to_int8_tiled": [_vp, _i64, _i, _i, _vp, _vp],
     "bsi_hip_dot_weighted": [_vp, _vp, _i, _i, _vp, _i, _vp, _i, _i64, _i64, _vp, _f, _i64, _vp, _vp],
+    "bsi_hip_dot_weighted_f64": [_vp, _vp, _i, _i, _vp, _i, _vp, _i, _i64, _i64, _vp, _i64, _vp, _vp],
+    "bsi_hip_quantize_trunc_to_int64": [_vp, _i, _i64, _f, _vp, _vp],
     "bsi_hip_dot_timed": [_vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _i, _i64, _i64, _f, _i64, _vp, _i, _vp, _sz, _i,
                           ctypes.POINTER(_f), _vp],
     "bsi_hip_probe_valu_popcount": [ctypes.POINTER(_d), _vp],

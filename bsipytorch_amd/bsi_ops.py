@@ -318,6 +318,16 @@ def _build_decimal(x2d: torch.Tensor, decimal_places: int):
     if Q > 0 and d > 0:
         check(lib.bsi_hip_quantize_round_to_int64(x2d.data_ptr(), _dtype_code(x2d), Q * d, 10.0 ** int(decimal_places),
                                                   ints.data_ptr(), st), "bsi_hip_quantize_round_to_int64")
+    return _planes_from_ints(ints)
+
+
+def _planes_from_ints(ints: torch.Tensor):
+    """Two's-complement planes of an int64 matrix [Q, d] with the decimal builder's slice rule
+    (bsi_vector_cuda.cpp:746-754): -> (words [Q,S,W] int64, slice_weights [Q,S] float32, S, row_negative [Q])."""
+    dev = ints.device
+    Q, d = ints.shape
+    W = (d + 63) // 64 if d > 0 else 1
+    st = _stream()
     max_abs = torch.empty((1,), dtype=torch.int64, device=dev)
     negative = torch.zeros((Q,), dtype=torch.int32, device=dev)
     check(lib.bsi_hip_decimal_stats(ints.data_ptr() if Q > 0 and d > 0 else None, Q, d, max_abs.data_ptr(),
@@ -1111,19 +1121,9 @@ def debug_quantize_int64_cpu(values: torch.Tensor, decimal_places: int) -> torch
     return torch.where(x >= 0, torch.floor(x + 0.5), -torch.floor(-x + 0.5)).to(torch.int64)
 
 
-def _cpu_path_absent(name: str):
-    def fn(*_a, **_k):
-        raise RuntimeError(
-            f"bsi_ops.{name}: the CPU BSI path of the reference lives in the bsiCPP library, which is not part "
-            "of this build; use the *_cuda functions")
-    fn.__name__ = name
-    fn.__doc__ = "CPU decimal-path entry of the reference (bsiFunctions.cpp:811-846); not built here."
-    return fn
-
-
-for _n in ("dot_product", "dot_product_decimal", "vector_dot_product", "vector_dot_product_no_precison",
-           "random_number_dot_product_vector", "random_number_dot_product_bsi", "batch_dot_product", "build_bsi_keys",
-           "build_bsi_query", "batch_dot_product_prebuilt", "batch_dot_product_prebuilt_capsule", "keyset_slice_stats",
-           "tensor_slice_stats", "keyset_size_on_disk", "save_keyset", "debug_bsi_query_words"):
-    globals()[_n] = _cpu_path_absent(_n)
-del _n
+# The reference's scalar ("non-CUDA") entry points (bsiFunctions.cpp:811-846): served by the device kernels here.
+from .bsi_scalar import (  # noqa: E402,F401
+    PrebuiltBSIKeys, PrebuiltBSIQuery, batch_dot_product, batch_dot_product_prebuilt, batch_dot_product_prebuilt_capsule,
+    build_bsi_keys, build_bsi_query, debug_bsi_query_words, dot_product, dot_product_decimal, keyset_size_on_disk,
+    keyset_slice_stats, random_number_dot_product_bsi, random_number_dot_product_vector, save_keyset, tensor_slice_stats,
+    vector_dot_product, vector_dot_product_no_precison)

@@ -27,6 +27,15 @@ __global__ void round_to_int64_kernel(const T* __restrict__ x, int64_t total, do
         out[i] = round_scaled(load_as_float<T>(x, i), dec_scale);
 }
 
+// (long long)(x * factor) with the product rounded to float first and the conversion towards zero: the scalar
+// entry points' value rule (bsiFunctions.cpp:265-271)
+template <typename T>
+__global__ void trunc_to_int64_kernel(const T* __restrict__ x, int64_t total, float factor, long long* __restrict__ out) {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += stride)
+        out[i] = static_cast<long long>(__fmul_rn(load_as_float<T>(x, i), factor));
+}
+
 __global__ void apply_shift_clamp_kernel(long long* __restrict__ ints, int64_t total, int64_t d, int chunks,
                                          const int* __restrict__ shifts, long long qmin, long long qmax) {
     // chunks == 0: one shift per row; else one per (row, col >> 8)
@@ -500,6 +509,18 @@ extern "C" int bsi_hip_quantize_round_to_int64(const void* x, int dtype, int64_t
                                                  0, as_stream(stream), static_cast<const T*>(x), total, dec_scale,
                                                  reinterpret_cast<long long*>(out)));
     BSI_LAUNCH_CHECK("round_to_int64_kernel");
+    return BSI_OK;
+}
+
+extern "C" int bsi_hip_quantize_trunc_to_int64(const void* x, int dtype, int64_t total, float factor, int64_t* out,
+                                               void* stream) {
+    BSI_REQUIRE(total >= 0, "total must be >= 0");
+    if (total == 0) return BSI_OK;
+    BSI_REQUIRE(x && out, "null pointer");
+    BSI_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(trunc_to_int64_kernel<T>, dim3(grid_elementwise(total)), dim3(kBlock),
+                                                 0, as_stream(stream), static_cast<const T*>(x), total, factor,
+                                                 reinterpret_cast<long long*>(out)));
+    BSI_LAUNCH_CHECK("trunc_to_int64_kernel");
     return BSI_OK;
 }
 

@@ -1878,7 +1878,8 @@ template <int WB, bool kTiled>
 __global__ __launch_bounds__(256) void dot_weighted_kernel(
     const unsigned long long* __restrict__ A, const float* __restrict__ Aw, int Sa, int W64,
     const unsigned long long* __restrict__ B, const float* __restrict__ Bw, int Sb, int chunks, int64_t R, int64_t Q,
-    const long long* __restrict__ key_indices, float scale_inv, int64_t R_total, float* __restrict__ out) {
+    const long long* __restrict__ key_indices, float scale_inv, int64_t R_total, float* __restrict__ out,
+    double* __restrict__ out64) {
     extern __shared__ __attribute__((aligned(16))) unsigned char wlds[];
     const int strideA = Sa * WB + 1, strideB = Sb * WB + 1;  // in 64-bit words; odd, so rows start in different banks
     unsigned long long* As = reinterpret_cast<unsigned long long*>(wlds);  // [32][strideA]
@@ -1951,7 +1952,8 @@ __global__ __launch_bounds__(256) void dot_weighted_kernel(
             const int64_t q = q0 + tq + 16 * a, r = r0 + tr + 16 * b;
             if (q < Q && r < R) {
                 const int64_t col = key_indices ? key_indices[r] : r;
-                out[q * R_total + col] = static_cast<float>(acc[a][b]) * scale_inv;
+                if (out64 != nullptr) out64[q * R_total + col] = acc[a][b];  // the exact weighted sum itself
+                else out[q * R_total + col] = static_cast<float>(acc[a][b]) * scale_inv;
             }
         }
 }
@@ -2513,7 +2515,7 @@ extern "C" int bsi_hip_dot_ewah_query(const uint64_t* comp_words, const int64_t*
 template <int WB, bool kTiled>
 static int launch_dot_weighted(const uint64_t* A, const float* Aw, int Sa, int W64, const uint64_t* B, const float* Bw,
                                int Sb, int64_t R, int64_t Q, const int64_t* key_indices, float scale_inv,
-                               int64_t R_total, float* out, hipStream_t st) {
+                               int64_t R_total, float* out, double* out64, hipStream_t st) {
     const size_t lds = static_cast<size_t>(32) * ((Sa * WB + 1) + (Sb * WB + 1)) * 8 + static_cast<size_t>(32) * (Sa + Sb) * 4;
     if (lds > 150 * 1024) return fail(BSI_ERR_UNSUPPORTED, "slice counts %d + %d do not fit the LDS tile", Sa, Sb);
     static bool configured = false;
@@ -2526,15 +2528,14 @@ static int launch_dot_weighted(const uint64_t* A, const float* Aw, int Sa, int W
     hipLaunchKernelGGL((dot_weighted_kernel<WB, kTiled>), grid, dim3(256), lds, st,
                        reinterpret_cast<const unsigned long long*>(A), Aw, Sa, W64,
                        reinterpret_cast<const unsigned long long*>(B), Bw, Sb, (W64 + 3) / 4, R, Q,
-                       reinterpret_cast<const long long*>(key_indices), scale_inv, R_total, out);
+                       reinterpret_cast<const long long*>(key_indices), scale_inv, R_total, out, out64);
     BSI_LAUNCH_CHECK("dot_weighted_kernel");
     return BSI_OK;
 }
 
-extern "C" int bsi_hip_dot_weighted(const uint64_t* A, const float* Aw, int Sa, int W64, const uint64_t* B,
-                                    int b_layout, const float* Bw, int Sb, int64_t R, int64_t Q,
-                                    const int64_t* key_indices, float scale_inv, int64_t R_total, float* out,
-                                    void* stream) {
+static int dot_weighted_impl(const uint64_t* A, const float* Aw, int Sa, int W64, const uint64_t* B, int b_layout,
+                             const float* Bw, int Sb, int64_t R, int64_t Q, const int64_t* key_indices, float scale_inv,
+                             int64_t R_total, float* out, double* out64, void* stream) {
     BSI_REQUIRE(R >= 0 && Q >= 0 && W64 >= 1, "bad shape");
     BSI_REQUIRE(Sa >= 1 && Sa <= 64 && Sb >= 1 && Sb <= 64, "slice counts must be in [1, 64] (got %d, %d)", Sa, Sb);
     BSI_REQUIRE(R_total >= R, "R_total (%lld) < R (%lld)", static_cast<long long>(R_total), static_cast<long long>(R));
@@ -2542,15 +2543,28 @@ extern "C" int bsi_hip_dot_weighted(const uint64_t* A, const float* Aw, int Sa, 
                 "the weighted dot reads key planes (canonical or tiled16), got layout %d", b_layout);
     BSI_REQUIRE((Q + 31) / 32 <= 65535, "too many query rows for one launch");
     if (R == 0 || Q == 0) return BSI_OK;
-    BSI_REQUIRE(A && Aw && B && Bw && out, "null pointer");
+    BSI_REQUIRE(A && Aw && B && Bw && (out || out64), "null pointer");
     hipStream_t st = as_stream(stream);
     const bool tiled = b_layout == BSI_LAYOUT_TILED16;
     // 8 words of every slice per step while that fits 60 KiB of LDS, else 2
-    if (Sa + Sb <= 28)
-        return tiled ? launch_dot_weighted<8, true>(A, Aw, Sa, W64, B, Bw, Sb, R, Q, key_indices, scale_inv, R_total, out, st)
-                     : launch_dot_weighted<8, false>(A, Aw, Sa, W64, B, Bw, Sb, R, Q, key_indices, scale_inv, R_total, out, st);
-    return tiled ? launch_dot_weighted<2, true>(A, Aw, Sa, W64, B, Bw, Sb, R, Q, key_indices, scale_inv, R_total, out, st)
-                 : launch_dot_weighted<2, false>(A, Aw, Sa, W64, B, Bw, Sb, R, Q, key_indices, scale_inv, R_total, out, st);
+#define BSI_WEIGHTED_GO(WB, T) \
+    launch_dot_weighted<WB, T>(A, Aw, Sa, W64, B, Bw, Sb, R, Q, key_indices, scale_inv, R_total, out, out64, st)
+    if (Sa + Sb <= 28) return tiled ? BSI_WEIGHTED_GO(8, true) : BSI_WEIGHTED_GO(8, false);
+    return tiled ? BSI_WEIGHTED_GO(2, true) : BSI_WEIGHTED_GO(2, false);
+#undef BSI_WEIGHTED_GO
+}
+
+extern "C" int bsi_hip_dot_weighted(const uint64_t* A, const float* Aw, int Sa, int W64, const uint64_t* B,
+                                    int b_layout, const float* Bw, int Sb, int64_t R, int64_t Q,
+                                    const int64_t* key_indices, float scale_inv, int64_t R_total, float* out,
+                                    void* stream) {
+    return dot_weighted_impl(A, Aw, Sa, W64, B, b_layout, Bw, Sb, R, Q, key_indices, scale_inv, R_total, out, nullptr, stream);
+}
+
+extern "C" int bsi_hip_dot_weighted_f64(const uint64_t* A, const float* Aw, int Sa, int W64, const uint64_t* B,
+                                        int b_layout, const float* Bw, int Sb, int64_t R, int64_t Q,
+                                        const int64_t* key_indices, int64_t R_total, double* out, void* stream) {
+    return dot_weighted_impl(A, Aw, Sa, W64, B, b_layout, Bw, Sb, R, Q, key_indices, 1.0f, R_total, nullptr, out, stream);
 }
 
 extern "C" int bsi_hip_planes_to_int8_digits(const uint64_t* words, int64_t rows, int S, int W64, int8_t* out,

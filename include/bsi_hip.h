@@ -60,6 +60,12 @@ int bsi_hip_device_info(char* arch, int arch_len, int* cu_count, int* lds_bytes)
 int bsi_hip_quantize_round_to_int64(const void* x_device, int dtype, int64_t total, double dec_scale,
                                     int64_t* out_device, void* stream);
 
+/* out[i] = (int64)(float(x[i]) * factor): the product rounded to float, the conversion towards zero.  The value rule
+ * of the reference's scalar entry points dot_product / vector_dot_product (bsiFunctions.cpp:265-271, :165-170:
+ * static_cast<long>(m_a[i] * precision_factor_long)). */
+int bsi_hip_quantize_trunc_to_int64(const void* x_device, int dtype, int64_t total, float factor, int64_t* out,
+                                    void* stream);
+
 /* Per-row / per-(row, 256-element chunk) shift and power-of-two scale from already rounded ints.
  * Replace launch_compute_row_shift_scale / launch_compute_chunk_shift_scale
  * (bsi_cuda_kernels_quant.cuh:670-700). shifts/scales are [Q] or [Q, chunks]. */
@@ -267,6 +273,14 @@ int bsi_hip_dot_ewah_query(const uint64_t* comp_words, const int64_t* comp_off, 
 int bsi_hip_dot_weighted(const uint64_t* A, const float* Aw, int Sa, int W64, const uint64_t* B, int b_layout,
                          const float* Bw, int Sb, int64_t R, int64_t Q, const int64_t* key_indices, float scale_inv,
                          int64_t R_total, float* out, void* stream);
+
+/* The same weighted sum, unscaled and unrounded, as float64: out[q, idx[r]] = sum of popcount * (Aw * Bw), exact
+ * while its magnitude stays below 2^53.  The double results of the reference's scalar entry points divide this
+ * integer by 10^(decimals) on the host (bsiFunctions.cpp:368-373, :455-459: raw = vec->dot(other);
+ * score = raw / scale). */
+int bsi_hip_dot_weighted_f64(const uint64_t* A, const float* Aw, int Sa, int W64, const uint64_t* B, int b_layout,
+                             const float* Bw, int Sb, int64_t R, int64_t Q, const int64_t* key_indices, int64_t R_total,
+                             double* out, void* stream);
 
 /* Decimal-mode operands on the matrix cores.  bsi_hip_planes_to_int8_digits splits the two's-complement values
  * of S planes [rows, S, W64] into ceil(S / 7) int8 digit images out[digit][row][chunks * 256] (value =

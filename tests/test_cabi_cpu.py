@@ -96,9 +96,19 @@ def test_module_surface_matches_reference_names():
            "keyset_slice_stats", "tensor_slice_stats", "keyset_size_on_disk", "save_keyset", "debug_bsi_query_words"]
     for n in gpu + cpu + ["debug_quantize_int64_cpu", "CUDA_BUILDER_VERSION"]:
         assert hasattr(bsi_ops, n), n
-    for n in cpu:
-        with pytest.raises(RuntimeError, match="bsiCPP"):
-            getattr(bsi_ops, n)(torch.zeros(2), torch.zeros(2))
+    # the scalar entry points run on the device kernels too: without a GPU they refuse, they do not fall back
+    if not torch.cuda.is_available():
+        with pytest.raises(RuntimeError, match="no GPU visible"):
+            bsi_ops.dot_product(torch.zeros(2), torch.zeros(2), 10.0)
+        with pytest.raises(RuntimeError, match="no GPU visible"):
+            bsi_ops.batch_dot_product(torch.zeros(2), torch.zeros(3, 2), 2)
+        with pytest.raises(RuntimeError, match="no GPU visible"):
+            bsi_ops.tensor_slice_stats(torch.zeros(2), 2)
+    with pytest.raises(RuntimeError, match="must be 2D"):
+        bsi_ops.build_bsi_keys(torch.zeros(2), 2)
+    with pytest.raises(RuntimeError, match="Invalid BSI keys capsule"):
+        bsi_ops.keyset_slice_stats(object())
+    assert bsi_ops.PrebuiltBSIKeys.name == "PrebuiltBSIKeys" and bsi_ops.PrebuiltBSIQuery.name == "PrebuiltBSIQuery"
     assert bsi_ops.get_last_query_build_profile_cuda() == (0, 0, 0)
     assert bsi_ops.PrebuiltBSIKeysCUDA.name == "PrebuiltBSIKeysCUDA"
     assert bsi_ops.PrebuiltBSIQueryBatchCUDA.name == "PrebuiltBSIQueryBatchCUDA"
