@@ -1182,6 +1182,45 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
 // indexed by chunk; after a workgroup barrier 256 * NT lanes run the fp32 chain of their (query,
 // key) pair over the chunks in order, so the result is bit-identical to a sequential pass
 // whatever the number of waves.  Problems with more chunks than LDS slots run in several passes.
+// The epilogue's operands (the key's slice-0 weight and, optionally, its bias), requested when the kernel starts
+// instead of after the chain, where two dependent cache misses would end every workgroup.  Buffer loads: a lane
+// without an output, or a call without bias, reads nothing and gets 0; no branch, so the loads stay where they
+// are written.
+struct EpilogueOperands {
+    float bw, bias;
+};
+__device__ __forceinline__ EpilogueOperands load_epilogue_operands(const float* Bw, const float* bias, int64_t R, bool valid,
+                                                                   int64_t r) {
+    const bsi_rsrc wr = make_rsrc(Bw, static_cast<size_t>(R) * 6 * sizeof(float));
+    const bsi_rsrc br = make_rsrc(bias != nullptr ? bias : Bw, bias != nullptr ? static_cast<size_t>(R) * sizeof(float) : 0);
+    EpilogueOperands e;
+    e.bw = __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(wr, valid ? static_cast<int>(r * 24) : -1, 0, 0));
+    e.bias = __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(br, valid ? static_cast<int>(r * 4) : -1, 0, 0));
+    return e;
+}
+
+// The fp32 chain of one output over chunks [c0, c1): accf = fmaf(float(I_c), scale_c * down, accf) in chunk order,
+// eight chunks' integers and scales fetched ahead of their eight dependent steps (fetched one step at a time the
+// chain costs an LDS or cache round trip per chunk: 4 us of a 17 us kernel at 64 chunks).  int_at(c) / scale_at(c)
+// read chunk c's integer and chunk scale; the arithmetic and its order are those of the one-step loop.
+template <typename IntAt, typename ScaleAt>
+__device__ __forceinline__ float chain_chunks(float accf, int c0, int c1, float down, IntAt int_at, ScaleAt scale_at) {
+    int c = c0;
+    for (; c + 8 <= c1; c += 8) {
+        int v[8];
+        float sc[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            v[u] = int_at(c + u);
+            sc[u] = scale_at(c + u);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) accf = fmaf(static_cast<float>(v[u]), sc[u] * down, accf);
+    }
+    for (; c < c1; ++c) accf = fmaf(static_cast<float>(int_at(c)), scale_at(c) * down, accf);
+    return accf;
+}
+
 constexpr int kStreamMaxQ = 32;        // above this the 128 x 128 tiled kernel takes over
 constexpr int kStreamLdsInts = 16384;  // at most 64 KiB of chunk accumulators per pass
 
@@ -1220,6 +1259,7 @@ __global__ __launch_bounds__(1024) void dot_mfma_stream_kernel(
     const float down = __uint_as_float(static_cast<uint32_t>(127 - down_shift) << 23);
     const float* csrc = qscale + (cvalid ? cq : 0) * qscale_stride;
     const int sstep = (qscale_stride == 1) ? 0 : 1;
+    const EpilogueOperands eo = load_epilogue_operands(Bw, bias, R, cvalid, cr);
 
     for (int p0 = 0; p0 < chunks; p0 += pass_chunks) {
         const int pend = (p0 + pass_chunks < chunks) ? p0 + pass_chunks : chunks;
@@ -1288,17 +1328,17 @@ __global__ __launch_bounds__(1024) void dot_mfma_stream_kernel(
         }
         __syncthreads();
         if (cvalid) {
-            for (int cc = p0; cc < pend; ++cc) {
-                const int v = ints[(cc - p0) * kSlot + tid];
-                accf = fmaf(static_cast<float>(v), csrc[cc * sstep] * down, accf);
-                if (kInts) chunk_ints[(cq * R + cr) * chunks + cc] = v >> down_shift;
-            }
+            accf = chain_chunks(accf, p0, pend, down, [&](int cc) { return ints[(cc - p0) * kSlot + tid]; },
+                                [&](int cc) { return csrc[cc * sstep]; });
+            if (kInts)
+                for (int cc = p0; cc < pend; ++cc)
+                    chunk_ints[(cq * R + cr) * chunks + cc] = ints[(cc - p0) * kSlot + tid] >> down_shift;
         }
         if (pend < chunks) __syncthreads();
     }
     if (cvalid) {
-        float v = (accf * Bw[cr * 6]) * scale_inv;
-        if (bias != nullptr) v = v + bias[cr];
+        float v = (accf * eo.bw) * scale_inv;
+        if (bias != nullptr) v = v + eo.bias;
         out[static_cast<size_t>(cq) * R_total + cr] = v;
     }
 }
@@ -1483,6 +1523,7 @@ __global__ __launch_bounds__(1024) void dot_mfma_stream_fused_kernel(
     // the first pass's first chunk; a wave without one loads the last chunk's planes for nothing, because a branch
     // here would make the compiler's load counting assume the worst and wait for these loads in the query build
     load_keys(wave < pass_chunks ? wave : pass_chunks - 1, kc);
+    const EpilogueOperands eo = load_epilogue_operands(Bw, bias, R, cvalid, cr);
     __builtin_amdgcn_sched_barrier(0);
     {
         unsigned wide = 0u;  // items left to the 64-bit routine
@@ -1570,16 +1611,14 @@ __global__ __launch_bounds__(1024) void dot_mfma_stream_fused_kernel(
         }
         __syncthreads();
         if (cvalid) {
-            for (int cc = p0; cc < pend; ++cc) {
-                const int v = ints[(cc - p0) * kSlot + tid];
-                accf = fmaf(static_cast<float>(v), qsc[cc * Q + cn] * down, accf);
-            }
+            accf = chain_chunks(accf, p0, pend, down, [&](int cc) { return ints[(cc - p0) * kSlot + tid]; },
+                                [&](int cc) { return qsc[cc * Q + cn]; });
         }
         if (pend < chunks) __syncthreads();
     }
     if (cvalid) {
-        float v = (accf * Bw[cr * 6]) * scale_inv;
-        if (bias != nullptr) v = v + bias[cr];
+        float v = (accf * eo.bw) * scale_inv;
+        if (bias != nullptr) v = v + eo.bias;
         out[static_cast<size_t>(cn) * R_total + cr] = v;
     }
 }
@@ -1689,11 +1728,10 @@ __global__ __launch_bounds__(1024) void dot_mfma_stream_ewah_kernel(
         }
         __syncthreads();
         if (cvalid) {
-            for (int cc = p0; cc < pend; ++cc) {
-                const int v = ints[(cc - p0) * 256 + ckey];  // query 0, key ckey
-                accf = fmaf(static_cast<float>(v), qscale[cc * sstep] * down, accf);
-                if (kInts) chunk_ints[cr * chunks + cc] = v >> down_shift;
-            }
+            accf = chain_chunks(accf, p0, pend, down, [&](int cc) { return ints[(cc - p0) * 256 + ckey]; },  // query 0, key ckey
+                                [&](int cc) { return qscale[cc * sstep]; });
+            if (kInts)
+                for (int cc = p0; cc < pend; ++cc) chunk_ints[cr * chunks + cc] = ints[(cc - p0) * 256 + ckey] >> down_shift;
         }
         if (pend < chunks) __syncthreads();
     }
