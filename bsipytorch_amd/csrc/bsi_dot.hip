@@ -1101,6 +1101,46 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
             const int64_t q = q0 + wq * (WN * 16) + b * 16 + ln;
             qf[b] = (q < Q) ? static_cast<double>(qscale[q * qscale_stride]) * down2 : 0.0;
         }
+        if (key_indices == nullptr) {
+            // identity key order: the key factors and biases of all the wave's rows in one round trip (buffer loads:
+            // rows past R and a missing bias read nothing and give 0), then four outputs per store
+            float kfv[WM][4], biv[WM][4];
+            const bsi_rsrc wrs = make_rsrc(Bw, static_cast<size_t>(R) * Sb * sizeof(float));
+            const bsi_rsrc brs = make_rsrc(bias != nullptr ? bias : Bw, bias != nullptr ? static_cast<size_t>(R) * sizeof(float) : 0);
+#pragma unroll
+            for (int a = 0; a < WM; ++a) {
+                const int rb = static_cast<int>(r0 + wr * (WM * 16) + a * 16 + lg * 4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    kfv[a][e] = __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(wrs, (rb + e) * Sb * 4, 0, 0));
+                    biv[a][e] = __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(brs, (rb + e) * 4, 0, 0));
+                }
+            }
+#pragma unroll
+            for (int a = 0; a < WM; ++a) {
+                const int64_t rb = r0 + wr * (WM * 16) + a * 16 + lg * 4;
+#pragma unroll
+                for (int b = 0; b < WN; ++b) {
+                    const int64_t q = q0 + wq * (WN * 16) + b * 16 + ln;
+                    if (q >= Q) continue;
+                    float v[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        v[e] = static_cast<float>(static_cast<double>(acc0[a][b][e]) * qf[b] * static_cast<double>(kfv[a][e])) * scale_inv;
+                        if (bias != nullptr) v[e] = v[e] + biv[a][e];
+                    }
+                    float* dst = out + static_cast<size_t>(q) * R_total + rb;
+                    if (rb + 3 < R && ((reinterpret_cast<uintptr_t>(dst) & 15) == 0)) {
+                        *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (rb + e < R) dst[e] = v[e];
+                    }
+                }
+            }
+            return;
+        }
 #pragma unroll
         for (int a = 0; a < WM; ++a) {
             const int64_t rb = r0 + wr * (WM * 16) + a * 16 + lg * 4;
@@ -1136,22 +1176,33 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
                 if (kInts && int_off[a][b] >= 0 && e < int_rows[a])
                     chunk_ints[int_off[a][b] + static_cast<int64_t>(e) * chunks + (chunks - 1)] = v >> down_shift;
             }
+    // The key scales and biases of all the wave's rows in one go (the chunk accumulators are dead by now, so the
+    // registers are there): one cache round trip before the stores instead of one per 16-key tile.  Buffer loads:
+    // rows past R, and every bias of a call without one, read nothing and give 0.
+    float bs[WM][4], bi[WM][4];
+    {
+        const bsi_rsrc wrs = make_rsrc(Bw, static_cast<size_t>(R) * Sb * sizeof(float));
+        const bsi_rsrc brs = make_rsrc(bias != nullptr ? bias : Bw, bias != nullptr ? static_cast<size_t>(R) * sizeof(float) : 0);
+#pragma unroll
+        for (int a = 0; a < WM; ++a) {
+            const int rb = static_cast<int>(r0 + wr * (WM * 16) + a * 16 + lg * 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                bs[a][e] = __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(wrs, (rb + e) * Sb * 4, 0, 0));
+                bi[a][e] = __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(brs, (rb + e) * 4, 0, 0));
+            }
+        }
+    }
 #pragma unroll
     for (int a = 0; a < WM; ++a) {
         const int64_t rb = r0 + wr * (WM * 16) + a * 16 + lg * 4;
-        float bs[4], bi[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            bs[e] = (rb + e < R) ? Bw[(rb + e) * Sb] : 0.0f;
-            bi[e] = (bias != nullptr && rb + e < R) ? bias[rb + e] : 0.0f;
-        }
 #pragma unroll
         for (int b = 0; b < WN; ++b)
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 // (acc * key scale) * scale_inv, then + bias: each step rounded on its own, as separate kernels would
-                float v = ((accf[a][b][e] * down) * bs[e]) * scale_inv;
-                if (bias != nullptr) v = v + bi[e];
+                float v = ((accf[a][b][e] * down) * bs[a][e]) * scale_inv;
+                if (bias != nullptr) v = v + bi[a][e];
                 accf[a][b][e] = v;
             }
 #pragma unroll
