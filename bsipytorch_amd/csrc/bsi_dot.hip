@@ -2746,16 +2746,16 @@ extern "C" int bsi_hip_dot_timed(const uint64_t* A, const int8_t* A_ints8, const
     BSI_HIP_CHECK(hipEventCreate(&e0));
     BSI_HIP_CHECK(hipEventCreate(&e1));
     int rc = BSI_OK;
-    hipEventRecord(e0, st);
+    hipError_t se = hipEventRecord(e0, st);
     for (int i = 0; i < iters && rc == BSI_OK; ++i)
         rc = bsi_hip_dot(A, A_ints8, A_chunk_scales, A_scale_stride, Sa, W64, B, b_layout, Bw, Sb, R, Q, scale_inv,
                          R_total, out, nullptr, core, workspace, workspace_bytes, stream);
-    hipEventRecord(e1, st);
-    hipError_t se = hipEventSynchronize(e1);
+    if (se == hipSuccess) se = hipEventRecord(e1, st);
+    if (se == hipSuccess) se = hipEventSynchronize(e1);
     float ms = 0.0f;
     if (se == hipSuccess) se = hipEventElapsedTime(&ms, e0, e1);
-    hipEventDestroy(e0);
-    hipEventDestroy(e1);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
     if (rc != BSI_OK) return rc;
     if (se != hipSuccess) return fail(BSI_ERR_HIP, "event timing failed: %s", hipGetErrorString(se));
     *mean_us = ms * 1000.0f / static_cast<float>(iters);
