@@ -3,8 +3,10 @@
 TEST INFRASTRUCTURE ONLY: imported by ``tests/``, by the smoke check and by the CPU-baseline
 leg of the benchmark, never by the library.  Each function forwards to the C restatement of
 the reference block named in its docstring (paths relative to the reference's
-``bsi_ops/csrc/cuda/``); the decimal-mode functions at the end are numpy.  Every function is
-pinned by an independent check in ``tests/test_oracle_*.py`` (none is "parity unpinned").
+``bsi_ops/csrc/cuda/``); the decimal-mode functions and the scalar entry points at the end are
+numpy.  Every function is pinned by an independent check in ``tests/test_oracle_*.py`` (none is
+"parity unpinned"; of the scalar entry points only the VALUES are restated: their byte counts and
+slice statistics come out of the bsiCPP containers, which the reference's tree does not hold).
 """
 from __future__ import annotations
 
@@ -301,3 +303,42 @@ def int8_digits(ints: np.ndarray, S: int) -> np.ndarray:
         out[j] = (v >> (7 * j)) & 127
     out[n - 1] = v >> (7 * (n - 1))  # arithmetic shift keeps the sign
     return out
+
+
+# --------------------------------------------------------------------------- the scalar entry points (values only)
+
+
+def trunc_scaled(x: np.ndarray, factor: float) -> np.ndarray:
+    """``static_cast<long>(x * (long)factor)`` (bsi_ops/bsiFunctions.cpp:265-271, :165-170): the product is a
+    float (float times long converts the long), the conversion goes towards zero."""
+    return (np.asarray(x, dtype=np.float32) * np.float32(int(factor))).astype(np.int64)
+
+
+def scalar_dot_product(m: np.ndarray, n: np.ndarray, precision_factor: float) -> float:
+    """bsi_ops/bsiFunctions.cpp:249-340: exact dot of the truncated integers over
+    ``float(precision_factor * precision_factor)`` (a float product), in double."""
+    raw = int(trunc_scaled(m, precision_factor).astype(object) @ trunc_scaled(n, precision_factor).astype(object))
+    pf = np.float32(precision_factor)
+    return float(raw) / float(np.float32(pf * pf))
+
+
+def scalar_dot_product_decimal(m: np.ndarray, n: np.ndarray, decimal_places: int) -> float:
+    """bsi_ops/bsiFunctions.cpp:342-384: exact dot of the rounded integers (half away from zero, the builders'
+    rule) over ``10^(2 dec)`` (1 when dec = 0), in double."""
+    raw = int(round_to_int64(np.asarray(m, dtype=np.float32), decimal_places).astype(object)
+              @ round_to_int64(np.asarray(n, dtype=np.float32), decimal_places).astype(object))
+    total = 2 * int(decimal_places)
+    return float(raw) / (10.0 ** total if total > 0 else 1.0)
+
+
+def scalar_batch_dot_product(q: np.ndarray, K: np.ndarray, decimal_places: int) -> np.ndarray:
+    """bsi_ops/bsiFunctions.cpp:426-478: scalar_dot_product_decimal of q with every row of K, float64 [num_keys]."""
+    return np.array([scalar_dot_product_decimal(q, row, decimal_places) for row in np.asarray(K)], dtype=np.float64)
+
+
+def scalar_vector_dot_product(m: np.ndarray, n: np.ndarray, precision_factor: float) -> int:
+    """bsi_ops/bsiFunctions.cpp:157-208: the plain-integer baseline, accumulated in an ``int`` (``auto res = 0``),
+    hence reduced to 32 bits, and not divided by the factor."""
+    raw = int(trunc_scaled(m, precision_factor).astype(object) @ trunc_scaled(n, precision_factor).astype(object))
+    return (raw + (1 << 31)) % (1 << 32) - (1 << 31)
+

@@ -59,17 +59,18 @@ def test_known_answers_of_the_reference_scripts(ops):
 
 
 @pytest.mark.parametrize("n,dec", [(1, 2), (63, 0), (64, 1), (1000, 2), (4097, 3)])
-def test_dot_product_decimal_is_the_exact_integer_dot(ops, n, dec):
+def test_dot_product_decimal_is_the_exact_integer_dot(ops, oracle, n, dec):
     rng = np.random.default_rng(n + dec)
     m = (rng.standard_normal(n) * 7).astype(np.float32)
     k = (rng.standard_normal(n) * 0.3).astype(np.float32)
     res, _, _, _ = ops.dot_product_decimal(torch.from_numpy(m), torch.from_numpy(k).cuda(), dec)
     exact = int(_round_half_away(m, dec) @ _round_half_away(k, dec))
-    assert res == exact / 10.0 ** (2 * dec)
+    assert res == exact / (10.0 ** (2 * dec) if dec > 0 else 1.0)
+    assert res == oracle.scalar_dot_product_decimal(m, k, dec)
 
 
 @pytest.mark.parametrize("pf", [1.0, 10.0, 1000.0, 12345.0])
-def test_dot_product_truncates_the_float_product(ops, pf):
+def test_dot_product_truncates_the_float_product(ops, oracle, pf):
     rng = np.random.default_rng(int(pf))
     m = (rng.standard_normal(777) * 3).astype(np.float32)
     k = (rng.standard_normal(777) * 3).astype(np.float32)
@@ -78,10 +79,12 @@ def test_dot_product_truncates_the_float_product(ops, pf):
     im, ik = (m * factor).astype(np.int64), (k * factor).astype(np.int64)   # float32 product, towards zero
     res, _, _, _ = ops.dot_product(torch.from_numpy(m), torch.from_numpy(k), pf)
     assert res == float(int(im @ ik)) / float(np.float32(np.float32(pf) * np.float32(pf)))
+    assert res == oracle.scalar_dot_product(m, k, pf)
     # the plain-integer baselines: same integers, int accumulator (32 bits), no division
     v, _, b1, b2, bits1, bits2 = ops.vector_dot_product(torch.from_numpy(m), torch.from_numpy(k), pf)
     want = (int(im @ ik) + (1 << 31)) % (1 << 32) - (1 << 31)
     assert v == want and (b1, b2, bits1, bits2) == (1024 * 8, 1024 * 8, 64, 64)
+    assert v == oracle.scalar_vector_dot_product(m, k, pf)
 
 
 def test_random_number_and_int16_variants(ops):
@@ -96,7 +99,7 @@ def test_random_number_and_int16_variants(ops):
     assert (b1, b2, bits1, bits2) == (600, 600, 16, 16)
 
 
-def test_batch_against_integer_matrix_product_and_capsules(ops, tmp_path):
+def test_batch_against_integer_matrix_product_and_capsules(ops, oracle, tmp_path):
     rng = np.random.default_rng(9)
     K = (rng.standard_normal((37, 300)) * 0.5).astype(np.float32)
     K[3] = np.abs(K[3])
@@ -106,6 +109,7 @@ def test_batch_against_integer_matrix_product_and_capsules(ops, tmp_path):
     want = (_round_half_away(K, dec) @ _round_half_away(q, dec)).astype(np.float64) / 10.0 ** (2 * dec)
     out, _, mem_q, mem_k0 = ops.batch_dot_product(torch.from_numpy(q), torch.from_numpy(K), dec)
     np.testing.assert_array_equal(out.numpy(), want)
+    np.testing.assert_array_equal(out.numpy(), oracle.scalar_batch_dot_product(q, K, dec))
     cap, total, R, d = ops.build_bsi_keys(torch.from_numpy(K), dec, 0.5)
     out2, _, _, _, mem_q2 = ops.batch_dot_product_prebuilt(torch.from_numpy(q), cap, 0.5)
     np.testing.assert_array_equal(out2.numpy(), want)
