@@ -162,7 +162,7 @@ def run(model_name="opt-1.3b", seq_len=512, batch=1, iters=5, warmup=2, decimal_
     if graph:
         with torch.no_grad():
             eager = model(input_ids).clone()
-            linear._last_query_build.clear()
+            linear.forget_shared_builds()
             static_in = input_ids.clone()
             side = torch.cuda.Stream()
             side.wait_stream(torch.cuda.current_stream())
@@ -171,11 +171,11 @@ def run(model_name="opt-1.3b", seq_len=512, batch=1, iters=5, warmup=2, decimal_
                     model(static_in)
             torch.cuda.current_stream().wait_stream(side)
             torch.cuda.synchronize()
-            linear._last_query_build.clear()
+            linear.forget_shared_builds()
             hip_graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(hip_graph):
                 static_out = model(static_in)
-            linear._last_query_build.clear()
+            linear.forget_shared_builds()
             same = True
             times = []
             for _ in range(max(iters, 3)):

@@ -943,6 +943,70 @@ def linear_few_rows_cuda(x2d: torch.Tensor, keyset_cuda_cap, decimal_places: int
     return out
 
 
+_last_linear_rebuilt = [False]  # whether the last linear_cuda call ran the query build (layer counters read it)
+_linear_ws: dict = {}  # device index -> {"bytes": size of one workspace, "buf": tensor of two, "eager": [...], "capture": [...]}
+
+
+def can_linear_one_call(x2d: torch.Tensor, keys: "PrebuiltBSIKeysCUDA") -> bool:
+    """Whether linear_cuda serves this call: chunk-scaled fixed-bit queries without clipping against fixed-bit keys,
+    the matrix-core route, no per-call profiling."""
+    f = _flags()
+    d = int(x2d.shape[1])
+    return (x2d.shape[0] > 0 and x2d.is_cuda and x2d.is_contiguous()
+            and x2d.dtype in (torch.float32, torch.float16, torch.bfloat16)
+            and keys.fixed and keys.d == d and 2 <= f["bits_q"] <= 8 and f["chunk_scale"] and f["clip_k"] == 0.0
+            and ((d + 63) // 64) % 4 == 0 and f["core"] != _lib.CORE_VALU and not f["profile"]
+            and os.environ.get("BSI_TC_DOT", "1").strip() != "0" and os.environ.get("BSI_LINEAR_ONE_CALL", "1").strip() != "0")
+
+
+def linear_cuda(x2d: torch.Tensor, keyset_cuda_cap, decimal_places: int, bias=None, warm_keys=None) -> torch.Tensor:
+    """out[Q, R] float32 of a BSI-linear layer in one library call (bsi_hip_linear): the query build into a workspace
+    kept per device, then the dot, bit for bit what build_bsi_queries_cuda_batch_packed followed by
+    batch_dot_product_multiquery_cuda_batch_caps returns.  A call on the very tensor the workspace was last built
+    from (same storage, shape, dtype and version: the next layer fed the same activations) skips the build.
+    Launches recorded into a HIP graph use a workspace of their own, so that replays and eager calls never find
+    each other's builds.  Not in the reference; it takes the operand handles and half of the binding work out of
+    an eager forward."""
+    keys = _capsule(keyset_cuda_cap, PrebuiltBSIKeysCUDA, "Invalid CUDA keys capsule")
+    _check(x2d.dim() == 2 and can_linear_one_call(x2d, keys), "linear_cuda: call not served by the one-call path")
+    _check(int(decimal_places) == keys.decimals,
+           f"Decimal mismatch between queries and keys: q={int(decimal_places)} k={keys.decimals}")
+    f = _flags()
+    Q, d, R = int(x2d.shape[0]), int(x2d.shape[1]), keys.num_keys
+    bits = f["bits_q"]
+    need = int(lib.bsi_hip_linear_workspace_bytes(Q, d, bits))
+    capturing = _capturing()
+    idx = x2d.device.index
+    ws = _linear_ws.get(idx)
+    if ws is None or ws["bytes"] < need:
+        _check(not capturing, "linear_cuda: the workspace must exist before a graph is captured (run the forward once)")
+        size = (max(need, 1 << 20) + 255) // 256 * 256
+        ws = _linear_ws[idx] = {"bytes": size, "buf": torch.empty((2 * size,), dtype=torch.uint8, device=x2d.device),
+                                "eager": [None, None], "capture": [None, None]}
+    slot = ws["capture" if capturing else "eager"]
+    key = (x2d.data_ptr(), Q, d, x2d.dtype, x2d._version, bits, int(decimal_places))
+    rebuild = 0 if slot[0] == key else 1
+    slot[0], slot[1] = key, x2d  # holds the input, so that its address is not reused while the build stands for it
+    wsptr = ws["buf"].data_ptr() + (ws["bytes"] if capturing else 0)
+    out = torch.empty((Q, R), dtype=torch.float32, device=x2d.device)
+    core = f["core"]
+    kptr, klayout = key_operand(keys, Q, bits, core)
+    wptr, wbytes = _warm_region(_capsule(warm_keys, PrebuiltBSIKeysCUDA, "Invalid CUDA keys capsule") if warm_keys is not None
+                                else None, Q, bits, core)
+    check(lib.bsi_hip_linear(x2d.data_ptr(), _dtype_code(x2d), Q, d, int(decimal_places), bits, rebuild, wsptr, ws["bytes"],
+                             kptr, klayout, keys.slice_weights.data_ptr(), keys.Sb, R,
+                             _scale_inv(int(decimal_places), keys.decimals), R, _ptr(bias), out.data_ptr(), core, wptr,
+                             wbytes, _stream()), "bsi_hip_linear")
+    _last_linear_rebuilt[0] = bool(rebuild)
+    return out
+
+
+def linear_cuda_forget() -> None:
+    """Drop what linear_cuda remembers of its last build (and the input tensor it holds)."""
+    for ws in _linear_ws.values():
+        ws["eager"], ws["capture"] = [None, None], [None, None]
+
+
 def _dot_result(out, ns, Q, R):
     per_q = float(ns) / float(Q) if Q > 0 else 0.0
     per_s = float(ns) / (float(Q) * float(R)) if (Q > 0 and R > 0) else 0.0

@@ -2514,6 +2514,54 @@ static void launch_stream_fused_t(const T* x, int64_t d, double dec_scale, int s
 #undef BSI_FUSED_GO
 }
 
+// Workspace of bsi_hip_linear: the query operands of one build (planes, shifts, scales, int8 image), each 256-aligned.
+struct LinearWorkspace {
+    size_t words, shifts, scales, ints8, total;
+};
+static LinearWorkspace linear_workspace(int64_t Q, int64_t d, int fixed_bits) {
+    const size_t W = static_cast<size_t>((d + 63) / 64), chunks = static_cast<size_t>((d + 255) / 256);
+    auto up = [](size_t v) { return (v + 255) / 256 * 256; };
+    LinearWorkspace w;
+    w.words = 0;
+    w.shifts = up(static_cast<size_t>(Q) * fixed_bits * W * 8);
+    w.scales = w.shifts + up(static_cast<size_t>(Q) * chunks * 4);
+    w.ints8 = w.scales + up(static_cast<size_t>(Q) * chunks * 4);
+    w.total = w.ints8 + up(static_cast<size_t>(Q) * chunks * 256);
+    return w;
+}
+
+extern "C" size_t bsi_hip_linear_workspace_bytes(int64_t Q, int64_t d, int fixed_bits) {
+    if (Q <= 0 || d <= 0 || fixed_bits < 2 || fixed_bits > 8) return 0;
+    return linear_workspace(Q, d, fixed_bits).total;
+}
+
+extern "C" int bsi_hip_linear(const void* x, int dtype, int64_t Q, int64_t d, int decimal_places, int fixed_bits, int rebuild,
+                              void* workspace, size_t workspace_bytes, const uint64_t* B, int b_layout, const float* Bw,
+                              int Sb, int64_t R, float scale_inv, int64_t R_total, const float* bias, float* out, int core,
+                              const void* warm, size_t warm_bytes, void* stream) {
+    BSI_REQUIRE(Q >= 0 && R >= 0 && d >= 1, "bad shape");
+    BSI_REQUIRE(fixed_bits >= 2 && fixed_bits <= 8, "fixed_bits must be in [2, 8] (got %d)", fixed_bits);
+    const int W64 = static_cast<int>((d + 63) / 64);
+    if (W64 % 4 != 0)
+        return fail(BSI_ERR_UNSUPPORTED, "chunk scales need a multiple of 4 words per slice (d = %lld)", static_cast<long long>(d));
+    if (Q == 0 || R == 0) return BSI_OK;
+    const LinearWorkspace w = linear_workspace(Q, d, fixed_bits);
+    BSI_REQUIRE(workspace != nullptr && workspace_bytes >= w.total, "workspace of %zu bytes needed, %zu given", w.total,
+                workspace_bytes);
+    BSI_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0, "workspace must be 256-byte aligned");
+    unsigned char* ws = static_cast<unsigned char*>(workspace);
+    uint64_t* words = reinterpret_cast<uint64_t*>(ws + w.words);
+    int32_t* shifts = reinterpret_cast<int32_t*>(ws + w.shifts);
+    float* scales = reinterpret_cast<float*>(ws + w.scales);
+    int8_t* ints8 = reinterpret_cast<int8_t*>(ws + w.ints8);
+    if (rebuild) {
+        const int rc = bsi_hip_build_fixed(x, dtype, Q, d, decimal_places, fixed_bits, 1, 0.0f, words, shifts, scales, ints8, stream);
+        if (rc != BSI_OK) return rc;
+    }
+    return bsi_hip_dot_bias_warm(words, ints8, scales, W64 / 4, fixed_bits, W64, B, b_layout, Bw, Sb, R, Q, scale_inv, R_total,
+                                 bias, out, core, nullptr, 0, warm, warm_bytes, stream);
+}
+
 extern "C" int bsi_hip_linear_few_rows_upfront(int64_t Q, int64_t d, int64_t R) {
     if (Q < 1 || Q > kFusedMaxQ || d < 1 || R < 1) return 0;
     const FusedPlan p = fused_plan(Q, static_cast<int>((d + 255) / 256), R);

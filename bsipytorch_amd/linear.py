@@ -23,6 +23,14 @@ from . import bsi_ops
 _last_query_build: Dict[str, Any] = {}
 
 
+def forget_shared_builds() -> None:
+    """Drop every remembered query build (the shared build of sibling layers, the one-call path's workspaces).  Call it
+    before and after recording a forward into a HIP graph: what was built while recording has not run, and what
+    an earlier recording built is not part of a new graph."""
+    _last_query_build.clear()
+    bsi_ops.linear_cuda_forget()
+
+
 def _cached_query_build(batch_inputs: torch.Tensor, decimal_places: int, threshold: float, packed: bool):
     use_cache = os.getenv("BSI_QUERY_CACHE", "1") != "0"
     key = (batch_inputs.data_ptr(), tuple(batch_inputs.shape), batch_inputs.dtype, batch_inputs._version,
@@ -131,6 +139,9 @@ class BSIQuantizedLinear(nn.Module):
             scores = self._forward_few_rows(batch_inputs, original_dtype)
             if scores is not None:
                 return scores.view(*original_shape[:-1], -1) if len(original_shape) != 2 else scores
+        scores = self._forward_one_call(batch_inputs, original_dtype)
+        if scores is not None:
+            return scores.view(*original_shape[:-1], -1) if len(original_shape) != 2 else scores
         t0 = time.perf_counter_ns()
         use_packed = os.getenv("BSI_QUERY_PACKED", "1") != "0"
         qcap, reused = _cached_query_build(batch_inputs, self.decimalPlaces, float(self.query_compress_threshold),
@@ -180,6 +191,50 @@ class BSIQuantizedLinear(nn.Module):
             self._track_error(batch_inputs, scores)
         if len(original_shape) != 2:
             scores = scores.view(*original_shape[:-1], -1)
+        return scores
+
+    def _forward_one_call(self, batch_inputs, original_dtype):
+        """Query build and dot in one library call (bsi_ops.linear_cuda), or None when that path does not serve the
+        call: the same two launches as below with a fraction of the host work, which is what an eager forward of
+        many small layers is bound by.  Layers fed the same tensor share the build (the workspace remembers what it
+        was built from); fused q/k/v siblings share the whole call."""
+        c = self.__dict__
+        fused = c.get("_fused")
+        keys = fused[0].keys if fused is not None else self._bsi_keys_cuda
+        if (c.get("collect_stats") or os.getenv("BSI_QUERY_PACKED", "1") == "0" or os.getenv("BSI_QUERY_CACHE", "1") == "0"
+                or not bsi_ops.can_linear_one_call(batch_inputs, keys)):
+            return None
+        fp32 = original_dtype == torch.float32
+        if fused is not None:
+            group, start, stop = fused
+            key = (batch_inputs.data_ptr(), tuple(batch_inputs.shape), batch_inputs.dtype, batch_inputs._version)
+            last = group.__dict__.get("_last_call")
+            if last is not None and last[0] == key:
+                scores, bias_done = last[2][:, start:stop], last[3]
+                last[4] -= 1
+                if last[4] <= 0:
+                    group.__dict__["_last_call"] = None
+            else:
+                gb = group.bias if (fp32 and group.bias is not None) else None
+                all_scores = bsi_ops.linear_cuda(batch_inputs, keys, self.decimalPlaces, gb, _keys_to_warm(group.next_layer))
+                group.__dict__["_last_call"] = [key, batch_inputs, all_scores, gb is not None, len(group.members) - 1]
+                scores, bias_done = all_scores[:, start:stop], gb is not None
+                c["dot_calls"] += 1
+                c["build_calls"] += int(bsi_ops._last_linear_rebuilt[0])
+        else:
+            b = self.bias if (fp32 and self.bias is not None and self.bias.dtype == torch.float32
+                              and self.bias.is_cuda and self.bias.is_contiguous()) else None
+            scores = bsi_ops.linear_cuda(batch_inputs, keys, self.decimalPlaces, b, _keys_to_warm(c.get("_next_bsi_layer")))
+            bias_done = b is not None
+            c["dot_calls"] += 1
+            c["build_calls"] += int(bsi_ops._last_linear_rebuilt[0])
+        q_rows = int(batch_inputs.shape[0])
+        c["dot_query_vectors_total"] += q_rows
+        c["dot_output_elements_total"] += q_rows * int(self.out_features)
+        if scores.dtype != original_dtype:
+            scores = scores.to(dtype=original_dtype)
+        if self.bias is not None and not bias_done:
+            scores = scores + self.bias.to(device=scores.device, dtype=original_dtype)
         return scores
 
     def _forward_few_rows(self, batch_inputs, original_dtype):

@@ -243,6 +243,19 @@ int bsi_hip_linear_few_rows(const void* x_device, int dtype, int64_t Q, int64_t 
                             const uint64_t* B_tiled, const float* Bw, int Sb, int64_t R, float scale_inv, int64_t R_total,
                             const float* bias, float* out, void* stream);
 
+/* A BSI-linear layer in one call for any number of rows: bsi_hip_build_fixed (chunk scales, no clipping) into
+ * `workspace`, then bsi_hip_dot_bias_warm on what it built -- the two launches a layer forward makes
+ * (verify_accuracy_bsi.py:143-178: build_bsi_queries_cuda_batch_packed, then
+ * batch_dot_product_multiquery_cuda_batch_caps), with one trip through the host binding instead of two and no
+ * per-call operand allocations.  rebuild = 0 skips the build and reuses the workspace's contents (layers that
+ * read the same activations).  workspace: bsi_hip_linear_workspace_bytes(Q, d, fixed_bits) bytes, 256-aligned,
+ * owned by the caller; B / b_layout as for bsi_hip_dot (int8 image or planes); warm as for bsi_hip_dot_bias_warm. */
+size_t bsi_hip_linear_workspace_bytes(int64_t Q, int64_t d, int fixed_bits);
+int bsi_hip_linear(const void* x_device, int dtype, int64_t Q, int64_t d, int decimal_places, int fixed_bits, int rebuild,
+                   void* workspace, size_t workspace_bytes, const uint64_t* B, int b_layout, const float* Bw, int Sb,
+                   int64_t R, float scale_inv, int64_t R_total, const float* bias, float* out, int core, const void* warm,
+                   size_t warm_bytes, void* stream);
+
 /* 1 when bsi_hip_linear_few_rows, for this shape, issues the loads of the whole query build before its first key
  * loads (the case in which the launch costs the GPU no more than the dot alone), 0 when some of the build waits
  * behind the key traffic (then the one launch still saves host time, but build + dot is the faster pair on the

@@ -1609,6 +1609,71 @@ def test_linear_few_rows_half_inputs_and_limits(hip, oracle, dtype):
                                      None, out.data_ptr(), st()) != 0
 
 
+@pytest.mark.parametrize("Q,R,d,with_bias", [(64, 200, 1024, True), (130, 75, 2048, False), (7, 33, 512, True), (33, 4100, 256, True)])
+def test_linear_one_call_matches_build_plus_dot(hip, oracle, ops, Q, R, d, with_bias):
+    """bsi_hip_linear (through bsi_ops.linear_cuda) against the oracle's build + dot, with and without the shared
+    build (second call on the same tensor), with a changed input in between, and against the two-call path."""
+    x = _inputs(Q, d, seed=Q + R, kind="outliers")
+    k = (np.random.default_rng(R).standard_normal((R, d)) * 0.02).astype(np.float32)
+    qb, kb = oracle.build_queries(x, 2, 7), oracle.build_keys(k, 2, 6)
+    _, want = oracle.dot_fixed(qb["words"], qb["scales"], kb["words"], kb["scales"], oracle.scale_inv(2, 2), want_ints=False)
+    keys = ops.build_bsi_keys_cuda(torch.from_numpy(k), 2, 0.5)[0]
+    bias = torch.randn(R, device="cuda") if with_bias else None
+    expect = want if bias is None else want + bias.cpu().numpy()[None, :]
+    xd = torch.from_numpy(x).cuda()
+    ops.linear_cuda_forget()
+    out1 = ops.linear_cuda(xd, keys, 2, bias)
+    out2 = ops.linear_cuda(xd, keys, 2, bias)          # same tensor: the build is reused
+    assert np.array_equal(out1.cpu().numpy(), expect.astype(np.float32)) and torch.equal(out1, out2)
+    other = torch.from_numpy(_inputs(Q, d, seed=99)).cuda()
+    ops.linear_cuda(other, keys, 2, bias)              # overwrites the workspace
+    xd.mul_(1.0)                                       # same values, new version: rebuilt, same result
+    assert torch.equal(ops.linear_cuda(xd, keys, 2, bias), out1)
+    qcap = ops.build_bsi_queries_cuda_batch_packed(xd, 2, 0.5)
+    two = ops.batch_dot_product_multiquery_cuda_batch_caps(qcap, keys, bias)[0]
+    assert torch.equal(two, out1)
+
+
+def test_layer_forward_one_call_path_and_graph_replay(ops, monkeypatch):
+    """BSIQuantizedLinear takes the one-call path for ordinary batches: same bits as with BSI_LINEAR_ONE_CALL=0,
+    sibling layers share the build, and a captured forward replays correctly after eager work in between."""
+    from bsipytorch_amd import linear
+
+    torch.manual_seed(5)
+    layers = [torch.nn.Linear(512, 300).cuda(), torch.nn.Linear(512, 200, bias=False).cuda()]
+    model = torch.nn.ModuleList(layers)
+    linear.quantize_model_bsi(model, decimalPlaces=2, compress_threshold=0.5, verbose=False)
+    x = torch.randn(48, 512, device="cuda")
+    with torch.no_grad():
+        monkeypatch.setenv("BSI_LINEAR_ONE_CALL", "0")
+        ref = [m(x).clone() for m in model]
+        monkeypatch.setenv("BSI_LINEAR_ONE_CALL", "1")
+        ops.linear_cuda_forget()
+        got = [m(x).clone() for m in model]          # the second layer reuses the first one's build
+        assert all(torch.equal(a, b) for a, b in zip(ref, got))
+        static_x = x.clone()
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            [m(static_x) for m in model]
+        torch.cuda.current_stream().wait_stream(s)
+        torch.cuda.synchronize()
+        linear.forget_shared_builds()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            outs = [m(static_x) for m in model]
+        linear.forget_shared_builds()
+        for rep in range(3):
+            static_x.copy_(x * (rep + 1))
+            [m(torch.randn(20, 512, device="cuda")) for m in model]   # eager work in between overwrites the workspace
+            g.replay()
+            torch.cuda.synchronize()
+            monkeypatch.setenv("BSI_LINEAR_ONE_CALL", "0")
+            want = [m(x * (rep + 1)) for m in model]
+            monkeypatch.setenv("BSI_LINEAR_ONE_CALL", "1")
+            assert all(torch.equal(a, b) for a, b in zip(outs, want))
+
+
 def test_layer_forward_uses_the_fused_few_rows_kernel(ops, monkeypatch):
     """A decode-sized call through BSIQuantizedLinear (alone and as fused q/k/v siblings) gives the bits of the
     build + dot path, for fp32 and fp16 activations."""
