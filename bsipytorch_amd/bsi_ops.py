@@ -32,6 +32,22 @@ from ._lib import check, lib
 # --------------------------------------------------------------------------- flags
 
 
+_ENV_DATA = getattr(os.environ, "_data", None)   # CPython on POSIX: the bytes-keyed dict behind os.environ
+_ENV_KEYS: dict = {}
+
+
+def fast_getenv(name: str, default: str) -> str:
+    """os.environ.get for the per-call switches (read on every forward, as the reference reads its own): a plain dict
+    lookup instead of os.environ's encode/decode round trip, which costs a forward of 100 layers half a millisecond."""
+    if _ENV_DATA is None:
+        return os.environ.get(name, default)
+    key = _ENV_KEYS.get(name)
+    if key is None:
+        key = _ENV_KEYS[name] = os.fsencode(name)
+    v = _ENV_DATA.get(key)
+    return default if v is None else os.fsdecode(v)
+
+
 def _env_int(name: str, default: Optional[int]) -> Optional[int]:
     s = os.environ.get(name)
     if s is None:
@@ -808,7 +824,7 @@ def _dot(words, ints8, scales, scale_stride, Sa, W, keys: PrebuiltBSIKeysCUDA, Q
     core = f["core"] if core is None else core
     # the reference's A/B switch between its tensor-core and popcount kernels is read on every call
     # (bsi_cuda_kernels_dot.cuh:2642); 0 selects the popcount core here
-    if os.environ.get("BSI_TC_DOT", "1").strip() == "0" and words is not None:
+    if fast_getenv("BSI_TC_DOT", "1").strip() == "0" and words is not None:
         core = _lib.CORE_VALU
     ws = None
     ws_bytes = 0
@@ -917,7 +933,7 @@ def can_fuse_linear_few_rows(x2d: torch.Tensor, keys: "PrebuiltBSIKeysCUDA") -> 
             and keys.fixed and keys.Sb == 6 and keys.layout == _lib.LAYOUT_TILED16 and keys.d == d
             and 2 <= f["bits_q"] <= 8 and f["chunk_scale"] and f["clip_k"] == 0.0 and ((d + 63) // 64) % 4 == 0
             and ((d + 255) // 256) * int(x2d.shape[0]) * 260 <= FUSED_LINEAR_QUERY_LDS_BYTES and f["core"] != _lib.CORE_VALU and not f["profile"]
-            and os.environ.get("BSI_TC_DOT", "1").strip() != "0" and os.environ.get("BSI_FUSED_LINEAR", "1").strip() != "0")
+            and fast_getenv("BSI_TC_DOT", "1").strip() != "0" and fast_getenv("BSI_FUSED_LINEAR", "1").strip() != "0")
 
 
 def linear_few_rows_is_free(x2d: torch.Tensor, keys: "PrebuiltBSIKeysCUDA") -> bool:
@@ -956,10 +972,11 @@ def can_linear_one_call(x2d: torch.Tensor, keys: "PrebuiltBSIKeysCUDA") -> bool:
             and x2d.dtype in (torch.float32, torch.float16, torch.bfloat16)
             and keys.fixed and keys.d == d and 2 <= f["bits_q"] <= 8 and f["chunk_scale"] and f["clip_k"] == 0.0
             and ((d + 63) // 64) % 4 == 0 and f["core"] != _lib.CORE_VALU and not f["profile"]
-            and os.environ.get("BSI_TC_DOT", "1").strip() != "0" and os.environ.get("BSI_LINEAR_ONE_CALL", "1").strip() != "0")
+            and fast_getenv("BSI_TC_DOT", "1").strip() != "0" and fast_getenv("BSI_LINEAR_ONE_CALL", "1").strip() != "0")
 
 
-def linear_cuda(x2d: torch.Tensor, keyset_cuda_cap, decimal_places: int, bias=None, warm_keys=None) -> torch.Tensor:
+def linear_cuda(x2d: torch.Tensor, keyset_cuda_cap, decimal_places: int, bias=None, warm_keys=None,
+                _checked: bool = False) -> torch.Tensor:
     """out[Q, R] float32 of a BSI-linear layer in one library call (bsi_hip_linear): the query build into a workspace
     kept per device, then the dot, bit for bit what build_bsi_queries_cuda_batch_packed followed by
     batch_dot_product_multiquery_cuda_batch_caps returns.  A call on the very tensor the workspace was last built
@@ -968,7 +985,8 @@ def linear_cuda(x2d: torch.Tensor, keyset_cuda_cap, decimal_places: int, bias=No
     each other's builds.  Not in the reference; it takes the operand handles and half of the binding work out of
     an eager forward."""
     keys = _capsule(keyset_cuda_cap, PrebuiltBSIKeysCUDA, "Invalid CUDA keys capsule")
-    _check(x2d.dim() == 2 and can_linear_one_call(x2d, keys), "linear_cuda: call not served by the one-call path")
+    if not _checked:  # the layer has asked can_linear_one_call already
+        _check(x2d.dim() == 2 and can_linear_one_call(x2d, keys), "linear_cuda: call not served by the one-call path")
     _check(int(decimal_places) == keys.decimals,
            f"Decimal mismatch between queries and keys: q={int(decimal_places)} k={keys.decimals}")
     f = _flags()

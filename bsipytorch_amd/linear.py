@@ -32,7 +32,7 @@ def forget_shared_builds() -> None:
 
 
 def _cached_query_build(batch_inputs: torch.Tensor, decimal_places: int, threshold: float, packed: bool):
-    use_cache = os.getenv("BSI_QUERY_CACHE", "1") != "0"
+    use_cache = bsi_ops.fast_getenv("BSI_QUERY_CACHE", "1") != "0"
     key = (batch_inputs.data_ptr(), tuple(batch_inputs.shape), batch_inputs.dtype, batch_inputs._version,
            int(decimal_places), bool(packed))
     if use_cache and _last_query_build.get("key") == key and _last_query_build.get("src") is not None:
@@ -128,7 +128,7 @@ class BSIQuantizedLinear(nn.Module):
         original_shape = x.shape
         if x.dim() != 2:
             x = x.reshape(-1, x.shape[-1])
-        if os.getenv("BSI_QUERY_FP32", "0") != "0":
+        if bsi_ops.fast_getenv("BSI_QUERY_FP32", "0") != "0":
             x = x.to(torch.float32)
         batch_inputs = x.detach().contiguous()
         q_rows = int(batch_inputs.shape[0])
@@ -143,7 +143,7 @@ class BSIQuantizedLinear(nn.Module):
         if scores is not None:
             return scores.view(*original_shape[:-1], -1) if len(original_shape) != 2 else scores
         t0 = time.perf_counter_ns()
-        use_packed = os.getenv("BSI_QUERY_PACKED", "1") != "0"
+        use_packed = bsi_ops.fast_getenv("BSI_QUERY_PACKED", "1") != "0"
         qcap, reused = _cached_query_build(batch_inputs, self.decimalPlaces, float(self.query_compress_threshold),
                                            use_packed)
         c["build_ns_total"] += time.perf_counter_ns() - t0
@@ -201,7 +201,7 @@ class BSIQuantizedLinear(nn.Module):
         c = self.__dict__
         fused = c.get("_fused")
         keys = fused[0].keys if fused is not None else self._bsi_keys_cuda
-        if (c.get("collect_stats") or os.getenv("BSI_QUERY_PACKED", "1") == "0" or os.getenv("BSI_QUERY_CACHE", "1") == "0"
+        if (c.get("collect_stats") or bsi_ops.fast_getenv("BSI_QUERY_PACKED", "1") == "0" or bsi_ops.fast_getenv("BSI_QUERY_CACHE", "1") == "0"
                 or not bsi_ops.can_linear_one_call(batch_inputs, keys)):
             return None
         fp32 = original_dtype == torch.float32
@@ -216,7 +216,7 @@ class BSIQuantizedLinear(nn.Module):
                     group.__dict__["_last_call"] = None
             else:
                 gb = group.bias if (fp32 and group.bias is not None) else None
-                all_scores = bsi_ops.linear_cuda(batch_inputs, keys, self.decimalPlaces, gb, _keys_to_warm(group.next_layer))
+                all_scores = bsi_ops.linear_cuda(batch_inputs, keys, self.decimalPlaces, gb, _keys_to_warm(group.next_layer), True)
                 group.__dict__["_last_call"] = [key, batch_inputs, all_scores, gb is not None, len(group.members) - 1]
                 scores, bias_done = all_scores[:, start:stop], gb is not None
                 c["dot_calls"] += 1
@@ -224,7 +224,7 @@ class BSIQuantizedLinear(nn.Module):
         else:
             b = self.bias if (fp32 and self.bias is not None and self.bias.dtype == torch.float32
                               and self.bias.is_cuda and self.bias.is_contiguous()) else None
-            scores = bsi_ops.linear_cuda(batch_inputs, keys, self.decimalPlaces, b, _keys_to_warm(c.get("_next_bsi_layer")))
+            scores = bsi_ops.linear_cuda(batch_inputs, keys, self.decimalPlaces, b, _keys_to_warm(c.get("_next_bsi_layer")), True)
             bias_done = b is not None
             c["dot_calls"] += 1
             c["build_calls"] += int(bsi_ops._last_linear_rebuilt[0])
@@ -250,7 +250,7 @@ class BSIQuantizedLinear(nn.Module):
         # its share of the activations before its key planes; past that (more rows, longer rows) it repeats too much
         # arithmetic, so a forward that is being captured into a graph, where host time does not count, then keeps
         # the two launches.  BSI_FUSED_LINEAR=2 forces the fused kernel in both cases.
-        if (torch.cuda.is_current_stream_capturing() and os.getenv("BSI_FUSED_LINEAR", "1") != "2"
+        if (torch.cuda.is_current_stream_capturing() and bsi_ops.fast_getenv("BSI_FUSED_LINEAR", "1") != "2"
                 and not bsi_ops.linear_few_rows_is_free(batch_inputs, keys)):
             return None
         fp32 = original_dtype == torch.float32
