@@ -375,6 +375,7 @@ def _digit_images(words: torch.Tensor) -> Optional[torch.Tensor]:
 
 
 _expanded_cache: dict = {}
+_warmed_query_caches: set = set()
 
 
 def _expanded_slice_weights(base: torch.Tensor, Q: int, bits: int, dev) -> torch.Tensor:
@@ -385,6 +386,7 @@ def _expanded_slice_weights(base: torch.Tensor, Q: int, bits: int, dev) -> torch
     if t is None:
         if len(_expanded_cache) > 64:
             _expanded_cache.clear()
+            _warmed_query_caches.clear()
         t = base.unsqueeze(0).expand(Q, -1).contiguous()
         if _capturing():
             return t  # filled when the graph runs: not for the cache
@@ -397,10 +399,14 @@ def warm_query_build_caches(Q: int) -> None:
     so that a build recorded into a HIP graph later finds them.  A forward that skips the builder when run eagerly
     (the fused few-rows kernel) calls this for the graph capture that does not skip it."""
     f = _flags()
-    if f["bits_q"] == 0 or _capturing():
+    if f["bits_q"] == 0:
+        return
+    done = (int(Q), f["bits_q"], torch.cuda.current_device())
+    if done in _warmed_query_caches or _capturing():
         return
     dev = _device()
     _expanded_slice_weights(_slice_weights(f["bits_q"], 0, True, dev), int(Q), f["bits_q"], dev)
+    _warmed_query_caches.add(done)
 
 
 def _build_query_batch(q2d: torch.Tensor, decimal_places: int) -> PrebuiltBSIQueryBatchCUDA:
@@ -942,12 +948,13 @@ def linear_few_rows_is_free(x2d: torch.Tensor, keys: "PrebuiltBSIKeysCUDA") -> b
     return bool(lib.bsi_hip_linear_few_rows_upfront(int(x2d.shape[0]), int(x2d.shape[1]), int(keys.num_keys)))
 
 
-def linear_few_rows_cuda(x2d: torch.Tensor, keyset_cuda_cap, decimal_places: int, bias=None) -> torch.Tensor:
+def linear_few_rows_cuda(x2d: torch.Tensor, keyset_cuda_cap, decimal_places: int, bias=None, _checked: bool = False) -> torch.Tensor:
     """out[Q, R] float32 = BSI dot of the rows of ``x2d`` (Q <= 4) with the keyset, query build included, in one
     launch (bsi_hip_linear_few_rows): what build_bsi_queries_cuda_batch_packed followed by
     batch_dot_product_multiquery_cuda_batch_caps returns, bit for bit.  Not in the reference."""
     keys = _capsule(keyset_cuda_cap, PrebuiltBSIKeysCUDA, "Invalid CUDA keys capsule")
-    _check(x2d.dim() == 2 and can_fuse_linear_few_rows(x2d, keys), "linear_few_rows_cuda: call not served by the fused kernel")
+    if not _checked:  # the layer has asked can_fuse_linear_few_rows already
+        _check(x2d.dim() == 2 and can_fuse_linear_few_rows(x2d, keys), "linear_few_rows_cuda: call not served by the fused kernel")
     _check(int(decimal_places) == keys.decimals,
            f"Decimal mismatch between queries and keys: q={int(decimal_places)} k={keys.decimals}")
     Q, R = int(x2d.shape[0]), keys.num_keys

@@ -266,14 +266,14 @@ class BSIQuantizedLinear(nn.Module):
                     group.__dict__["_last_few"] = None
             else:
                 gb = group.bias if (fp32 and group.bias is not None) else None
-                all_scores = bsi_ops.linear_few_rows_cuda(batch_inputs, keys, self.decimalPlaces, gb)
+                all_scores = bsi_ops.linear_few_rows_cuda(batch_inputs, keys, self.decimalPlaces, gb, True)
                 # holds the input's storage (so that its address is not reused) until every member has been served
                 group.__dict__["_last_few"] = [key, batch_inputs, all_scores, gb is not None, len(group.members) - 1]
                 scores, bias_done = all_scores[:, start:stop], gb is not None
                 c["dot_calls"] += 1
         else:
             b = self.bias if (fp32 and self.bias is not None and self.bias.dtype == torch.float32) else None
-            scores, bias_done = bsi_ops.linear_few_rows_cuda(batch_inputs, keys, self.decimalPlaces, b), b is not None
+            scores, bias_done = bsi_ops.linear_few_rows_cuda(batch_inputs, keys, self.decimalPlaces, b, True), b is not None
             c["dot_calls"] += 1
         q_rows = int(batch_inputs.shape[0])
         c["dot_query_vectors_total"] += q_rows
