@@ -781,7 +781,8 @@ struct I8Cfg {
     static constexpr int kOperandK = TM * 128;         // bytes of the key tile of one half-chunk
     static constexpr int kStage = (TM + TN) * 128;     // keys then queries
     static constexpr int kScaleBytes = 4 * kLoaders * 256;  // chunk scales: ring of 4 chunks x loader regions x 64 floats
-    static constexpr int kLds = 4 * kStage + kScaleBytes;
+    static constexpr int kEpilogueBytes = 2 * TM * 4;  // the tile's key factors, then its biases (chain modes)
+    static constexpr int kLds = 4 * kStage + kScaleBytes + kEpilogueBytes;
 };
 
 // One k-step (64 of a chunk's 256 elements) of an MFMA wave: WM WN MFMAs on the operands in (ka, qb), one
@@ -872,6 +873,24 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
                                       static_cast<size_t>(Q - q0) * rowbytes +
                                           (kSum ? static_cast<size_t>(ndig - 1) * static_cast<size_t>(dig_stride) : 0));
         const bsi_rsrc rs = make_rsrc(qscale + q0 * qscale_stride, static_cast<size_t>(Q - q0) * qscale_stride * 4);
+        if (!kSum) {
+            // The epilogue's operands, staged once per workgroup: the slice-0 weight (key factor) and the bias of the
+            // tile's TM keys, 64 rows per load.  Fetched per lane at the end they are 32 vector-memory instructions
+            // for every MFMA wave, half as many as the whole chunk loop issues, all queued in front of the stores.
+            // Issued first, they have landed before any stage has (loads return in order).  Rows past R, and the
+            // biases of a call without one, read nothing and give 0 (buffer bounds).
+            const bsi_rsrc wrs = make_rsrc(Bw + static_cast<size_t>(r0) * Sb, static_cast<size_t>(R - r0) * Sb * sizeof(float));
+            const bsi_rsrc brs = make_rsrc(bias != nullptr ? bias + r0 : Bw,
+                                           bias != nullptr ? static_cast<size_t>(R - r0) * sizeof(float) : 0);
+            unsigned char* const epi = lds + 4 * C::kStage + C::kScaleBytes;
+            for (int j = lw; j < 2 * (TM / 64); j += C::kLoaders) {
+                const bool is_bias = j >= TM / 64;
+                const int blk = is_bias ? j - TM / 64 : j;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(is_bias ? brs : wrs,
+                                                         BSI_LDS_PTR(epi + (is_bias ? TM * 4 : 0) + blk * 256), 4,
+                                                         (blk * 64 + lane) * (is_bias ? 4 : Sb * 4), 0, 0, 0);
+            }
+        }
         // the stage has kGroups groups of 8 rows, keys first; loader lw moves groups lw, lw + kLoaders, ... (when
         // the groups do not divide evenly the last load wraps around and fetches a group a second time, so that
         // every loader wave has the same number of loads in flight)
@@ -937,10 +956,19 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NI + (kSum ? 0 : 1)) : "memory");
         lds_barrier();
         for (int h = 0; h < halves; ++h) {
-            issue(h + 3);  // its slot was released by the barrier that ended half h - 1
-            // stage h + 1 (and the scales issued right behind it) landed; stages h + 2, h + 3 and one
-            // scale load, 2 NI + 1 instructions, may still be in flight
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NI + (kSum ? 0 : 1)) : "memory");
+            if (h + 3 < halves) {
+                issue(h + 3);  // its slot was released by the barrier that ended half h - 1
+                // stage h + 1 (and the scales issued right behind it) landed; stages h + 2, h + 3 and one
+                // scale load, 2 NI + 1 instructions, may still be in flight
+                asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NI + (kSum ? 0 : 1)) : "memory");
+            } else if (h + 3 == halves) {
+                // nothing left to issue (a copy of the last stage here, as the prologue does for a single chunk, would
+                // queue 96 KiB of loads in front of every workgroup's output stores); the last stage and its
+                // scales may be in flight
+                asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NI + (kSum ? 0 : 1)) : "memory");
+            } else {
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            }
             lds_barrier();
         }
         if (warm_lines > 0) {
@@ -1176,21 +1204,18 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
                 if (kInts && int_off[a][b] >= 0 && e < int_rows[a])
                     chunk_ints[int_off[a][b] + static_cast<int64_t>(e) * chunks + (chunks - 1)] = v >> down_shift;
             }
-    // The key scales and biases of all the wave's rows in one go (the chunk accumulators are dead by now, so the
-    // registers are there): one cache round trip before the stores instead of one per 16-key tile.  Buffer loads:
-    // rows past R, and every bias of a call without one, read nothing and give 0.
+    // The key factors and biases of the wave's rows, from the copy the loader waves staged in LDS when the workgroup
+    // started (0 for rows past R and for a call without bias): two 16-byte reads per 16-key tile.
     float bs[WM][4], bi[WM][4];
     {
-        const bsi_rsrc wrs = make_rsrc(Bw, static_cast<size_t>(R) * Sb * sizeof(float));
-        const bsi_rsrc brs = make_rsrc(bias != nullptr ? bias : Bw, bias != nullptr ? static_cast<size_t>(R) * sizeof(float) : 0);
+        const float* epi = reinterpret_cast<const float*>(lds + 4 * C::kStage + C::kScaleBytes);
 #pragma unroll
         for (int a = 0; a < WM; ++a) {
-            const int rb = static_cast<int>(r0 + wr * (WM * 16) + a * 16 + lg * 4);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                bs[a][e] = __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(wrs, (rb + e) * Sb * 4, 0, 0));
-                bi[a][e] = __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(brs, (rb + e) * 4, 0, 0));
-            }
+            const int rl = wr * (WM * 16) + a * 16 + lg * 4;  // row of the tile
+            const float4 w4 = *reinterpret_cast<const float4*>(epi + rl);
+            const float4 b4 = *reinterpret_cast<const float4*>(epi + TM + rl);
+            bs[a][0] = w4.x, bs[a][1] = w4.y, bs[a][2] = w4.z, bs[a][3] = w4.w;
+            bi[a][0] = b4.x, bi[a][1] = b4.y, bi[a][2] = b4.z, bi[a][3] = b4.w;
         }
     }
 #pragma unroll
