@@ -23,7 +23,7 @@ MFMA_I8_PEAK_TOPS = 5000.0     # MI355X published dense int8
 Q, R, D = 512, 8192, 2048
 # HBM bytes per launch of the dot kernel on this workload, from rocprofv3 FETCH_SIZE and WRITE_SIZE runs scaled by a
 # 256 MiB copy (profiles/dot_mfma_i8_kernel_fc1_Q512_R8192_D2048_hbm_traffic.txt); counters cannot be read in-process
-MEASURED_TRAFFIC_BYTES = {"mfma": 42445000}
+MEASURED_TRAFFIC_BYTES = {"mfma": 42466000}
 SA, SB = 7, 6
 
 
