@@ -982,6 +982,32 @@ def can_linear_one_call(x2d: torch.Tensor, keys: "PrebuiltBSIKeysCUDA") -> bool:
             and fast_getenv("BSI_TC_DOT", "1").strip() != "0" and fast_getenv("BSI_LINEAR_ONE_CALL", "1").strip() != "0")
 
 
+def _linear_workspace(device, need: int, capturing: bool) -> dict:
+    """linear_cuda's workspace record of ``device``, (re)allocated when it is missing or smaller than ``need`` bytes."""
+    ws = _linear_ws.get(device.index)
+    if ws is None or ws["bytes"] < need:
+        _check(not capturing, "linear_cuda: the workspace must exist before a graph is captured (run the forward once)")
+        size = (max(need, 1 << 20) + 255) // 256 * 256
+        ws = _linear_ws[device.index] = {"bytes": size, "buf": torch.empty((2 * size,), dtype=torch.uint8, device=device),
+                                         "eager": [None, None], "capture": [None, None]}
+    return ws
+
+
+_reserved_linear_shapes: set = set()
+
+
+def reserve_linear_workspace(x2d: torch.Tensor) -> None:
+    """Make sure linear_cuda's workspace can take inputs of this shape.  A forward that runs eagerly on the few-rows
+    kernel never calls linear_cuda, yet the same forward recorded into a graph may (build + dot is the faster pair
+    there for longer rows), and a capture cannot allocate: the eager few-rows path calls this instead."""
+    bits = _flags()["bits_q"]
+    key = (x2d.device.index, int(x2d.shape[0]), int(x2d.shape[1]), bits)
+    if key in _reserved_linear_shapes or not (2 <= bits <= 8) or _capturing():
+        return
+    _linear_workspace(x2d.device, int(lib.bsi_hip_linear_workspace_bytes(key[1], key[2], bits)), False)
+    _reserved_linear_shapes.add(key)
+
+
 def linear_cuda(x2d: torch.Tensor, keyset_cuda_cap, decimal_places: int, bias=None, warm_keys=None,
                 _checked: bool = False) -> torch.Tensor:
     """out[Q, R] float32 of a BSI-linear layer in one library call (bsi_hip_linear): the query build into a workspace
@@ -1001,13 +1027,7 @@ def linear_cuda(x2d: torch.Tensor, keyset_cuda_cap, decimal_places: int, bias=No
     bits = f["bits_q"]
     need = int(lib.bsi_hip_linear_workspace_bytes(Q, d, bits))
     capturing = _capturing()
-    idx = x2d.device.index
-    ws = _linear_ws.get(idx)
-    if ws is None or ws["bytes"] < need:
-        _check(not capturing, "linear_cuda: the workspace must exist before a graph is captured (run the forward once)")
-        size = (max(need, 1 << 20) + 255) // 256 * 256
-        ws = _linear_ws[idx] = {"bytes": size, "buf": torch.empty((2 * size,), dtype=torch.uint8, device=x2d.device),
-                                "eager": [None, None], "capture": [None, None]}
+    ws = _linear_workspace(x2d.device, need, capturing)
     slot = ws["capture" if capturing else "eager"]
     key = (x2d.data_ptr(), Q, d, x2d.dtype, x2d._version, bits, int(decimal_places))
     rebuild = 0 if slot[0] == key else 1

@@ -255,6 +255,7 @@ class BSIQuantizedLinear(nn.Module):
             return None
         fp32 = original_dtype == torch.float32
         bsi_ops.warm_query_build_caches(int(batch_inputs.shape[0]))
+        bsi_ops.reserve_linear_workspace(batch_inputs)  # a later capture of this forward may take the one-call path
         if fused is not None:
             group, start, stop = fused
             key = (batch_inputs.data_ptr(), tuple(batch_inputs.shape), batch_inputs.dtype, batch_inputs._version)

@@ -1674,6 +1674,43 @@ def test_layer_forward_one_call_path_and_graph_replay(ops, monkeypatch):
             assert all(torch.equal(a, b) for a, b in zip(outs, want))
 
 
+def test_few_rows_forward_captured_after_eager_runs(ops):
+    """Four rows of long activations: the eager forward runs on the fused few-rows kernel, the same forward recorded
+    into a graph on build + dot (the fused kernel is not free there), whose workspace must exist by then.  Replays
+    give the eager bits."""
+    from bsipytorch_amd import linear
+
+    torch.manual_seed(12)
+    model = torch.nn.ModuleList([torch.nn.Linear(16384, 256).cuda()])
+    linear.quantize_model_bsi(model, decimalPlaces=2, compress_threshold=0.5, verbose=False)
+    layer = model[0]
+    x = torch.randn(4, 16384, device="cuda")
+    assert not ops.linear_few_rows_is_free(x, layer._bsi_keys_cuda)
+    ops._linear_ws.clear()
+    ops._reserved_linear_shapes.clear()
+    with torch.no_grad():
+        want = layer(x).clone()
+        static_x = x.clone()
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            layer(static_x)
+        torch.cuda.current_stream().wait_stream(s)
+        torch.cuda.synchronize()
+        linear.forget_shared_builds()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            out = layer(static_x)
+        linear.forget_shared_builds()
+        for rep in range(3):
+            static_x.copy_(x * (rep + 1))
+            layer(torch.randn(4, 16384, device="cuda"))  # eager work in between
+            g.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, layer(x * (rep + 1)))
+        assert torch.equal(want, layer(x))
+
+
 def test_layer_forward_uses_the_fused_few_rows_kernel(ops, monkeypatch):
     """A decode-sized call through BSIQuantizedLinear (alone and as fused q/k/v siblings) gives the bits of the
     build + dot path, for fp32 and fp16 activations."""
