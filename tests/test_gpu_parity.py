@@ -567,6 +567,40 @@ def test_dot_row_stride_int8_image_and_few_rows(hip, oracle):
     assert np.isnan(out[:, 150:]).all()
 
 
+@pytest.mark.parametrize("tile", ["int8-128", "int8-12864", "int8-64", "int8-6432"])
+@pytest.mark.parametrize("d", [256, 512, 768, 1280, 1792])
+def test_dot_int8_image_short_and_odd_chunk_counts(hip, oracle, d, tile):
+    """1, 2, 3, 5 and 7 chunks through every tile of the int8-image kernel: the loader's prologue (three stages ahead of
+    a loop that may have fewer) and its tail (no loads behind the last stage) meet the MFMA waves' barriers one for one;
+    outputs and per-chunk integers bit-identical to the oracle, with and without bias."""
+    Q, R, W = 70, 150, d // 64
+    chunks = d // 256
+    x, k, qb, kb, want_ints, want_out = _oracle_case(oracle, Q, R, d, seed=d)
+    bias = np.random.default_rng(d).standard_normal(R).astype(np.float32)
+    L = hip.lib
+    A, scales, Bc, Bw = dev(qb["words"]), dev(qb["scales"]), dev(kb["words"]), dev(kb["slice_weights"])
+    a8 = torch.zeros((Q, chunks * 256), dtype=torch.int8, device="cuda")
+    hip.check(L.bsi_hip_planes_to_int8(A.data_ptr(), Q, 7, W, a8.data_ptr(), st()), "p2i8")
+    B = torch.zeros((R, chunks * 256), dtype=torch.int8, device="cuda")
+    hip.check(L.bsi_hip_planes_to_int8(Bc.data_ptr(), R, 6, W, B.data_ptr(), st()), "image")
+    hip.check(L.bsi_hip_set_option(hip.OPT_I8_TILE, _I8_TILES[tile]), "opt")
+    try:
+        out = torch.full((Q, R), float("nan"), dtype=torch.float32, device="cuda")
+        ints = torch.full((Q, R, chunks), -7, dtype=torch.int32, device="cuda")
+        hip.check(L.bsi_hip_dot(A.data_ptr(), a8.data_ptr(), scales.data_ptr(), chunks, 7, W, B.data_ptr(), 2, Bw.data_ptr(),
+                                6, R, Q, float(np.float32(1e-4)), R, out.data_ptr(), ints.data_ptr(), 2, None, 0, st()), "dot")
+        outb = torch.full((Q, R), float("nan"), dtype=torch.float32, device="cuda")
+        hip.check(L.bsi_hip_dot_bias(A.data_ptr(), a8.data_ptr(), scales.data_ptr(), chunks, 7, W, B.data_ptr(), 2,
+                                     Bw.data_ptr(), 6, R, Q, float(np.float32(1e-4)), R, dev(bias).data_ptr(),
+                                     outb.data_ptr(), 2, None, 0, st()), "dot_bias")
+        torch.cuda.synchronize()
+    finally:
+        hip.check(L.bsi_hip_set_option(hip.OPT_I8_TILE, 0), "opt")
+    np.testing.assert_array_equal(ints.cpu().numpy(), want_ints)
+    np.testing.assert_array_equal(out.cpu().numpy(), want_out)
+    np.testing.assert_array_equal(outb.cpu().numpy(), want_out + bias[None, :])
+
+
 @pytest.mark.parametrize("Q,tiled", [(70, "int8-128"), (70, "int8-12864"), (70, "int8-64"), (70, "int8-6432"), (9, True), (70, True), (70, False)])
 def test_dot_bias_entry_point(hip, oracle, Q, tiled):
     """bsi_hip_dot_bias == bsi_hip_dot followed by a float addition of the bias row, bit for bit, whether the
