@@ -568,11 +568,11 @@ def test_dot_row_stride_int8_image_and_few_rows(hip, oracle):
 
 
 @pytest.mark.parametrize("tile", ["int8-128", "int8-12864", "int8-64", "int8-6432"])
-@pytest.mark.parametrize("d", [256, 512, 768, 1280, 1792])
+@pytest.mark.parametrize("d", [256, 512, 768, 1280, 1792, 2304, 4352])
 def test_dot_int8_image_short_and_odd_chunk_counts(hip, oracle, d, tile):
-    """1, 2, 3, 5 and 7 chunks through every tile of the int8-image kernel: the loader's prologue (three stages ahead of
-    a loop that may have fewer) and its tail (no loads behind the last stage) meet the MFMA waves' barriers one for one;
-    outputs and per-chunk integers bit-identical to the oracle, with and without bias."""
+    """1, 2, 3, 5, 7, 9 and 17 chunks through every tile of the int8-image kernel: the loader's prologue (three stages
+    ahead of a loop that may have fewer) and its tail (no loads behind the last stage) meet the MFMA waves' barriers
+    one for one; outputs and per-chunk integers bit-identical to the oracle, with and without bias."""
     Q, R, W = 70, 150, d // 64
     chunks = d // 256
     x, k, qb, kb, want_ints, want_out = _oracle_case(oracle, Q, R, d, seed=d)
