@@ -223,6 +223,16 @@ class PrebuiltBSIQueryCUDA(_Capsule):
         self.comp_len: Optional[torch.Tensor] = None
 
 
+def tensor_build_key(t: torch.Tensor, *extra):
+    """What identifies the query build of ``t``: its storage address, shape, dtype, version counter and the flags the
+    build depends on -- or None when the contents cannot be tracked (a tensor made under ``torch.inference_mode()``
+    keeps no version counter), in which case nothing is shared and every call builds anew."""
+    if t.is_inference():
+        return None
+    f = _flags()
+    return (t.data_ptr(), tuple(t.shape), t.dtype, t._version, f["bits_q"], f["chunk_scale"], f["clip_k"]) + extra
+
+
 def _capsule(obj, cls, what: str):
     _check(isinstance(obj, cls), what)
     return obj
@@ -788,14 +798,25 @@ _workspace: dict = {}
 _FEW_ROWS_MAX_Q = 32  # up to here the dot streams the packed planes (bandwidth-bound); above, the int8 image
 
 
+_retired_workspaces: list = []  # buffers whose address a recorded graph holds: never freed, never reused
+
+
 def _get_workspace(nbytes: int, dev) -> Optional[torch.Tensor]:
+    """Scratch memory for one dot on ``dev`` (derived int8 queries, digit products).  A launch recorded into a HIP
+    graph has the buffer's address baked in, so a buffer that a capture has used is never given back to the
+    allocator: when a later call needs more, a new one is added and the old one is kept alive for the replays."""
     if nbytes <= 0:
         return None
-    ws = _workspace.get(dev)
-    if ws is None or ws.numel() < nbytes:
-        ws = torch.empty((nbytes,), dtype=torch.uint8, device=dev)
-        _workspace[dev] = ws
-    return ws
+    rec = _workspace.get(dev)
+    capturing = _capturing()
+    if rec is None or rec["buf"].numel() < nbytes:
+        _check(not capturing, "bsi_ops: this dot needs a larger workspace than exists; run it once before capturing a graph")
+        if rec is not None and rec["captured"]:
+            _retired_workspaces.append(rec["buf"])
+        rec = _workspace[dev] = {"buf": torch.empty((nbytes,), dtype=torch.uint8, device=dev), "captured": False}
+    if capturing:
+        rec["captured"] = True
+    return rec["buf"]
 
 
 def _scale_inv(dec_q: int, dec_k: int) -> float:
@@ -860,7 +881,7 @@ def _dot(words, ints8, scales, scale_stride, Sa, W, keys: PrebuiltBSIKeysCUDA, Q
                               _scale_inv(decimals_q, keys.decimals), R, out.data_ptr(), _ptr(chunk_ints), core,
                               _ptr(ws), ws_bytes, _stream()), "bsi_hip_dot")
         if bias is not None:
-            out += bias
+            check(lib.bsi_hip_add_bias(out.data_ptr(), bias.data_ptr(), Q, R, R, _stream()), "bsi_hip_add_bias")
     ns = 0
     if prof:
         e1.record()
@@ -912,7 +933,7 @@ def _dot_weighted(words, slice_weights, Sa, W, keys: PrebuiltBSIKeysCUDA, Q, dec
                                        _scale_inv(decimals_q, keys.decimals), R, out.data_ptr(), _stream()),
               "bsi_hip_dot_weighted")
         if bias is not None:
-            out += bias
+            check(lib.bsi_hip_add_bias(out.data_ptr(), bias.data_ptr(), Q, R, R, _stream()), "bsi_hip_add_bias")
     ns = 0
     if prof:
         e1.record()
@@ -967,7 +988,7 @@ def linear_few_rows_cuda(x2d: torch.Tensor, keyset_cuda_cap, decimal_places: int
 
 
 _last_linear_rebuilt = [False]  # whether the last linear_cuda call ran the query build (layer counters read it)
-_linear_ws: dict = {}  # device index -> {"bytes": size of one workspace, "buf": tensor of two, "eager": [...], "capture": [...]}
+_linear_ws: dict = {}  # device index -> {"bytes", "eager_buf", "capture_buf", "captured", "eager": [key, input], "capture": [...]}
 
 
 def can_linear_one_call(x2d: torch.Tensor, keys: "PrebuiltBSIKeysCUDA") -> bool:
@@ -983,13 +1004,22 @@ def can_linear_one_call(x2d: torch.Tensor, keys: "PrebuiltBSIKeysCUDA") -> bool:
 
 
 def _linear_workspace(device, need: int, capturing: bool) -> dict:
-    """linear_cuda's workspace record of ``device``, (re)allocated when it is missing or smaller than ``need`` bytes."""
+    """linear_cuda's workspace record of ``device``: one buffer for eager calls and one for launches recorded into a
+    graph, both (re)allocated outside captures when they are missing or smaller than ``need`` bytes.  A recorded
+    launch holds the capture buffer's address, so once a capture has used it, it is kept alive for good: a larger
+    need adds a new buffer for later captures and retires the old one instead of freeing it."""
     ws = _linear_ws.get(device.index)
     if ws is None or ws["bytes"] < need:
         _check(not capturing, "linear_cuda: the workspace must exist before a graph is captured (run the forward once)")
         size = (max(need, 1 << 20) + 255) // 256 * 256
-        ws = _linear_ws[device.index] = {"bytes": size, "buf": torch.empty((2 * size,), dtype=torch.uint8, device=device),
+        if ws is not None and ws["captured"]:
+            _retired_workspaces.append(ws["capture_buf"])
+        ws = _linear_ws[device.index] = {"bytes": size, "captured": False,
+                                         "eager_buf": torch.empty((size,), dtype=torch.uint8, device=device),
+                                         "capture_buf": torch.empty((size,), dtype=torch.uint8, device=device),
                                          "eager": [None, None], "capture": [None, None]}
+    if capturing:
+        ws["captured"] = True
     return ws
 
 
@@ -1029,10 +1059,10 @@ def linear_cuda(x2d: torch.Tensor, keyset_cuda_cap, decimal_places: int, bias=No
     capturing = _capturing()
     ws = _linear_workspace(x2d.device, need, capturing)
     slot = ws["capture" if capturing else "eager"]
-    key = (x2d.data_ptr(), Q, d, x2d.dtype, x2d._version, bits, int(decimal_places))
-    rebuild = 0 if slot[0] == key else 1
+    key = tensor_build_key(x2d, int(decimal_places))
+    rebuild = 0 if (key is not None and slot[0] == key) else 1
     slot[0], slot[1] = key, x2d  # holds the input, so that its address is not reused while the build stands for it
-    wsptr = ws["buf"].data_ptr() + (ws["bytes"] if capturing else 0)
+    wsptr = ws["capture_buf" if capturing else "eager_buf"].data_ptr()
     out = torch.empty((Q, R), dtype=torch.float32, device=x2d.device)
     core = f["core"]
     kptr, klayout = key_operand(keys, Q, bits, core)

@@ -724,7 +724,7 @@ extern "C" int bsi_hip_decimal_stats(const int64_t* ints, int64_t Q, int64_t d, 
     return BSI_OK;
 }
 
-int bsi::g_build_items = 0;
+std::atomic<int> bsi::g_build_items{0};
 
 extern "C" int bsi_hip_build_fixed(const void* x, int dtype, int64_t Q, int64_t d, int decimal_places, int fixed_bits,
                                    int chunk_scale, float clip_k, uint64_t* words, int32_t* shifts, float* scales,
@@ -751,7 +751,7 @@ extern "C" int bsi_hip_build_fixed(const void* x, int dtype, int64_t Q, int64_t 
     }
         // a wave gets more items only once there are about 8 waves per SIMD (8192 in all); measured on
         // 4096 ... 131072 items, every other choice is within a few percent or slower
-        int per_wave = g_build_items;
+        int per_wave = g_build_items.load(std::memory_order_relaxed);
         if (per_wave == 0) per_wave = items > 8 * 16384 ? 8 : (items >= 16384 ? 4 : (items >= 8192 ? 2 : 1));
         if (per_wave == 8) BSI_LAUNCH_FAST(8)
         else if (per_wave == 4) BSI_LAUNCH_FAST(4)

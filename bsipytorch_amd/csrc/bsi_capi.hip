@@ -8,6 +8,11 @@ std::string& last_error_ref() {
     return msg;
 }
 
+hipError_t& pending_config_error() {
+    static thread_local hipError_t e = hipSuccess;
+    return e;
+}
+
 int fail(int code, const char* fmt, ...) {
     char buf[1024];
     va_list ap;
@@ -65,7 +70,10 @@ template <typename F>
 static int time_launch(hipStream_t st, int reps, float* ms_best, F&& launch) {
     hipEvent_t e0, e1;
     BSI_HIP_CHECK(hipEventCreate(&e0));
-    BSI_HIP_CHECK(hipEventCreate(&e1));
+    if (hipError_t ec = hipEventCreate(&e1); ec != hipSuccess) {
+        (void)hipEventDestroy(e0);
+        return fail(BSI_ERR_HIP, "hipEventCreate failed: %s", hipGetErrorString(ec));
+    }
     float best = 1e30f;
     hipError_t err = hipSuccess;
     for (int r = 0; r < reps && err == hipSuccess; ++r) {

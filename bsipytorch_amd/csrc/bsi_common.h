@@ -6,6 +6,7 @@
 #include <hip/hip_bf16.h>
 #include <stdint.h>
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <string>
@@ -34,10 +35,31 @@ int fail(int code, const char* fmt, ...);
             return ::bsi::fail(BSI_ERR_HIP, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(_e), __FILE__, __LINE__); \
     } while (0)
 
+// A kernel's opt-in to more than 64 KiB of dynamic LDS, done once per kernel and device.  Any number of threads may
+// launch the kernel at the same time (the worst case is that two of them set the attribute); a failure is kept for
+// the launch check that follows, which reports it instead of the launch error it would cause.
+struct LdsOptIn {
+    std::atomic<uint64_t> devices{0};  // bit d: done on device d (devices past 63 set it on every launch)
+};
+hipError_t& pending_config_error();
+inline void lds_opt_in(LdsOptIn& once, const void* kernel, int bytes) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    const uint64_t bit = (dev >= 0 && dev < 64) ? (uint64_t{1} << dev) : 0;
+    if (e == hipSuccess && bit != 0 && (once.devices.load(std::memory_order_acquire) & bit) != 0) return;
+    if (e == hipSuccess) e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess) once.devices.fetch_or(bit, std::memory_order_release);
+    else pending_config_error() = e;
+}
+
 // After a kernel launch: surface launch-configuration errors immediately.
 #define BSI_LAUNCH_CHECK(name)                                                                       \
     do {                                                                                             \
+        hipError_t _c = ::bsi::pending_config_error();                                               \
+        ::bsi::pending_config_error() = hipSuccess;                                                  \
         hipError_t _e = hipGetLastError();                                                           \
+        if (_c != hipSuccess)                                                                        \
+            return ::bsi::fail(BSI_ERR_HIP, "LDS opt-in of %s failed: %s", name, hipGetErrorString(_c)); \
         if (_e != hipSuccess)                                                                        \
             return ::bsi::fail(BSI_ERR_HIP, "launch of %s failed: %s", name, hipGetErrorString(_e)); \
     } while (0)
@@ -144,7 +166,7 @@ __device__ __forceinline__ unsigned wave_max_u32(unsigned v) {
     return ab > cd ? ab : cd;
 }
 
-extern int g_build_items;  // BSI_OPT_BUILD_ITEMS (bsi_build.hip)
+extern std::atomic<int> g_build_items;  // BSI_OPT_BUILD_ITEMS (bsi_build.hip)
 
 // 10^dec as an integer when scaled_magnitude_u32 can take it (at most 127), else 0: float64 arithmetic then.
 static inline unsigned integer_decimal_scale(double dec_scale) {

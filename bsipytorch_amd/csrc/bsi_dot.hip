@@ -765,8 +765,8 @@ __device__ __forceinline__ void load16_to_lds(bsi_rsrc r, uint32_t lane_off, uin
 // Tile configuration: TM keys x TN queries per workgroup (128 x 128, 128 x 64, 64 x 64 or 64 x 32; the smaller
 // ones for grids that would leave CUs without a workgroup), MFMA waves arranged 2 (keys) x kWavesN (queries),
 // each WM x WN tiles of 16 x 16; one loader wave per (up to) 64 operand rows.
-static int g_i8_tile = 0;  // 0 = by grid size; 128, 12864 (128 keys x 64 queries) or 64 force a tile
-static int g_digits_route = 0;  // bsi_hip_dot_digits: 0 = by cost, 1 = stacked digits + combine pass, 2 = in-accumulator
+static std::atomic<int> g_i8_tile{0};  // 0 = by grid size; 128, 12864 (128 keys x 64 queries) or 64 force a tile
+static std::atomic<int> g_digits_route{0};  // bsi_hip_dot_digits: 0 = by cost, 1 = stacked digits + combine pass, 2 = in-accumulator
 
 template <int TM, int TN>
 struct I8Cfg {
@@ -2110,14 +2110,10 @@ static void launch_mfma(const int8_t* A8, const float* qscale, int stride, const
                         float* out, int32_t* chunk_ints, hipStream_t st) {
     const dim3 grid(static_cast<unsigned>((R + kTileR - 1) / kTileR), static_cast<unsigned>((Q + kTileQ - 1) / kTileQ));
     constexpr int kLds = (kTileR + kTileQ) * kRowBytes;  // above the 64 KiB default: opt in once per kernel
-    static bool configured = false;
-    if (!configured) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dot_mfma_kernel<SB, kTiled, true>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dot_mfma_kernel<SB, kTiled, false>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
-        configured = true;
-    }
+    static LdsOptIn once0;
+    lds_opt_in(once0, reinterpret_cast<const void*>(&dot_mfma_kernel<SB, kTiled, true>), kLds);
+    static LdsOptIn once1;
+    lds_opt_in(once1, reinterpret_cast<const void*>(&dot_mfma_kernel<SB, kTiled, false>), kLds);
     if (chunk_ints)
         hipLaunchKernelGGL((dot_mfma_kernel<SB, kTiled, true>), grid, dim3(kMfmaBlock), kLds, st, A8, qscale, stride,
                            reinterpret_cast<const uint32_t*>(B), Bw, Sb, W64, chunks, R, Q, down_shift, scale_inv,
@@ -2134,14 +2130,10 @@ static void launch_mfma_ws(const int8_t* A8, const float* qscale, int stride, co
                            float* out, int32_t* chunk_ints, hipStream_t st) {
     const dim3 grid(static_cast<unsigned>((R + kTileR - 1) / kTileR), static_cast<unsigned>((Q + kTileQ - 1) / kTileQ));
     constexpr int kLds = 2 * kWsStage;
-    static bool configured = false;
-    if (!configured) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dot_mfma_ws_kernel<SB, true>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dot_mfma_ws_kernel<SB, false>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
-        configured = true;
-    }
+    static LdsOptIn once0;
+    lds_opt_in(once0, reinterpret_cast<const void*>(&dot_mfma_ws_kernel<SB, true>), kLds);
+    static LdsOptIn once1;
+    lds_opt_in(once1, reinterpret_cast<const void*>(&dot_mfma_ws_kernel<SB, false>), kLds);
     if (chunk_ints)
         hipLaunchKernelGGL((dot_mfma_ws_kernel<SB, true>), grid, dim3(kWsBlock), kLds, st, A8, qscale, stride,
                            reinterpret_cast<const unsigned long long*>(B), Bw, chunks, R, Q, down_shift, scale_inv,
@@ -2163,12 +2155,8 @@ static void launch_mfma_i8_tm(const int8_t* A8, const float* qscale, int stride,
                               int ndig, long long dig_stride, const long long* key_indices, int key_tiled) {
     using C = I8Cfg<TM, TN>;
     const dim3 grid(static_cast<unsigned>((R + TM - 1) / TM), static_cast<unsigned>((Q + TN - 1) / TN));
-    static bool configured = false;
-    if (!configured) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dot_mfma_i8_kernel<TM, TN, kMode>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, C::kLds);
-        configured = true;
-    }
+    static LdsOptIn once0;
+    lds_opt_in(once0, reinterpret_cast<const void*>(&dot_mfma_i8_kernel<TM, TN, kMode>), C::kLds);
     hipLaunchKernelGGL((dot_mfma_i8_kernel<TM, TN, kMode>), grid, dim3(C::kBlock), C::kLds, st, A8, qscale, stride, K8,
                        Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias, ndig, dig_stride,
                        key_indices, key_tiled, static_cast<const unsigned char*>(g_warm_ptr),
@@ -2201,7 +2189,7 @@ static void launch_mfma_i8_t(int ndig, long long dig_stride, const long long* ke
 static int choose_i8_tile(int64_t R, int64_t Q, int64_t* cost_out = nullptr) {
     const int64_t n128 = ((R + 127) / 128) * ((Q + 127) / 128);
     if (cost_out) *cost_out = ((n128 + 255) / 256) * 100;
-    if (g_i8_tile != 0) return g_i8_tile;
+    if (const int forced = g_i8_tile.load(std::memory_order_relaxed)) return forced;
     if (n128 > 256) return 128;
     const int64_t cost[4] = {100, ((((R + 127) / 128) * ((Q + 63) / 64) + 255) / 256) * 63,
                              ((((R + 63) / 64) * ((Q + 63) / 64) + 255) / 256) * 35,
@@ -2445,6 +2433,17 @@ static int dot_with_bias(const uint64_t* A, const int8_t* A_ints8, const float* 
     return BSI_OK;
 }
 
+extern "C" int bsi_hip_add_bias(float* out, const float* bias, int64_t Q, int64_t R, int64_t R_total, void* stream) {
+    BSI_REQUIRE(Q >= 0 && R >= 0 && R_total >= R, "bad shape");
+    if (Q == 0 || R == 0) return BSI_OK;
+    BSI_REQUIRE(out && bias, "null pointer");
+    const int64_t total = Q * R;
+    hipLaunchKernelGGL(add_bias_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, as_stream(stream),
+                       out, bias, Q, R, R_total);
+    BSI_LAUNCH_CHECK("add_bias_kernel");
+    return BSI_OK;
+}
+
 extern "C" int bsi_hip_dot(const uint64_t* A, const int8_t* A_ints8, const float* A_chunk_scales, int A_scale_stride,
                            int Sa, int W64, const uint64_t* B, int b_layout, const float* Bw, int Sb, int64_t R,
                            int64_t Q, float scale_inv, int64_t R_total, float* out, int32_t* chunk_ints, int core,
@@ -2509,12 +2508,8 @@ static void launch_stream_fused(const FusedPlan& plan, const T* x, int64_t d, do
     if (pass_chunks > fit) pass_chunks = fit;
     if (pass_chunks > chunks) pass_chunks = chunks;
     const size_t lds = static_cast<size_t>(pass_chunks) * kSlot * sizeof(int) + query_bytes;
-    static bool configured = false;
-    if (!configured) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dot_mfma_stream_fused_kernel<T, KT, NI>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        configured = true;
-    }
+    static LdsOptIn once0;
+    lds_opt_in(once0, reinterpret_cast<const void*>(&dot_mfma_stream_fused_kernel<T, KT, NI>), 160 * 1024);
     const unsigned scale_int = integer_decimal_scale(dec_scale);
     hipLaunchKernelGGL((dot_mfma_stream_fused_kernel<T, KT, NI>), dim3(plan.grid), dim3(plan.waves * 64), lds, st, x, d,
                        dec_scale, scale_int, slices, reinterpret_cast<const unsigned long long*>(B), Bw, chunks, pass_chunks,
@@ -2649,14 +2644,10 @@ extern "C" int bsi_hip_dot_ewah_query(const uint64_t* comp_words, const int64_t*
     if (waves < 4) waves = 4;
     hipStream_t st = as_stream(stream);
     const dim3 grid(static_cast<unsigned>((R + 15) / 16));
-    static bool configured = false;
-    if (!configured) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dot_mfma_stream_ewah_kernel<true>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dot_mfma_stream_ewah_kernel<false>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        configured = true;
-    }
+    static LdsOptIn once0;
+    lds_opt_in(once0, reinterpret_cast<const void*>(&dot_mfma_stream_ewah_kernel<true>), 160 * 1024);
+    static LdsOptIn once1;
+    lds_opt_in(once1, reinterpret_cast<const void*>(&dot_mfma_stream_ewah_kernel<false>), 160 * 1024);
     const int down_shift = 16 - Sa - Sb;
     if (chunk_ints)
         hipLaunchKernelGGL((dot_mfma_stream_ewah_kernel<true>), grid, dim3(waves * 64), lds, st,
@@ -2680,12 +2671,8 @@ static int launch_dot_weighted(const uint64_t* A, const float* Aw, int Sa, int W
                                int64_t R_total, float* out, double* out64, hipStream_t st) {
     const size_t lds = static_cast<size_t>(32) * ((Sa * WB + 1) + (Sb * WB + 1)) * 8 + static_cast<size_t>(32) * (Sa + Sb) * 4;
     if (lds > 150 * 1024) return fail(BSI_ERR_UNSUPPORTED, "slice counts %d + %d do not fit the LDS tile", Sa, Sb);
-    static bool configured = false;
-    if (!configured) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dot_weighted_kernel<WB, kTiled>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
-        configured = true;
-    }
+    static LdsOptIn once0;
+    lds_opt_in(once0, reinterpret_cast<const void*>(&dot_weighted_kernel<WB, kTiled>), 150 * 1024);
     const dim3 grid(static_cast<unsigned>((R + 31) / 32), static_cast<unsigned>((Q + 31) / 32));
     hipLaunchKernelGGL((dot_weighted_kernel<WB, kTiled>), grid, dim3(256), lds, st,
                        reinterpret_cast<const unsigned long long*>(A), Aw, Sa, W64,
@@ -2787,7 +2774,8 @@ extern "C" int bsi_hip_dot_digits(const int8_t* A_digits, int nq, const float* A
     const double us_fold = 0.012 * static_cast<double>(cost_fold) * chunks * nq * ((tile_fold == 64 || tile_fold == 6432) ? 1.3 : 1.0);
     const double us_stack = 0.012 * static_cast<double>(cost_stack) * chunks * ((tile_stack == 64 || tile_stack == 6432) ? 1.3 : 1.0) + 3.0 +
                             static_cast<double>(nq * nk + 1) * static_cast<double>(Q) * static_cast<double>(R) * 4.0 / 4.0e6;
-    const bool fold = g_digits_route == 2 || (g_digits_route == 0 && (nq == 1 || us_fold <= us_stack));
+    const int route = g_digits_route.load(std::memory_order_relaxed);
+    const bool fold = route == 2 || (route == 0 && (nq == 1 || us_fold <= us_stack));
     if (can_fold && fold) {
         launch_mfma_i8(A_digits, Aw, Sa, K_digits, Bw, Sb, chunks, R, Q, preshift, scale_inv, R_total, out, nullptr, bias,
                        st, k_tiled, nq, dig_stride, reinterpret_cast<const long long*>(key_indices));

@@ -33,8 +33,8 @@ def forget_shared_builds() -> None:
 
 def _cached_query_build(batch_inputs: torch.Tensor, decimal_places: int, threshold: float, packed: bool):
     use_cache = bsi_ops.fast_getenv("BSI_QUERY_CACHE", "1") != "0"
-    key = (batch_inputs.data_ptr(), tuple(batch_inputs.shape), batch_inputs.dtype, batch_inputs._version,
-           int(decimal_places), bool(packed))
+    key = bsi_ops.tensor_build_key(batch_inputs, int(decimal_places), bool(packed)) if use_cache else None
+    use_cache = use_cache and key is not None  # a tensor without a version counter (inference mode) is built anew
     if use_cache and _last_query_build.get("key") == key and _last_query_build.get("src") is not None:
         return _last_query_build["cap"], True
     if packed:
@@ -207,9 +207,9 @@ class BSIQuantizedLinear(nn.Module):
         fp32 = original_dtype == torch.float32
         if fused is not None:
             group, start, stop = fused
-            key = (batch_inputs.data_ptr(), tuple(batch_inputs.shape), batch_inputs.dtype, batch_inputs._version)
+            key = bsi_ops.tensor_build_key(batch_inputs)
             last = group.__dict__.get("_last_call")
-            if last is not None and last[0] == key:
+            if last is not None and key is not None and last[0] == key:
                 scores, bias_done = last[2][:, start:stop], last[3]
                 last[4] -= 1
                 if last[4] <= 0:
@@ -258,9 +258,9 @@ class BSIQuantizedLinear(nn.Module):
         bsi_ops.reserve_linear_workspace(batch_inputs)  # a later capture of this forward may take the one-call path
         if fused is not None:
             group, start, stop = fused
-            key = (batch_inputs.data_ptr(), tuple(batch_inputs.shape), batch_inputs.dtype, batch_inputs._version)
+            key = bsi_ops.tensor_build_key(batch_inputs)
             last = group.__dict__.get("_last_few")
-            if last is not None and last[0] == key:
+            if last is not None and key is not None and last[0] == key:
                 scores, bias_done = last[2][:, start:stop], last[3]
                 last[4] -= 1
                 if last[4] <= 0:

@@ -219,6 +219,11 @@ int bsi_hip_dot_bias(const uint64_t* A, const int8_t* A_ints8, const float* A_ch
                      float scale_inv, int64_t R_total, const float* bias, float* out, int core, void* workspace,
                      size_t workspace_bytes, void* stream);
 
+/* out[q, r] += bias[r] for q < Q, r < R on out float [Q, R_total]: the bias step of a BSI-linear forward
+ * (scores + bias, verify_accuracy_bsi.py:193-195, a PyTorch addition in the reference) for the dots that do not
+ * take a bias argument (bsi_hip_dot with chunk_ints, bsi_hip_dot_weighted). */
+int bsi_hip_add_bias(float* out, const float* bias, int64_t Q, int64_t R, int64_t R_total, void* stream);
+
 /* bsi_hip_dot_bias that also warms the memory-side cache for the NEXT dot: `warm` .. `warm + warm_bytes` (device
  * memory, typically the key operand of the layer that runs next) is read once, one access per 128-byte line, by
  * the int8-image kernel's loader waves after they have issued their last stage.  A keyset that is not cache-resident

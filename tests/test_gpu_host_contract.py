@@ -1,0 +1,139 @@
+"""Host-side contracts of the BSI-linear drop-in that need the GPU: workspaces whose addresses a recorded HIP
+graph holds stay valid when later calls need larger ones, and the layer works on tensors that carry no version
+counter (``torch.inference_mode()``), as the reference layer does (verify_accuracy_bsi.py:118-215)."""
+import os
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture()
+def ops(monkeypatch):
+    from bsipytorch_amd import bsi_ops
+
+    for k in list(os.environ):
+        if k.startswith("BSI_"):
+            monkeypatch.delenv(k)
+    bsi_ops._reset_flag_cache()
+    yield bsi_ops
+    bsi_ops._reset_flag_cache()
+
+
+def _capture(fn, warm):
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        warm()
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        out = fn()
+    return g, out
+
+
+def test_graph_replay_survives_a_larger_eager_call(ops):
+    """Capture a forward at 64 rows, then run an eager forward that needs a workspace sixteen times larger, then
+    replay: the replay must still build into memory it owns and give the eager bits."""
+    from bsipytorch_amd import linear
+
+    torch.manual_seed(3)
+    model = torch.nn.ModuleList([torch.nn.Linear(1024, 320).cuda(), torch.nn.Linear(1024, 192).cuda()])
+    linear.quantize_model_bsi(model, decimalPlaces=2, compress_threshold=0.5, verbose=False)
+    ops._linear_ws.clear()
+    ops._reserved_linear_shapes.clear()
+    x = torch.randn(64, 1024, device="cuda")
+    big = torch.randn(4096, 1024, device="cuda")
+    with torch.no_grad():
+        want = [m(x).clone() for m in model]
+        static_x = x.clone()
+        linear.forget_shared_builds()
+        g, outs = _capture(lambda: [m(static_x) for m in model], lambda: [m(static_x) for m in model])
+        linear.forget_shared_builds()
+        small_bytes = ops._linear_ws[x.device.index]["bytes"]
+        captured_ptr = ops._linear_ws[x.device.index]["capture_buf"].data_ptr()
+        big_out = [m(big) for m in model]                     # grows both workspaces
+        assert ops._linear_ws[x.device.index]["bytes"] > small_bytes
+        assert any(t.data_ptr() == captured_ptr for t in ops._retired_workspaces)
+        # memory the allocator hands out now must not be what the recorded launches write
+        fill = [torch.full((small_bytes,), 0x5A, dtype=torch.uint8, device="cuda") for _ in range(4)]
+        for rep in range(3):
+            static_x.copy_(x * (rep + 1))
+            g.replay()
+            torch.cuda.synchronize()
+            assert all(torch.equal(a, m(x * (rep + 1))) for a, m in zip(outs, model))
+            assert all(bool((t == 0x5A).all()) for t in fill)
+        static_x.copy_(x)
+        g.replay()
+        torch.cuda.synchronize()
+        assert all(torch.equal(a, b) for a, b in zip(outs, want))
+        assert all(torch.equal(a, m(big)) for a, m in zip(big_out, model))
+
+
+def test_dot_workspace_is_retired_not_freed_after_a_capture(ops):
+    """The dot's own scratch buffer (decimal digit products): a buffer a capture has used is kept when a larger one
+    replaces it, and growing inside a capture raises."""
+    dev = torch.device("cuda", torch.cuda.current_device())
+    ops._workspace.clear()
+    a = ops._get_workspace(1 << 16, dev)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        inside = ops._get_workspace(1 << 12, dev)
+        inside[:16].zero_()
+    assert inside.data_ptr() == a.data_ptr() and ops._workspace[dev]["captured"]
+    before = len(ops._retired_workspaces)
+    b = ops._get_workspace(1 << 20, dev)
+    assert b.data_ptr() != a.data_ptr() and len(ops._retired_workspaces) == before + 1
+    assert ops._retired_workspaces[-1].data_ptr() == a.data_ptr()
+    g2 = torch.cuda.CUDAGraph()
+    with pytest.raises(RuntimeError, match="larger workspace"):
+        with torch.cuda.graph(g2):
+            ops._get_workspace(1 << 24, dev)
+    torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("rows", [3, 48])
+def test_layer_and_fused_qkv_under_inference_mode(ops, monkeypatch, dtype, rows):
+    """Inference tensors keep no version counter: nothing may read it, builds are not shared, results are the bits of
+    the same forward under no_grad (few-rows kernel, one-call path and the two-call path)."""
+    from bsipytorch_amd import linear
+
+    class Attn(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.q_proj = torch.nn.Linear(512, 128)
+            self.k_proj = torch.nn.Linear(512, 128)
+            self.v_proj = torch.nn.Linear(512, 192, bias=False)
+            self.out_proj = torch.nn.Linear(512, 100)
+
+        def forward(self, x):
+            return self.q_proj(x), self.k_proj(x), self.v_proj(x), self.out_proj(x)
+
+    torch.manual_seed(9)
+    plain = Attn().cuda()
+    fused = Attn().cuda()
+    fused.load_state_dict(plain.state_dict())
+    linear.quantize_model_bsi(plain, decimalPlaces=2, compress_threshold=0.5, verbose=False)
+    linear.quantize_model_bsi(fused, decimalPlaces=2, compress_threshold=0.5, verbose=False, fuse_qkv=True)
+    x = torch.randn(rows, 512, device="cuda").to(dtype)
+    for one_call in ("1", "0"):
+        monkeypatch.setenv("BSI_LINEAR_ONE_CALL", one_call)
+        linear.forget_shared_builds()
+        with torch.no_grad():
+            want = [t.clone() for t in plain(x)]
+        linear.forget_shared_builds()
+        with torch.no_grad():
+            want2 = [t.clone() for t in plain(x + 1.0)]
+        linear.forget_shared_builds()
+        with torch.inference_mode():
+            for model in (plain, fused):
+                xi = x.clone()                  # an inference tensor
+                assert xi.is_inference()
+                got = model(xi)
+                assert all(torch.equal(a, b) for a, b in zip(got, want))
+                xi.add_(1.0)                    # in-place work on it must not be mistaken for "unchanged"
+                got2 = model(xi)
+                assert all(torch.equal(a, b) for a, b in zip(got2, want2))

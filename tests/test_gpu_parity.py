@@ -1525,16 +1525,6 @@ def test_model_harness_helpers(ops, capsys):
     assert linear.collect_bsi_error_stats(model)[0]["samples_tracked"] == 20
 
 
-def test_collect_bsi_shape_stats(ops):
-    from bsipytorch_amd import linear
-    from bsipytorch_amd.benchmarks import collect_bsi_shape_stats as cs
-
-    model = torch.nn.Sequential(torch.nn.Linear(256, 128), torch.nn.ReLU(), torch.nn.Linear(128, 64)).cuda()
-    linear.quantize_model_bsi(model, decimalPlaces=2, compress_threshold=0.5, verbose=False)
-    res = cs.collect(model)
-    assert res["W"] == {4: 1, 2: 1} and res["Sb"] == {6: 192} and [r[0] for r in res["layers"]] == ["0", "2"]
-
-
 # ------------------------------------------------------------------ fused build + dot for a few rows
 
 
