@@ -52,6 +52,7 @@ PROTOTYPES = {
     "bsi_hip_set_option": [_i, _i],
     "bsi_hip_dot_workspace_bytes": [_i64, _i, _i],
     "bsi_hip_dot": [_vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _i, _i64, _i64, _f, _i64, _vp, _vp, _i, _vp, _sz, _vp],
+    "bsi_hip_dot_static_scratch": [_vp, _vp, _i, _i, _i, _vp, _i, _vp, _i, _i64, _i64, _f, _i64, _vp, _vp, _vp],
     "bsi_hip_add_bias": [_vp, _vp, _i64, _i64, _i64, _vp],
     "bsi_hip_dot_bias": [_vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _i, _i64, _i64, _f, _i64, _vp, _vp, _i, _vp, _sz, _vp],
     "bsi_hip_dot_bias_warm": [_vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _i, _i64, _i64, _f, _i64, _vp, _vp, _i, _vp, _sz, _vp, _sz, _vp],

@@ -2475,6 +2475,46 @@ extern "C" int bsi_hip_dot_bias_warm(const uint64_t* A, const int8_t* A_ints8, c
     return rc;
 }
 
+// ------------------------------------------------------------------ the dot without any allocation
+// The int8 query operands that bsi_hip_dot derives into a caller's workspace go, here, into an array that is part
+// of the library's device image: one copy per GPU, there from the moment the code object is loaded until the
+// process ends.  In host code the array's name is only a handle for hipGetSymbolAddress; the device address it
+// returns (one per device) is what the kernels get.
+constexpr size_t kStaticScratchBytes = BSI_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+static std::atomic<void*> g_scratch_ptr[64];  // per device: the array's address there, once looked up
+
+static int static_scratch(void** out) {
+    int dev = 0;
+    BSI_HIP_CHECK(hipGetDevice(&dev));
+    BSI_REQUIRE(dev >= 0 && dev < 64, "device index %d is beyond the 64 this entry point keeps addresses for", dev);
+    void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (p == nullptr) {
+        BSI_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        BSI_REQUIRE(p != nullptr, "hipGetSymbolAddress returned no address for the scratch array");
+        g_scratch_ptr[dev].store(p, std::memory_order_release);
+    }
+    *out = p;
+    return BSI_OK;
+}
+
+extern "C" int bsi_hip_dot_static_scratch(const uint64_t* A, const float* A_chunk_scales, int A_scale_stride, int Sa,
+                                          int W64, const uint64_t* B, int b_layout, const float* Bw, int Sb, int64_t R,
+                                          int64_t Q, float scale_inv, int64_t R_total, float* out, int32_t* chunk_ints,
+                                          void* stream) {
+    BSI_REQUIRE(A != nullptr, "the query planes are required (the int8 operands are derived from them)");
+    BSI_REQUIRE(Sa >= 2 && Sa <= 8 && Sb >= 2 && Sb <= 8, "the matrix-core dot needs Sa, Sb in [2, 8] (got %d, %d)", Sa, Sb);
+    BSI_REQUIRE(Q >= 0 && W64 >= 1, "bad shape");
+    const size_t need = bsi_hip_dot_workspace_bytes(Q, W64, BSI_CORE_MFMA);
+    BSI_REQUIRE(need <= kStaticScratchBytes,
+                "Q x padded D = %zu bytes of int8 query operands exceed the %zu-byte static scratch; use bsi_hip_dot "
+                "with a workspace", need, kStaticScratchBytes);
+    void* ws = nullptr;
+    if (int rc = static_scratch(&ws)) return rc;
+    return dot_with_bias(A, nullptr, A_chunk_scales, A_scale_stride, Sa, W64, B, b_layout, Bw, Sb, R, Q, scale_inv, R_total,
+                         out, chunk_ints, BSI_CORE_MFMA, ws, kStaticScratchBytes, stream, nullptr);
+}
+
 // Launch shape of the fused few-rows kernel: key tiles per workgroup, waves, and how many (chunk, row) items of the
 // query build a wave takes up front (loads issued before the key loads; the rest go one at a time, each waiting for
 // its own loads).

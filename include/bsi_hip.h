@@ -210,6 +210,19 @@ int bsi_hip_dot(const uint64_t* A, const int8_t* A_ints8, const float* A_chunk_s
                 float scale_inv, int64_t R_total, float* out, int32_t* chunk_ints, int core, void* workspace,
                 size_t workspace_bytes, void* stream);
 
+/* bsi_hip_dot on the matrix cores for callers that cannot allocate device memory or hold a workspace of their own
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  The int8 query operands are derived from the planes A into a BSI_STATIC_SCRATCH_BYTES array inside the
+ * library's device image (one per GPU, held until the process ends) instead of a caller's workspace; the call makes no
+ * hipMalloc / hipFree and no other allocating call.  Q * ceil(W64 / 4) * 256 must not exceed BSI_STATIC_SCRATCH_BYTES
+ * (BSI_ERR_INVALID otherwise; bsi_hip_dot with a workspace has no such limit).  Every call on a GPU writes the same
+ * array: calls that overlap on one GPU (two streams, two threads) race, calls on one stream do not.  Nothing in the
+ * array has to start at zero: each call overwrites the part it reads.  Arguments and results as bsi_hip_dot. */
+#define BSI_STATIC_SCRATCH_BYTES (8u << 20)
+int bsi_hip_dot_static_scratch(const uint64_t* A, const float* A_chunk_scales, int A_scale_stride, int Sa, int W64,
+                               const uint64_t* B, int b_layout, const float* Bw, int Sb, int64_t R, int64_t Q,
+                               float scale_inv, int64_t R_total, float* out, int32_t* chunk_ints, void* stream);
+
 /* bsi_hip_dot followed by out[q, r] += bias[r] (bias: float [R], may be NULL), the two steps of a BSI-linear
  * forward (scores = dot(...); scores + bias, verify_accuracy_bsi.py:185-209) in one call.  The sum is rounded as
  * the separate addition would round it; the matrix-core kernels add the bias in their epilogue, the others
