@@ -254,3 +254,27 @@ def test_product_sources_never_reach_for_the_checker():
         if re.search(r"\boracle\b", open(f, errors="replace").read()):
             offenders.append(os.path.relpath(f, ROOT))
     assert offenders == []
+
+
+# The launchers the reference's C++ declares (bsi_cuda.cpp:29-57, bsi_vector_cuda.cpp:91-242).
+REFERENCE_LAUNCHERS = [
+    "launch_ewah_decompress", "launch_popcount_weighted_keys_literal_fused_multiq", "launch_pack_bits_all_ballot",
+    "launch_pack_bits_all_ballot_batch", "launch_quantize_round_to_int64_batch", "launch_compute_row_shift_scale",
+    "launch_compute_chunk_shift_scale", "launch_apply_row_shift_clamp", "launch_apply_chunk_shift_clamp",
+    "launch_compute_row_shift_scale_from_input", "launch_compute_chunk_shift_scale_from_input",
+    "launch_quantize_shift_pack_row_batch", "launch_quantize_shift_pack_chunk_batch", "launch_slice_popcount_sum",
+    "launch_compress_flags_from_density", "launch_ewah_size", "launch_ewah_emit",
+]
+
+
+def test_reference_launcher_library_exports_the_reference_symbols():
+    """libbsi_reference_launchers.so (what a ROCm build of the reference extension links instead of its CUDA
+    kernels) loads next to libbsi_hip.so and exports every launcher the reference's sources call."""
+    path = os.path.join(ROOT, "bsipytorch_amd", "libbsi_reference_launchers.so")
+    assert os.path.exists(path), "build it with make -C bsipytorch_amd/csrc"
+    raw = ctypes.CDLL(path)
+    for n in REFERENCE_LAUNCHERS:
+        assert hasattr(raw, n), f"{n} is not exported"
+    raw.bsi_launchers_last_error.restype = ctypes.c_char_p
+    raw.bsi_launchers_clear_status()
+    assert raw.bsi_launchers_last_status() == 0 and raw.bsi_launchers_last_error() == b""
