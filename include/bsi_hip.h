@@ -298,7 +298,8 @@ int bsi_hip_dot_ewah_query(const uint64_t* comp_words, const int64_t* comp_off, 
  * A [Q, Sa, W64], Aw [Q, Sa], B [R, Sb, W64] (canonical or tiled16), Bw [R, Sb], Sa, Sb in [1, 64];
  * key_indices (may be NULL = identity) maps row r of B to its output column, as the reference's keys grouped
  * by slice count need (bsi_cuda.cpp:956-1000).  The sum is exact in float64 while it stays below 2^53 and is
- * rounded once, where the reference adds the same terms in fp32 in an order set by its launch shape.
+ * rounded once, where the reference adds the same terms in fp32 in an order set by its launch shape (the two agree
+ * bit for bit while every fp32 partial sum stays below 2^24, and to the reference order's own rounding error beyond).
  * Replaces launch_popcount_weighted_keys_literal_fused_multiq without chunk scales
  * (bsi_cuda_kernels_dot.cuh:58-190 fallback kernel, :211-1283 tensor-core kernel, dispatch :2575-3090). */
 int bsi_hip_dot_weighted(const uint64_t* A, const float* Aw, int Sa, int W64, const uint64_t* B, int b_layout,
