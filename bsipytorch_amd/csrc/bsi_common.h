@@ -202,4 +202,39 @@ __device__ __forceinline__ unsigned long long wave_sum_u64(unsigned long long v)
     return v;
 }
 
+// One wave expands one EWAH stream (in[0 .. in_len), [marker][literals...] with marker = run_bit | run_len << 1 |
+// literal_count << 33) into dst[0 .. wpad): W decoded words, zeros after them.  Bounds as the reference decoder's
+// (bsi_ops/csrc/cuda/bsi_cuda_kernels_ewah.cuh:5-33): output clipped at W words, input at in_len, the rest zero.
+// dst may be global memory or LDS.  The markers form a chain; the wave follows it through a window of 64 stream
+// words held one per lane, so stepping to the next marker is a lane broadcast, not a dependent memory load.
+// Call it with all 64 lanes active and wave-uniform arguments.
+__device__ __forceinline__ void ewah_expand_wave(const unsigned long long* __restrict__ in, int in_len, int W,
+                                                 unsigned long long* __restrict__ dst, int wpad, int lane) {
+    int idx = 0, o = 0, win_at = 0;
+    unsigned long long win = (lane < in_len) ? in[lane] : 0ULL;
+    while (idx < in_len && o < W) {
+        if (idx - win_at >= BSI_WAVE) {
+            win_at = idx;
+            win = (win_at + lane < in_len) ? in[win_at + lane] : 0ULL;
+        }
+        const int at = __builtin_amdgcn_readfirstlane(idx - win_at);
+        const unsigned lo = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(static_cast<unsigned>(win)), at));
+        const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(static_cast<unsigned>(win >> 32)), at));
+        ++idx;
+        const unsigned long long run_val = (lo & 1u) ? ~0ULL : 0ULL;
+        const unsigned run_len = (lo >> 1) | (hi << 31);   // bits 1..32 of the marker
+        const unsigned lit = hi >> 1;                      // bits 33..63
+        const int n_run = static_cast<int>(run_len < static_cast<unsigned>(W - o) ? run_len : static_cast<unsigned>(W - o));
+        for (int k = lane; k < n_run; k += BSI_WAVE) dst[o + k] = run_val;
+        o += n_run;
+        int n_lit = static_cast<int>(lit < static_cast<unsigned>(W - o) ? lit : static_cast<unsigned>(W - o));
+        if (n_lit > in_len - idx) n_lit = in_len - idx;
+        for (int k = lane; k < n_lit; k += BSI_WAVE) dst[o + k] = in[idx + k];
+        o += n_lit;
+        idx += n_lit;
+        if (static_cast<unsigned>(n_lit) < lit) break;     // clipped: the reference loop stops here too
+    }
+    for (int k = o + lane; k < wpad; k += BSI_WAVE) dst[k] = 0ULL;
+}
+
 }  // namespace bsi

@@ -1731,28 +1731,8 @@ __global__ __launch_bounds__(1024) void dot_mfma_stream_ewah_kernel(
     const unsigned long long* ksrc = B64 + static_cast<size_t>(tile) * chunks * (6 * 64) + lane;
 
     // ---- inline EWAH decode: slices round-robin over the waves
-    for (int s = wave; s < Sa; s += nwaves) {
-        const unsigned long long* in = comp + comp_off[s];
-        const int in_len = comp_len[s];
-        unsigned long long* dst = planes + static_cast<size_t>(s) * wpad;
-        int idx = 0, o = 0;
-        while (idx < in_len && o < W64) {
-            const unsigned long long rlw = in[idx++];
-            const unsigned long long run_val = (rlw & 1ULL) ? ~0ULL : 0ULL;
-            const unsigned int run_len = static_cast<unsigned int>((rlw >> 1) & 0xFFFFFFFFULL);
-            const unsigned int lit = static_cast<unsigned int>(rlw >> 33);
-            const int n_run = static_cast<int>(run_len < static_cast<unsigned int>(W64 - o) ? run_len : W64 - o);
-            for (int k = lane; k < n_run; k += BSI_WAVE) dst[o + k] = run_val;
-            o += n_run;
-            int n_lit = static_cast<int>(lit < static_cast<unsigned int>(W64 - o) ? lit : W64 - o);
-            if (n_lit > in_len - idx) n_lit = in_len - idx;
-            for (int k = lane; k < n_lit; k += BSI_WAVE) dst[o + k] = in[idx + k];
-            o += n_lit;
-            idx += n_lit;
-            if (static_cast<unsigned int>(n_lit) < lit) break;  // clipped: the reference loop stops here too
-        }
-        for (int k = o + lane; k < wpad; k += BSI_WAVE) dst[k] = 0ULL;
-    }
+    for (int s = wave; s < Sa; s += nwaves)
+        ewah_expand_wave(comp + comp_off[s], comp_len[s], W64, planes + static_cast<size_t>(s) * wpad, wpad, lane);
     __syncthreads();
 
     const bool chain = tid < 256;

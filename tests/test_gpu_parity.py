@@ -311,6 +311,83 @@ def test_ewah_kernels_match_oracle(hip, oracle, seed):
         np.testing.assert_array_equal(host_u64(one), words[4])
 
 
+def _codec_round_trip(hip, oracle, words, thr):
+    """flags -> size -> emit -> decode on the GPU against the oracle's encoder and decoder."""
+    L = hip.lib
+    S, W = words.shape
+    wd = dev(words)
+    flags_np = oracle.compress_flags(words, thr)
+    flags = dev(flags_np)
+    stream, off, lens = oracle.ewah_encode(words, flags_np)
+    sizes = torch.full((S,), -1, dtype=torch.int64, device="cuda")
+    hip.check(L.bsi_hip_ewah_size(wd.data_ptr(), S, W, flags.data_ptr(), sizes.data_ptr(), st()), "size")
+    offd = dev(off)
+    out = torch.full((max(stream.size, 1),), -1, dtype=torch.int64, device="cuda")
+    out_len = torch.full((S,), -1, dtype=torch.int32, device="cuda")
+    hip.check(L.bsi_hip_ewah_emit(wd.data_ptr(), S, W, flags.data_ptr(), offd.data_ptr(), out.data_ptr(),
+                                  out_len.data_ptr(), st()), "emit")
+    back = torch.full((S, W), -1, dtype=torch.int64, device="cuda")
+    hip.check(L.bsi_hip_ewah_decompress_batch(out.data_ptr(), offd.data_ptr(), out_len.data_ptr(), S, W,
+                                              back.data_ptr(), st()), "decode")
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(sizes.cpu().numpy(), lens)
+    np.testing.assert_array_equal(out_len.cpu().numpy(), lens)
+    np.testing.assert_array_equal(host_u64(out)[:stream.size], stream)
+    np.testing.assert_array_equal(host_u64(back), words)
+    return stream, off, lens
+
+
+@pytest.mark.parametrize("W", [1, 2, 63, 64, 65, 128, 129, 200, 1000])
+def test_ewah_codec_block_edges_and_long_marker_chains(hip, oracle, W):
+    """Slices whose runs and literal blocks straddle the 64-word blocks the encoder works in, and streams with far
+    more than 64 markers (the decoder's window of stream words is refilled many times)."""
+    rng = np.random.default_rng(W)
+    ones = np.uint64(0xFFFFFFFFFFFFFFFF)
+    rows = []
+    lit = rng.integers(1, 2 ** 63, size=W).astype(np.uint64)
+    rows.append(lit.copy())                                            # no clean word at all
+    rows.append(np.zeros(W, dtype=np.uint64))                          # one run
+    rows.append(np.full(W, ones))                                      # one run of ones
+    alt = lit.copy(); alt[::2] = 0; rows.append(alt)                   # clean / literal alternating: W / 2 markers
+    alt2 = np.zeros(W, dtype=np.uint64); alt2[1::2] = ones; rows.append(alt2)   # zero / one fills alternating: W markers
+    blk = lit.copy(); blk[60:70] = 0; blk[70:W // 2 + 70] = ones; rows.append(blk)  # runs across the block edge at 64
+    tail = lit.copy(); tail[-1:] = 0; rows.append(tail)                # a run as the last word
+    head = lit.copy(); head[0] = ones; rows.append(head)               # a run of one as the first word
+    sparse = np.zeros(W, dtype=np.uint64); sparse[rng.integers(0, W, size=max(1, W // 40))] = 1; rows.append(sparse)
+    words = np.stack(rows)
+    for thr in (1.0, 0.5, 0.0):     # every slice flagged, flagged by density, none flagged
+        _codec_round_trip(hip, oracle, words, thr)
+
+
+def test_ewah_decoder_bounds_match_the_oracle(hip, oracle):
+    """Hand-built and damaged streams: a run longer than the slice, literal counts beyond the stream's end, a stream
+    cut short, trailing words after the slice is full, an empty stream -- decoded as the oracle's restatement of the
+    reference decoder does (output clipped at W, input at its length, the rest zero)."""
+    L = hip.lib
+    W = 70
+
+    def marker(bit, run, lit):
+        return np.uint64(bit | (run << 1) | (lit << 33))
+
+    lits = np.arange(1, 200, dtype=np.uint64) * np.uint64(0x0101010101010101)
+    streams = [
+        np.array([marker(1, 500, 0)], dtype=np.uint64),                                   # run beyond W
+        np.concatenate([[marker(0, 3, 100)], lits[:20]]),                                 # literal count beyond the input
+        np.concatenate([[marker(0, 0, 10)], lits[:10], [marker(1, 5, 2)], lits[10:11]]),  # second block cut short
+        np.concatenate([[marker(0, 60, 10)], lits[:10], [marker(1, 9, 9)], lits[10:19]]),  # words left after W
+        np.zeros(0, dtype=np.uint64),                                                     # nothing at all
+        np.concatenate([[marker(0, 0, 0)], [marker(1, 2, 1)], lits[:1]]),                 # an empty marker first
+        np.concatenate([np.array([marker(0, 1, 0), marker(1, 1, 0)] * 35, dtype=np.uint64)]),  # 70 markers, no literal
+    ]
+    for strm in streams:
+        want = oracle.ewah_decompress(strm, W)
+        buf = dev(strm if strm.size else np.zeros(1, dtype=np.uint64))
+        one = torch.full((W,), -1, dtype=torch.int64, device="cuda")
+        hip.check(L.bsi_hip_ewah_decompress(buf.data_ptr(), int(strm.size), W, one.data_ptr(), st()), "decode1")
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(host_u64(one), want)
+
+
 def test_hybrid_query_builder(ops, oracle):
     x = np.maximum(_inputs(1, 8192, 4), 0)[0]  # ReLU: sign plane all zero
     cap, mem, S, W = ops.build_bsi_query_cuda_hybrid(torch.from_numpy(x).cuda(), 2, 0.5)
