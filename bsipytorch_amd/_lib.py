@@ -62,6 +62,9 @@ PROTOTYPES = {
     "bsi_hip_linear": [_vp, _i, _i64, _i64, _i, _i, _i, _vp, _sz, _vp, _i, _vp, _i, _i64, _f, _i64, _vp, _vp, _i, _vp,
                        _sz, _vp],
     "bsi_hip_dot_ewah_query": [_vp, _vp, _vp, _i, _i, _vp, _i, _vp, _vp, _i, _i64, _f, _vp, _vp, _vp],
+    "bsi_hip_dot_ewah_batch_workspace_bytes": [_i64, _i],
+    "bsi_hip_dot_ewah_batch": [_vp, _vp, _vp, _i, _i, _vp, _i, _vp, _i, _vp, _i, _i64, _i64, _f, _i64, _vp, _vp, _vp, _vp,
+                               _sz, _vp],
     "bsi_hip_planes_to_int8_digits": [_vp, _i64, _i, _i, _vp, _vp],
     "bsi_hip_dot_digits_workspace_bytes": [_i64, _i, _i64, _i],
     "bsi_hip_dot_digits": [_vp, _i, _vp, _i, _vp, _i, _i, _vp, _i, _i, _i64, _i64, _vp, _f, _i64, _vp, _vp, _vp,
@@ -83,6 +86,7 @@ _RESTYPES = {
     "bsi_hip_version": ctypes.c_char_p,
     "bsi_hip_last_error": ctypes.c_char_p,
     "bsi_hip_dot_workspace_bytes": _sz,
+    "bsi_hip_dot_ewah_batch_workspace_bytes": _sz,
     "bsi_hip_linear_workspace_bytes": _sz,
     "bsi_hip_dot_digits_workspace_bytes": _sz,
     "bsi_hip_int8_tiled_bytes": _sz,

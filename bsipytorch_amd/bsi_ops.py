@@ -198,6 +198,28 @@ class PrebuiltBSIQueryBatchCUDA(_Capsule):
         self.mem_bytes = 0
 
 
+class PrebuiltBSIQueryBatchHybridCUDA(_Capsule):
+    """A query batch whose slices are kept as EWAH streams only (the batched form of the hybrid query of
+    bsi_cuda.cpp:386-431; the reference has no batched one): stream q * Sa + s is slice s of row q."""
+
+    name = "PrebuiltBSIQueryBatchHybridCUDA"
+
+    def __init__(self):
+        self.comp_words: torch.Tensor = None     # int64 [total]: all streams, back to back
+        self.comp_off: torch.Tensor = None       # int64 [Q * Sa]
+        self.comp_len: torch.Tensor = None       # int32 [Q * Sa]
+        self.flags: torch.Tensor = None          # int32 [Q * Sa]: 1 = the slice was run-length encoded
+        self.slice_weights: torch.Tensor = None  # [Q, Sa] float32
+        self.chunk_scales: Optional[torch.Tensor] = None
+        self.row_scales: Optional[torch.Tensor] = None
+        self.Sa = 0
+        self.W = 0
+        self.decimals = 0
+        self.Q = 0
+        self.mem_bytes = 0                       # bytes of the streams (+ offsets, lengths, scales)
+        self.verbatim_bytes = 0                  # bytes the same planes take verbatim
+
+
 class PrebuiltBSIQueryCUDA(_Capsule):
     """bsi_cuda.cpp:183-192: one query row (a view into its batch)."""
 
@@ -589,6 +611,60 @@ def build_bsi_query_cuda_hybrid(q: torch.Tensor, decimal_places: int, compress_t
     h.comp_words, h.comp_off, h.comp_len = comp_words, comp_off, comp_len
     h.mem_bytes = comp_words.numel() * 8 + decoded.numel() * 8
     return h, int(h.mem_bytes), h.S, h.W
+
+
+def build_bsi_queries_cuda_batch_hybrid(q2d: torch.Tensor, decimal_places: int, compress_threshold: float = 0.2):
+    """The batched hybrid query form: the fixed-bit build of build_bsi_queries_cuda_batch_packed, then every slice of
+    every row EWAH-encoded at ``compress_threshold`` (density flag, size pass, scan, emit pass, as
+    bsi_vector_cuda.cpp:896-951 does for the one query of build_bsi_query_cuda_hybrid) -- and only the streams are
+    kept: the dot decodes them in its load stage.  Not in the reference, whose only hybrid form is one query that it
+    decodes again right after encoding it (bsi_cuda.cpp:386-431)."""
+    _check(q2d.dim() == 2, "q must be 2D [Q, d]")
+    f = _flags()
+    _check(2 <= f["bits_q"] <= 8, "the hybrid query batch needs fixed-bit queries of 2 to 8 bits")
+    b = _build_query_batch(q2d, int(decimal_places))
+    Q, Sa, W = b.words.shape
+    _check(Q > 0, "Empty query batch")
+    comp_words, comp_off, comp_len, flags = ewah_compress_slices(b.words.view(Q * Sa, W), float(compress_threshold))
+    h = PrebuiltBSIQueryBatchHybridCUDA()
+    h.comp_words, h.comp_off, h.comp_len, h.flags = comp_words, comp_off, comp_len, flags
+    h.slice_weights, h.chunk_scales, h.row_scales = b.slice_weights, b.chunk_scales, b.row_scales
+    h.Sa, h.W, h.decimals, h.Q = int(Sa), int(W), b.decimals, int(Q)
+    scale_bytes = (b.chunk_scales.numel() if b.chunk_scales is not None else b.row_scales.numel()) * 4
+    h.mem_bytes = comp_words.numel() * 8 + comp_off.numel() * 8 + comp_len.numel() * 4 + scale_bytes
+    h.verbatim_bytes = b.words.numel() * 8 + scale_bytes
+    return h
+
+
+def _dot_ewah_batch(qb: "PrebuiltBSIQueryBatchHybridCUDA", keys: "PrebuiltBSIKeysCUDA", bias=None, chunk_ints=None):
+    """bsi_hip_dot_ewah_batch on a hybrid query batch -> (out [Q, R] float32, ns)."""
+    f = _flags()
+    Q, R, Sa, W = qb.Q, keys.num_keys, qb.Sa, qb.W
+    _check(2 <= keys.Sb <= 8 and keys.fixed, "the hybrid query batch needs fixed-bit keys of 2 to 8 bits")
+    if qb.chunk_scales is not None and qb.chunk_scales.numel() > 0:
+        _check(keys.W % 4 == 0 and qb.chunk_scales.shape[1] == keys.W // 4, "Chunk scale stride mismatch")
+        scales, stride = qb.chunk_scales, int(qb.chunk_scales.shape[1])
+    else:
+        scales, stride = qb.row_scales, 1
+    dev = qb.comp_words.device
+    out = torch.empty((Q, R), dtype=torch.float32, device=dev)
+    kptr, klayout = key_operand(keys, Q, Sa, _lib.CORE_MFMA)
+    ws_bytes = int(lib.bsi_hip_dot_ewah_batch_workspace_bytes(Q, W))
+    ws = _get_workspace(ws_bytes, dev)
+    prof = f["profile"]
+    if prof:
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+    check(lib.bsi_hip_dot_ewah_batch(qb.comp_words.data_ptr(), qb.comp_off.data_ptr(), qb.comp_len.data_ptr(), Sa, W,
+                                     scales.data_ptr(), stride, kptr, klayout, keys.slice_weights.data_ptr(), keys.Sb, R, Q,
+                                     _scale_inv(qb.decimals, keys.decimals), R, _ptr(bias), out.data_ptr(), _ptr(chunk_ints),
+                                     _ptr(ws), ws_bytes, _stream()), "bsi_hip_dot_ewah_batch")
+    ns = 0
+    if prof:
+        e1.record()
+        e1.synchronize()
+        ns = int(e0.elapsed_time(e1) * 1.0e6)
+    return out, ns
 
 
 def _install_fixed_key_planes(h: "PrebuiltBSIKeysCUDA", words: torch.Tensor) -> None:
@@ -1095,6 +1171,17 @@ def batch_dot_product_multiquery_cuda_batch_caps(query_batch_cap, keyset_cuda_ca
     row in the same launch, rounded as ``out + bias`` would be.  ``warm_keys`` (not in the reference either): the
     keyset the next dot will use; this launch also reads it once so that it is cache-resident by then."""
     keys = _capsule(keyset_cuda_cap, PrebuiltBSIKeysCUDA, "Invalid CUDA keys capsule")
+    if isinstance(query_batch_cap, PrebuiltBSIQueryBatchHybridCUDA):
+        # the batched hybrid form: EWAH streams, decoded in the dot's load stage
+        hb = query_batch_cap
+        _check(hb.W == keys.W, "Word count mismatch between query batch and keys")
+        _check(keys.num_keys > 0, "Empty keys")
+        _check(hb.decimals == keys.decimals, f"Decimal mismatch between queries and keys: q={hb.decimals} k={keys.decimals}")
+        if bias is not None:
+            _check(bias.is_cuda and bias.dtype == torch.float32 and bias.dim() == 1 and bias.numel() == keys.num_keys
+                   and bias.is_contiguous(), "bias must be a contiguous float32 CUDA tensor of [R]")
+        out, ns = _dot_ewah_batch(hb, keys, bias=bias)
+        return _dot_result(out, ns, hb.Q, keys.num_keys)
     qb = _capsule(query_batch_cap, PrebuiltBSIQueryBatchCUDA, "Invalid CUDA query-batch capsule")
     _check(qb.words is not None and qb.slice_weights is not None, "Query batch tensors are not defined")
     _check(qb.words.is_cuda and qb.slice_weights.is_cuda, "Query batch tensors must be CUDA tensors")

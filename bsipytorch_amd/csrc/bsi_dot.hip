@@ -1699,28 +1699,51 @@ __global__ __launch_bounds__(1024) void dot_mfma_stream_fused_kernel(
     }
 }
 
-// ------------------------------------------------------------------ one EWAH-compressed query, decode inline
+// ------------------------------------------------------------------ EWAH-compressed queries, decode inline
 //
-// The hybrid query form keeps each of its Sa slices as an EWAH stream ([marker][literals...],
+// The hybrid query form keeps each of a query's Sa slices as an EWAH stream ([marker][literals...],
 // marker = run_bit | run_len << 1 | literal_count << 33; bsi_cuda_kernels_ewah.cuh:5-33 is the
 // decoder this follows, including its bounds: output clipped at W words, input at the stream's
-// length, the rest zero).  This kernel is the few-rows kernel for that one query with the decode
-// folded into its load stage: every workgroup first expands the streams into bit planes in LDS
-// (wave s walks the markers of slice s; its lanes write a run or copy a literal block in
-// parallel), then recombines the planes of each chunk into the int8 MFMA operand in registers,
-// exactly as it does for the key planes it streams from HBM.
+// length, the rest zero).  This kernel is the few-rows kernel for up to 16 such queries per workgroup
+// (stream q * Sa + s is slice s of query q) with the decode folded into its load stage: every workgroup
+// first expands the streams into bit planes in LDS (a wave per stream: ewah_expand_wave), then
+// recombines the planes of each chunk into the int8 MFMA operand in registers, exactly as it does for
+// the key planes it streams from HBM.  A slice whose stream says "all zero" (one marker, a zero run
+// over the whole slice: the sign plane of ReLU'd activations, the high planes of small values) is not
+// expanded at all: its plane reads as zero without touching LDS.
+constexpr int kEwahQueriesPerGroup = 16;
+__host__ __device__ inline int ewah_stream_stride(int wpad) { return wpad + 1; }  // odd stride: queries spread over the banks
+// bytes of the plane region of `group` queries (a multiple of 16: the accumulators behind it are stored 16 bytes at a time)
+__host__ __device__ inline size_t ewah_plane_region(int group, int Sa, int wpad) {
+    return (static_cast<size_t>(group) * Sa * ewah_stream_stride(wpad) * 8 + 15) & ~static_cast<size_t>(15);
+}
+
+// Whether the stream is the encoder's form of an all-zero slice of W words (every lane gets the answer).
+__device__ __forceinline__ bool ewah_stream_is_zero(const unsigned long long* __restrict__ in, int in_len, int W) {
+    if (in_len == 0) return true;
+    if (in_len != 1) return false;
+    const unsigned long long m = in[0];
+    return (m & 1ULL) == 0ULL && ((m >> 1) & 0xFFFFFFFFULL) >= static_cast<unsigned long long>(W);
+}
+
 template <bool kInts>
 __global__ __launch_bounds__(1024) void dot_mfma_stream_ewah_kernel(
     const unsigned long long* __restrict__ comp, const long long* __restrict__ comp_off,
     const int* __restrict__ comp_len, int Sa, int W64, const float* __restrict__ qscale, int qscale_stride,
     const unsigned long long* __restrict__ B64,  // tiled key planes, Sb = 6
-    const float* __restrict__ Bw, int chunks, int pass_chunks, int64_t R, int down_shift, float scale_inv,
-    float* __restrict__ out, int* __restrict__ chunk_ints) {
+    const float* __restrict__ Bw, int chunks, int pass_chunks, int64_t R, int64_t Q, int group, int down_shift,
+    float scale_inv, int64_t R_total, const float* __restrict__ bias, float* __restrict__ out,
+    int* __restrict__ chunk_ints) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    // [Sa][4 * chunks] query plane words (zero-padded to whole chunks), then the chunk accumulators
+    // group = queries per workgroup (min(Q, 16)); LDS: [group][Sa] streams of ewah_stream_stride(4 * chunks) plane
+    // words, one presence byte per stream (128 bytes), then the chunk accumulators
+    const int wpad = chunks * 4, sstride = ewah_stream_stride(wpad);
+    const int64_t q0 = static_cast<int64_t>(blockIdx.y) * kEwahQueriesPerGroup;
+    const int nq = static_cast<int>((Q - q0) < kEwahQueriesPerGroup ? (Q - q0) : kEwahQueriesPerGroup);
+    const int nstreams = nq * Sa;
     unsigned long long* planes = reinterpret_cast<unsigned long long*>(smem);
-    const int wpad = chunks * 4;
-    int* ints = reinterpret_cast<int*>(smem + static_cast<size_t>(Sa) * wpad * 8);
+    unsigned char* present = smem + ewah_plane_region(group, Sa, wpad);
+    int* ints = reinterpret_cast<int*>(present + 128);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -1730,18 +1753,32 @@ __global__ __launch_bounds__(1024) void dot_mfma_stream_ewah_kernel(
     const int64_t tile = blockIdx.x;
     const unsigned long long* ksrc = B64 + static_cast<size_t>(tile) * chunks * (6 * 64) + lane;
 
-    // ---- inline EWAH decode: slices round-robin over the waves
-    for (int s = wave; s < Sa; s += nwaves)
-        ewah_expand_wave(comp + comp_off[s], comp_len[s], W64, planes + static_cast<size_t>(s) * wpad, wpad, lane);
+    // ---- inline EWAH decode: the group's streams round-robin over the waves
+    for (int s = wave; s < nstreams; s += nwaves) {
+        const unsigned long long* in = comp + comp_off[q0 * Sa + s];
+        const int in_len = comp_len[q0 * Sa + s];
+        const bool zero = ewah_stream_is_zero(in, in_len, W64);
+        if (lane == 0) present[s] = zero ? 0 : 1;
+        if (!zero) ewah_expand_wave(in, in_len, W64, planes + static_cast<size_t>(s) * sstride, wpad, lane);
+    }
     __syncthreads();
 
     const bool chain = tid < 256;
     const int ckey = tid & 15, cn = (tid >> 4) & 15;
     const int64_t cr = tile * 16 + ckey;
-    const bool cvalid = chain && cn == 0 && cr < R;
+    const bool cvalid = chain && cn < nq && cr < R;
     const float down = __uint_as_float(static_cast<uint32_t>(127 - down_shift) << 23);
     const int sstep = (qscale_stride == 1) ? 0 : 1;
+    const float* myscale = qscale + (q0 + (cn < nq ? cn : 0)) * qscale_stride;
     float accf = 0.0f;
+    // which of the lane's query's planes hold anything (bit t of the mask: row t of the 8 x 8 transposes)
+    unsigned have = 0;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+        const int j = t - (8 - Sa);
+        if (ln < nq && j >= 0 && present[ln * Sa + j]) have |= 1u << t;
+    }
+    const unsigned long long* myplanes = planes + static_cast<size_t>(ln < nq ? ln : 0) * Sa * sstride;
 
     for (int p0 = 0; p0 < chunks; p0 += pass_chunks) {
         const int pend = (p0 + pass_chunks < chunks) ? p0 + pass_chunks : chunks;
@@ -1752,13 +1789,12 @@ __global__ __launch_bounds__(1024) void dot_mfma_stream_ewah_kernel(
                 const unsigned long long w = ksrc[(static_cast<size_t>(c) * 6 + j) * 64];
                 kc[j] = make_uint2(static_cast<uint32_t>(w), static_cast<uint32_t>(w >> 32));
             }
-            // the query operand of this chunk from the decoded planes (column 0 of the MFMA; the other 15 stay zero)
+            // the query operand of this chunk from the decoded planes: MFMA column ln is query q0 + ln
             uint32_t qlo[8], qhi[8];
 #pragma unroll
             for (int t = 0; t < 8; ++t) {
                 const int j = t - (8 - Sa);
-                const unsigned long long w =
-                    (ln == 0 && j >= 0) ? planes[static_cast<size_t>(j) * wpad + c * 4 + lg] : 0ULL;
+                const unsigned long long w = ((have >> t) & 1u) ? myplanes[static_cast<size_t>(j) * sstride + c * 4 + lg] : 0ULL;
                 qlo[t] = static_cast<uint32_t>(w);
                 qhi[t] = static_cast<uint32_t>(w >> 32);
             }
@@ -1784,14 +1820,58 @@ __global__ __launch_bounds__(1024) void dot_mfma_stream_ewah_kernel(
         }
         __syncthreads();
         if (cvalid) {
-            accf = chain_chunks(accf, p0, pend, down, [&](int cc) { return ints[(cc - p0) * 256 + ckey]; },  // query 0, key ckey
-                                [&](int cc) { return qscale[cc * sstep]; });
+            accf = chain_chunks(accf, p0, pend, down, [&](int cc) { return ints[(cc - p0) * 256 + cn * 16 + ckey]; },
+                                [&](int cc) { return myscale[cc * sstep]; });
             if (kInts)
-                for (int cc = p0; cc < pend; ++cc) chunk_ints[cr * chunks + cc] = ints[(cc - p0) * 256 + ckey] >> down_shift;
+                for (int cc = p0; cc < pend; ++cc)
+                    chunk_ints[((q0 + cn) * R + cr) * chunks + cc] = ints[(cc - p0) * 256 + cn * 16 + ckey] >> down_shift;
         }
         if (pend < chunks) __syncthreads();
     }
-    if (cvalid) out[cr] = (accf * Bw[cr * 6]) * scale_inv;
+    if (cvalid) {
+        float v = (accf * Bw[cr * 6]) * scale_inv;
+        if (bias != nullptr) v = v + bias[cr];
+        out[(q0 + cn) * R_total + cr] = v;
+    }
+}
+
+// EWAH streams of a whole query batch -> the int8 query image the compute-bound dot contracts (value << (8 - Sa),
+// in-chunk byte order of planes_to_int8_kernel): one workgroup per query row expands the row's Sa streams into LDS
+// (a wave per stream, all-zero slices skipped) and recombines them 32 elements per thread.  The verbatim planes
+// never exist in memory.
+__global__ __launch_bounds__(256) void ewah_streams_to_int8_kernel(const unsigned long long* __restrict__ comp,
+                                                                    const long long* __restrict__ comp_off,
+                                                                    const int* __restrict__ comp_len, int Sa, int W64,
+                                                                    int chunks, uint32_t* __restrict__ out32) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int wpad = chunks * 4;
+    unsigned long long* planes = reinterpret_cast<unsigned long long*>(smem);  // [Sa][wpad]
+    unsigned char* present = smem + static_cast<size_t>(Sa) * wpad * 8;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int64_t row = blockIdx.x;
+    for (int s = wave; s < Sa; s += 4) {
+        const unsigned long long* in = comp + comp_off[row * Sa + s];
+        const int in_len = comp_len[row * Sa + s];
+        const bool zero = ewah_stream_is_zero(in, in_len, W64);
+        if (lane == 0) present[s] = zero ? 0 : 1;
+        if (!zero) ewah_expand_wave(in, in_len, W64, planes + static_cast<size_t>(s) * wpad, wpad, lane);
+    }
+    __syncthreads();
+    const uint32_t* planes32 = reinterpret_cast<const uint32_t*>(planes);
+    const int cols = chunks * 8;
+    for (int col = tid; col < cols; col += 256) {
+        uint32_t y[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const int j = t - (8 - Sa);
+            y[t] = (j >= 0 && present[j]) ? planes32[static_cast<size_t>(j) * wpad * 2 + col] : 0u;
+        }
+        transpose8x8(y);
+        uint4* dst = reinterpret_cast<uint4*>(out32 + (static_cast<size_t>(row) * cols + col) * 8);
+        dst[0] = make_uint4(y[0], y[1], y[2], y[3]);
+        dst[1] = make_uint4(y[4], y[5], y[6], y[7]);
+    }
 }
 
 // ------------------------------------------------------------------ VALU popcount core (Sa = 7, Sb = 6 shape templated)
@@ -2640,6 +2720,40 @@ extern "C" int bsi_hip_linear_few_rows(const void* x, int dtype, int64_t Q, int6
     return BSI_OK;
 }
 
+// Launch of the inline-decode kernel for Q queries (groups of 16 along grid.y), or BSI_ERR_UNSUPPORTED when the
+// planes of a group do not fit LDS.
+static int launch_stream_ewah(const uint64_t* comp_words, const int64_t* comp_off, const int32_t* comp_len, int Sa, int W64,
+                              const float* A_chunk_scales, int A_scale_stride, const uint64_t* B_tiled, const float* Bw,
+                              int64_t R, int64_t Q, float scale_inv, int64_t R_total, const float* bias, float* out,
+                              int32_t* chunk_ints, hipStream_t st) {
+    const int chunks = (W64 + 3) / 4;
+    const int group = static_cast<int>(Q < kEwahQueriesPerGroup ? Q : kEwahQueriesPerGroup);
+    const size_t plane_bytes = ewah_plane_region(group, Sa, chunks * 4) + 128;
+    if (plane_bytes > 120 * 1024)
+        return fail(BSI_ERR_UNSUPPORTED, "%d words per slice do not fit the LDS plane buffer of the inline-decode kernel", W64);
+    int pass_chunks = static_cast<int>((kStreamLdsInts * sizeof(int) < 156 * 1024 - plane_bytes
+                                            ? kStreamLdsInts * sizeof(int)
+                                            : 156 * 1024 - plane_bytes) / 1024);
+    if (pass_chunks > chunks) pass_chunks = chunks;
+    const size_t lds = plane_bytes + static_cast<size_t>(pass_chunks) * 1024;
+    int waves = chunks < 16 ? chunks : 16;
+    if (waves < 4) waves = 4;
+    const dim3 grid(static_cast<unsigned>((R + 15) / 16), static_cast<unsigned>((Q + kEwahQueriesPerGroup - 1) / kEwahQueriesPerGroup));
+    static LdsOptIn once0;
+    lds_opt_in(once0, reinterpret_cast<const void*>(&dot_mfma_stream_ewah_kernel<true>), 160 * 1024);
+    static LdsOptIn once1;
+    lds_opt_in(once1, reinterpret_cast<const void*>(&dot_mfma_stream_ewah_kernel<false>), 160 * 1024);
+    const int down_shift = 16 - Sa - 6;
+#define BSI_EWAH_ARGS reinterpret_cast<const unsigned long long*>(comp_words), reinterpret_cast<const long long*>(comp_off), \
+                      comp_len, Sa, W64, A_chunk_scales, A_scale_stride, reinterpret_cast<const unsigned long long*>(B_tiled), \
+                      Bw, chunks, pass_chunks, R, Q, group, down_shift, scale_inv, R_total, bias, out, chunk_ints
+    if (chunk_ints) hipLaunchKernelGGL((dot_mfma_stream_ewah_kernel<true>), grid, dim3(waves * 64), lds, st, BSI_EWAH_ARGS);
+    else hipLaunchKernelGGL((dot_mfma_stream_ewah_kernel<false>), grid, dim3(waves * 64), lds, st, BSI_EWAH_ARGS);
+#undef BSI_EWAH_ARGS
+    BSI_LAUNCH_CHECK("dot_mfma_stream_ewah_kernel");
+    return BSI_OK;
+}
+
 extern "C" int bsi_hip_dot_ewah_query(const uint64_t* comp_words, const int64_t* comp_off, const int32_t* comp_len,
                                       int Sa, int W64, const float* A_chunk_scales, int A_scale_stride,
                                       const uint64_t* B_tiled, const float* Bw, int Sb, int64_t R, float scale_inv,
@@ -2652,37 +2766,53 @@ extern "C" int bsi_hip_dot_ewah_query(const uint64_t* comp_words, const int64_t*
     const int chunks = (W64 + 3) / 4;
     BSI_REQUIRE(A_scale_stride == chunks || A_scale_stride == 1,
                 "chunk scale stride mismatch: got %d expected %d (or 1 for a row scale)", A_scale_stride, chunks);
-    const size_t plane_bytes = static_cast<size_t>(Sa) * chunks * 4 * 8;
-    if (plane_bytes > 96 * 1024)
-        return fail(BSI_ERR_UNSUPPORTED, "query of %d words per slice does not fit the LDS plane buffer", W64);
-    int pass_chunks = static_cast<int>((kStreamLdsInts * sizeof(int) < 150 * 1024 - plane_bytes
-                                            ? kStreamLdsInts * sizeof(int)
-                                            : 150 * 1024 - plane_bytes) / 1024);
-    if (pass_chunks > chunks) pass_chunks = chunks;
-    const size_t lds = plane_bytes + static_cast<size_t>(pass_chunks) * 1024;
-    int waves = chunks < 16 ? chunks : 16;
-    if (waves < 4) waves = 4;
+    return launch_stream_ewah(comp_words, comp_off, comp_len, Sa, W64, A_chunk_scales, A_scale_stride, B_tiled, Bw, R, 1,
+                              scale_inv, R, nullptr, out, chunk_ints, as_stream(stream));
+}
+
+extern "C" size_t bsi_hip_dot_ewah_batch_workspace_bytes(int64_t Q, int W64) {
+    return bsi_hip_dot_workspace_bytes(Q, W64, BSI_CORE_MFMA);
+}
+
+extern "C" int bsi_hip_dot_ewah_batch(const uint64_t* comp_words, const int64_t* comp_off, const int32_t* comp_len, int Sa,
+                                      int W64, const float* A_chunk_scales, int A_scale_stride, const uint64_t* B,
+                                      int b_layout, const float* Bw, int Sb, int64_t R, int64_t Q, float scale_inv,
+                                      int64_t R_total, const float* bias, float* out, int32_t* chunk_ints, void* workspace,
+                                      size_t workspace_bytes, void* stream) {
+    BSI_REQUIRE(Q >= 0 && R >= 0 && W64 >= 1 && R_total >= R, "bad shape");
+    BSI_REQUIRE(Sa >= 2 && Sa <= 8 && Sb >= 2 && Sb <= 8, "the matrix-core dot needs Sa, Sb in [2, 8] (got %d, %d)", Sa, Sb);
+    if (Q == 0 || R == 0) return BSI_OK;
+    BSI_REQUIRE(comp_words && comp_off && comp_len && A_chunk_scales && B && Bw && out, "null pointer");
+    const int chunks = (W64 + 3) / 4;
+    BSI_REQUIRE(A_scale_stride == chunks || A_scale_stride == 1,
+                "chunk scale stride mismatch: got %d expected %d (or 1 for row scales)", A_scale_stride, chunks);
     hipStream_t st = as_stream(stream);
-    const dim3 grid(static_cast<unsigned>((R + 15) / 16));
-    static LdsOptIn once0;
-    lds_opt_in(once0, reinterpret_cast<const void*>(&dot_mfma_stream_ewah_kernel<true>), 160 * 1024);
-    static LdsOptIn once1;
-    lds_opt_in(once1, reinterpret_cast<const void*>(&dot_mfma_stream_ewah_kernel<false>), 160 * 1024);
-    const int down_shift = 16 - Sa - Sb;
-    if (chunk_ints)
-        hipLaunchKernelGGL((dot_mfma_stream_ewah_kernel<true>), grid, dim3(waves * 64), lds, st,
-                           reinterpret_cast<const unsigned long long*>(comp_words),
-                           reinterpret_cast<const long long*>(comp_off), comp_len, Sa, W64, A_chunk_scales,
-                           A_scale_stride, reinterpret_cast<const unsigned long long*>(B_tiled), Bw, chunks,
-                           pass_chunks, R, down_shift, scale_inv, out, chunk_ints);
-    else
-        hipLaunchKernelGGL((dot_mfma_stream_ewah_kernel<false>), grid, dim3(waves * 64), lds, st,
-                           reinterpret_cast<const unsigned long long*>(comp_words),
-                           reinterpret_cast<const long long*>(comp_off), comp_len, Sa, W64, A_chunk_scales,
-                           A_scale_stride, reinterpret_cast<const unsigned long long*>(B_tiled), Bw, chunks,
-                           pass_chunks, R, down_shift, scale_inv, out, chunk_ints);
-    BSI_LAUNCH_CHECK("dot_mfma_stream_ewah_kernel");
-    return BSI_OK;
+    // A few rows against the packed planes: the call is bound by streaming the keys once, and each workgroup can
+    // afford to expand the queries itself -- the decode is part of the dot kernel's load stage.
+    const int64_t group = Q < kEwahQueriesPerGroup ? Q : kEwahQueriesPerGroup;
+    if (Q <= kStreamMaxQ && b_layout == BSI_LAYOUT_TILED16 && Sb == 6 &&
+        ewah_plane_region(static_cast<int>(group), Sa, chunks * 4) + 128 <= 120 * 1024)
+        return launch_stream_ewah(comp_words, comp_off, comp_len, Sa, W64, A_chunk_scales, A_scale_stride, B, Bw, R, Q,
+                                  scale_inv, R_total, bias, out, chunk_ints, st);
+    // Many rows: every key-tile workgroup of the compute-bound kernel reads the whole query tile, so expanding the
+    // streams there would repeat the decode and the plane -> int8 recombination once per key tile (32 times at
+    // Q512 x R2048).  The call's load stage therefore runs once, as a launch of its own: streams -> int8 query
+    // image in the workspace (the verbatim planes are never materialised), then the dot on that image.
+    const size_t need = bsi_hip_dot_ewah_batch_workspace_bytes(Q, W64);
+    BSI_REQUIRE(workspace != nullptr && workspace_bytes >= need, "%zu bytes of workspace needed for the int8 query image (got %zu)",
+                need, workspace_bytes);
+    BSI_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 15) == 0, "workspace must be 16-byte aligned");
+    const size_t lds = static_cast<size_t>(Sa) * chunks * 4 * 8 + 64;
+    if (lds > 150 * 1024)
+        return fail(BSI_ERR_UNSUPPORTED, "%d words per slice do not fit the LDS plane buffer of the stream decoder", W64);
+    static LdsOptIn once;
+    lds_opt_in(once, reinterpret_cast<const void*>(&ewah_streams_to_int8_kernel), 160 * 1024);
+    hipLaunchKernelGGL(ewah_streams_to_int8_kernel, dim3(static_cast<unsigned>(Q)), dim3(256), lds, st,
+                       reinterpret_cast<const unsigned long long*>(comp_words), reinterpret_cast<const long long*>(comp_off),
+                       comp_len, Sa, W64, chunks, static_cast<uint32_t*>(workspace));
+    BSI_LAUNCH_CHECK("ewah_streams_to_int8_kernel");
+    return dot_with_bias(nullptr, static_cast<const int8_t*>(workspace), A_chunk_scales, A_scale_stride, Sa, W64, B, b_layout,
+                         Bw, Sb, R, Q, scale_inv, R_total, out, chunk_ints, BSI_CORE_MFMA, nullptr, 0, stream, bias);
 }
 
 template <int WB, bool kTiled>

@@ -292,6 +292,26 @@ int bsi_hip_dot_ewah_query(const uint64_t* comp_words, const int64_t* comp_off, 
                            const float* Bw, int Sb, int64_t R, float scale_inv, float* out, int32_t* chunk_ints,
                            void* stream);
 
+/* The same dot for a BATCH of queries kept as EWAH streams (no counterpart in the reference, which compresses the
+ * single hybrid query only and feeds verbatim words to its kernels, bsi_cuda.cpp:386-431): stream q * Sa + s, at
+ * comp_words + comp_off[q * Sa + s] with comp_len[q * Sa + s] words, is slice s of query q, encoded as
+ * bsi_hip_ewah_emit writes it and decoded with the semantics of ewah_decompress_kernel
+ * (bsi_cuda_kernels_ewah.cuh:5-33).  The result is that of bsi_hip_dot_bias on the decoded planes, bit for bit.
+ * The decode is the call's load stage, never a pass that writes verbatim planes:
+ *   - at most 32 rows on tiled16 6-plane keys (the bandwidth-bound regime): inside the dot kernel -- every workgroup
+ *     expands its 16 queries' streams into LDS planes, then streams the key planes once;
+ *   - otherwise: one launch turns the streams straight into the int8 query image in `workspace`
+ *     (bsi_hip_dot_ewah_batch_workspace_bytes), a second one contracts it.  (Every key-tile workgroup of the
+ *     compute-bound kernel reads the whole query tile; decoding there would repeat the work once per key tile.)
+ * Slices whose stream is the encoder's all-zero form are skipped, not expanded.  B / b_layout / Bw / out /
+ * chunk_ints / bias as for bsi_hip_dot and bsi_hip_dot_bias; Sa, Sb in [2, 8]. */
+size_t bsi_hip_dot_ewah_batch_workspace_bytes(int64_t Q, int W64);
+int bsi_hip_dot_ewah_batch(const uint64_t* comp_words, const int64_t* comp_off, const int32_t* comp_len, int Sa, int W64,
+                           const float* A_chunk_scales, int A_scale_stride, const uint64_t* B, int b_layout,
+                           const float* Bw, int Sb, int64_t R, int64_t Q, float scale_inv, int64_t R_total,
+                           const float* bias, float* out, int32_t* chunk_ints, void* workspace, size_t workspace_bytes,
+                           void* stream);
+
 /* Weighted-slice dot for operands with arbitrary per-slice float weights (decimal-mode operands, whose
  * slice count follows the data, or fixed-bit operands without chunk scales):
  *   out[q, idx[r]] = float(sum_{i,j,w} popcount(A[q,i,w] & B[r,j,w]) * double(Aw[q,i] * Bw[r,j])) * scale_inv
