@@ -1,11 +1,15 @@
 """Benchmark of the BSI fixed76 chunk-scale dot on one MI355X.
 
-    python bench.py [--gpus 1] [--steps 50] [--warmup 10] [--core auto|mfma|valu] [--no-cpu]
+    python bench.py [--gpus 1] [--steps 50] [--warmup 10] [--core auto|mfma|valu] [--no-cpu] [--no-extras]
 
 Workload: the FC1-like configuration (queries fp32 Q=512 x D=2048 ~N(0,1) with 0.1% of the columns
 scaled x20, keys fp32 R=8192 x D=2048 ~N(0,0.02), decimal_places=2, compress_threshold=0.5, Sa=7,
 Sb=6, chunk scales), synthetic, seed 123.  A step is one dot over the prebuilt query and key planes
-(resident in HBM).  Prints ONE JSON line.
+(resident in HBM).  Prints ONE JSON line.  Its headline fields describe that workload; "other_configs" in the same
+line carries the other benchmark configurations, each bounded to a few seconds: the FC2-like dot (also with the
+queries kept as EWAH streams), the OPT-6.7B layer shapes at one query row on resident and on rotating keysets (GB/s
+on the packed key planes), and the OPT-1.3B-shaped prefill (tokens/s eager and as a replayed HIP graph, share of the
+dot).
 """
 import argparse
 import ctypes
@@ -21,10 +25,180 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 MFMA_I8_PEAK_TOPS = 5000.0     # MI355X published dense int8
 Q, R, D = 512, 8192, 2048
-# HBM bytes per launch of the dot kernel on this workload, from rocprofv3 FETCH_SIZE and WRITE_SIZE runs scaled by a
-# 256 MiB copy (profiles/dot_mfma_i8_kernel_fc1_Q512_R8192_D2048_hbm_traffic.txt); counters cannot be read in-process
+# HBM bytes per launch of the dot kernel on this workload: an OFFLINE figure, from rocprofv3 FETCH_SIZE and WRITE_SIZE
+# runs of this script scaled by a 256 MiB copy (profiles/dot_mfma_i8_kernel_fc1_Q512_R8192_D2048_hbm_traffic.txt).
+# Hardware counters cannot be read from inside the process, so it is not re-measured by a run of this script.
 MEASURED_TRAFFIC_BYTES = {"mfma": 42466000}
+TRAFFIC_SOURCE = "offline: profiles/dot_mfma_i8_kernel_fc1_Q512_R8192_D2048_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)"
 SA, SB = 7, 6
+
+
+def _graph_timed_us(launches, rounds=4, replays=5):
+    """Mean microseconds per launch of `launches` (callables that enqueue their kernels on the stream that is current
+    when they are called: a capture makes its own stream current),
+    recorded `rounds` times over into one HIP graph and replayed: no host work between the kernels, the same
+    back-to-back conditions for one resident keyset and for a rotation of many."""
+    import torch
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for f in launches:
+            f()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for _ in range(rounds):
+            for f in launches:
+                f()
+    g.replay()
+    torch.cuda.synchronize()
+    best = None
+    for _ in range(replays):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / (rounds * len(launches))
+        best = us if best is None else min(best, us)
+    return best
+
+
+def _fc2_like(_lib, bsi_ops, iters):
+    """FC2-like dot Q512 x R2048 x D8192, ReLU queries: the int8-image kernel on the verbatim batch, and the same
+    batch kept as EWAH streams (decode launch + dot) next to the verbatim planes taken through the same two steps."""
+    import torch
+
+    Q3, R3, D3 = 512, 2048, 8192
+    torch.manual_seed(123)
+    X = torch.relu(torch.randn(Q3, D3))
+    K = torch.randn(R3, D3) * 0.02
+    kcap, _, _, _, W = bsi_ops.build_bsi_keys_cuda(K, 2, 0.5)
+    qcap = bsi_ops.build_bsi_queries_cuda_batch_packed(X.cuda(), 2, 0.5)
+    hb = bsi_ops.build_bsi_queries_cuda_batch_hybrid(X.cuda(), 2, 0.5)
+    chunks = W // 4
+    out = torch.empty((Q3, R3), dtype=torch.float32, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    kptr, klayout = bsi_ops.key_operand(kcap, Q3, SA, _lib.CORE_MFMA)
+    us = ctypes.c_float(0.0)
+    args = (qcap.words.data_ptr(), qcap.ints8.data_ptr(), qcap.chunk_scales.data_ptr(), chunks, SA, W, kptr, klayout,
+            kcap.slice_weights.data_ptr(), SB, R3, Q3, 1e-4, R3, out.data_ptr(), _lib.CORE_MFMA, None, 0)
+    _lib.check(_lib.lib.bsi_hip_dot_timed(*args, 10, ctypes.byref(us), st), "warmup")
+    _lib.check(_lib.lib.bsi_hip_dot_timed(*args, iters, ctypes.byref(us), st), "timed")
+    t = float(us.value) * 1e-6
+    int8_ops = 2.0 * Q3 * R3 * D3
+    alg_bytes = Q3 * SA * W * 8 + Q3 * chunks * 4 + R3 * SB * W * 8 + R3 * 4 + Q3 * R3 * 4
+    res = {"workload": "FC2-like fixed76 chunk-scale dot Q512 R2048 D8192, ReLU queries", "us_per_call": t * 1e6,
+           "effective_bitop_TOPS": 2.0 * SA * SB * Q3 * R3 * D3 / t / 1e12,
+           "frac_of_int8_mfma_peak": int8_ops / t / 1e12 / MFMA_I8_PEAK_TOPS,
+           "frac_of_hbm_peak_algorithmic": alg_bytes / t / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": alg_bytes}
+    # queries as EWAH streams: the dot's load stage turns the streams into the int8 image (one launch), then the same
+    # kernel runs; next to it the verbatim planes through planes -> int8 image -> dot (what a caller holding planes pays)
+    ws_bytes = int(_lib.lib.bsi_hip_dot_ewah_batch_workspace_bytes(Q3, W))
+    ws = torch.empty((ws_bytes,), dtype=torch.uint8, device="cuda")
+
+    def ewah():
+        _lib.check(_lib.lib.bsi_hip_dot_ewah_batch(hb.comp_words.data_ptr(), hb.comp_off.data_ptr(), hb.comp_len.data_ptr(),
+                                                   SA, W, hb.chunk_scales.data_ptr(), chunks, kptr, klayout,
+                                                   kcap.slice_weights.data_ptr(), SB, R3, Q3, 1e-4, R3, None, out.data_ptr(),
+                                                   None, ws.data_ptr(), ws_bytes, bsi_ops._stream()), "bsi_hip_dot_ewah_batch")
+
+    def planes():
+        _lib.check(_lib.lib.bsi_hip_dot(qcap.words.data_ptr(), None, qcap.chunk_scales.data_ptr(), chunks, SA, W, kptr,
+                                        klayout, kcap.slice_weights.data_ptr(), SB, R3, Q3, 1e-4, R3, out.data_ptr(), None,
+                                        _lib.CORE_MFMA, ws.data_ptr(), ws_bytes, bsi_ops._stream()), "bsi_hip_dot")
+
+    res["ewah_queries"] = {
+        "us_per_call_streams": _graph_timed_us([ewah], rounds=8) ,
+        "us_per_call_verbatim_planes": _graph_timed_us([planes], rounds=8),
+        "stored_query_bytes_streams": int(hb.mem_bytes), "stored_query_bytes_verbatim": int(hb.verbatim_bytes),
+        "note": "both include the launch that derives the int8 query image (from streams / from planes); the headline "
+                "figure above reads the image the builder wrote with the planes"}
+    # a few rows (16 tokens against an OPT-6.7B attention projection): the streams are expanded inside the dot kernel
+    R6 = D6 = 4096
+    g6 = torch.Generator(device="cuda").manual_seed(6)
+    k6 = bsi_ops.build_bsi_keys_cuda(torch.randn(R6, D6, device="cuda", generator=g6) * 0.02, 2, 0.5)[0]
+    x6 = torch.relu(torch.randn(16, D6, device="cuda", generator=g6))
+    q6, h6 = bsi_ops.build_bsi_queries_cuda_batch_packed(x6, 2, 0.5), bsi_ops.build_bsi_queries_cuda_batch_hybrid(x6, 2, 0.5)
+    o6 = torch.empty((16, R6), dtype=torch.float32, device="cuda")
+
+    def few_streams():
+        _lib.check(_lib.lib.bsi_hip_dot_ewah_batch(h6.comp_words.data_ptr(), h6.comp_off.data_ptr(), h6.comp_len.data_ptr(), SA,
+                                                   D6 // 64, h6.chunk_scales.data_ptr(), D6 // 256, k6.words.data_ptr(), k6.layout,
+                                                   k6.slice_weights.data_ptr(), SB, R6, 16, 1e-4, R6, None, o6.data_ptr(), None,
+                                                   None, 0, bsi_ops._stream()), "bsi_hip_dot_ewah_batch")
+
+    def few_verbatim():
+        _lib.check(_lib.lib.bsi_hip_dot(q6.words.data_ptr(), q6.ints8.data_ptr(), q6.chunk_scales.data_ptr(), D6 // 256, SA,
+                                        D6 // 64, k6.words.data_ptr(), k6.layout, k6.slice_weights.data_ptr(), SB, R6, 16, 1e-4,
+                                        R6, o6.data_ptr(), None, _lib.CORE_MFMA, None, 0, bsi_ops._stream()), "bsi_hip_dot")
+
+    res["ewah_queries"]["few_rows_Q16_R4096_D4096"] = {"us_streams_decoded_in_kernel": _graph_timed_us([few_streams], rounds=16),
+                                                       "us_verbatim_int8_image": _graph_timed_us([few_verbatim], rounds=16)}
+    ewah()
+    torch.cuda.synchronize()
+    a = out.clone()
+    planes()
+    torch.cuda.synchronize()
+    res["ewah_queries"]["bit_identical_to_verbatim"] = bool(torch.equal(a, out))
+    return res
+
+
+def _decode_shapes(_lib, bsi_ops):
+    """OPT-6.7B layer shapes at ONE query row (the HBM-bound decode regime): microseconds and GB/s on the packed key
+    planes (0.75 byte per weight), on one resident keyset and on a rotation of keysets larger than the 256 MB
+    memory-side cache, so that every launch reads its planes from HBM."""
+    import torch
+
+    rows = []
+    st = torch.cuda.current_stream().cuda_stream
+    for name, R5, D5 in (("attn 4096x4096", 4096, 4096), ("fc1 16384x4096", 16384, 4096), ("fc2 4096x16384", 4096, 16384)):
+        plane_bytes = R5 * SB * (D5 // 64) * 8
+        n_sets = max(2, -(-640 * 1024 * 1024 // plane_bytes))           # at least 640 MB of planes in rotation
+        gen = torch.Generator(device="cuda").manual_seed(R5 + D5)
+        keysets = []
+        for _ in range(n_sets):
+            Kd = torch.randn(R5, D5, device="cuda", generator=gen) * 0.02
+            keysets.append(bsi_ops.build_bsi_keys_cuda(Kd, 2, 0.5)[0])
+            del Kd
+        for kc in keysets:
+            kc.ints8 = None                                            # the image is not read at one row: free it
+        x = torch.randn(1, D5, device="cuda", generator=gen)
+        qcap = bsi_ops.build_bsi_queries_cuda_batch_packed(x, 2, 0.5)
+        W, chunks = D5 // 64, D5 // 256
+        out = torch.empty((1, R5), dtype=torch.float32, device="cuda")
+
+        def launch(kc):
+            def f():
+                _lib.check(_lib.lib.bsi_hip_dot(qcap.words.data_ptr(), qcap.ints8.data_ptr(), qcap.chunk_scales.data_ptr(),
+                                                chunks, SA, W, kc.words.data_ptr(), kc.layout, kc.slice_weights.data_ptr(),
+                                                SB, R5, 1, 1e-4, R5, out.data_ptr(), None, _lib.CORE_MFMA, None, 0, bsi_ops._stream()),
+                           "bsi_hip_dot")
+            return f
+
+        resident = _graph_timed_us([launch(keysets[0])], rounds=32)
+        rotating = _graph_timed_us([launch(kc) for kc in keysets], rounds=2)
+        rows.append({"layer": name, "Q": 1, "packed_key_plane_bytes": plane_bytes, "keysets_in_rotation": n_sets,
+                     "us_resident": resident, "GBs_on_planes_resident": plane_bytes / resident / 1e3,
+                     "us_rotating": rotating, "GBs_on_planes_rotating": plane_bytes / rotating / 1e3,
+                     "frac_of_hbm_peak_rotating": plane_bytes / rotating / 1e3 / HBM_PEAK_GBS})
+        del keysets
+        torch.cuda.empty_cache()
+    return rows
+
+
+def _opt_prefill():
+    """OPT-1.3B-shaped prefill (24 layers, hidden 2048, 32 heads, FFN 8192, vocab 50272, batch 1 x 512 tokens, every
+    decoder linear layer BSI): tokens/s eager and as a replayed HIP graph, and the dot's share of the forward."""
+    from bsipytorch_amd.benchmarks import benchmark_opt_prefill
+
+    r = benchmark_opt_prefill.run("opt-1.3b", seq_len=512, batch=1, iters=5, warmup=2, dense=False, graph=True)
+    keep = ("model", "layers", "seq_len", "num_bsi_layers", "bsi_fwd_ms", "bsi_tokens_per_s", "bsi_graph_fwd_ms",
+            "bsi_graph_tokens_per_s", "graph_replays_match_eager", "dot_ms_per_prefill", "dot_share_of_fwd",
+            "query_build_kernel_ms_per_prefill", "key_build_s")
+    return {k: r[k] for k in keep if k in r}
 
 
 def main() -> int:
@@ -34,6 +208,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--core", default="auto", choices=["auto", "mfma", "valu"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extras", action="store_true", help="skip the other configurations (FC2-like, decode shapes, prefill)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (a dispatch of known traffic for scaling "
                          "FETCH_SIZE / WRITE_SIZE counters)")
@@ -102,15 +277,22 @@ def main() -> int:
     used_core = args.core if args.core != "auto" else "mfma"
     hbm_gbs = alg_bytes / (kern_us * 1e-6) / 1e9
     if used_core == "mfma":
-        # int8 MFMA contraction: 2*Q*R*D int8 operations per launch against the published dense int8 peak
-        roof = {"bound": "mfma", "achieved": int8_ops / (kern_us * 1e-6) / 1e12, "peak": MFMA_I8_PEAK_TOPS,
-                "unit": "TFLOP/s", "op": "int8 multiply-add counted as 2 ops (TOP/s)"}
+        # Two published roofs apply to the int8 MFMA contraction of this shape and lie close together: 2*Q*R*D int8
+        # operations against the dense int8 peak (floor 3.44 us) and the algorithmic bytes against HBM (floor 3.79 us).
+        # The larger floor binds, so the roofline object is the HBM one; both fractions are reported.
+        mfma_tops = int8_ops / (kern_us * 1e-6) / 1e12
+        floors = {"mfma_us": int8_ops / (MFMA_I8_PEAK_TOPS * 1e12) * 1e6, "hbm_us": alg_bytes / (HBM_PEAK_GBS * 1e9) * 1e6}
+        roof = {"bound": "hbm", "achieved": hbm_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "floors_us": floors,
+                "mfma": {"achieved": mfma_tops, "peak": MFMA_I8_PEAK_TOPS, "unit": "TOP/s (int8 multiply-add = 2 ops)",
+                         "frac": mfma_tops / MFMA_I8_PEAK_TOPS}}
     else:
         # The popcount core is VALU-bound, which the two published roofs do not describe; it is priced
         # against HBM here and against the VALU issue rate in "valu" below.
         roof = {"bound": "hbm", "achieved": hbm_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s"}
     roof["frac"] = roof["achieved"] / roof["peak"]
     roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(used_core)
+    roof["traffic_source"] = TRAFFIC_SOURCE if roof["traffic"] is not None else None
     roof["kernel_us"] = kern_us
     roof["algorithmic_bytes"] = alg_bytes
     roof["hbm_GBs_algorithmic"] = hbm_gbs
@@ -183,6 +365,8 @@ def main() -> int:
         os.environ["BSI_KEY_LAYOUT"] = "canonical"
         bsi_ops._reset_flag_cache()
         kc, *_ = bsi_ops.build_bsi_keys_cuda(K, 2, 0.5)
+        del os.environ["BSI_KEY_LAYOUT"]
+        bsi_ops._reset_flag_cache()
         B = kc.words.cpu().numpy().view(np.uint64)
         bs = kc.slice_weights[:, 0].contiguous().cpu().numpy()
         reps, t_cpu = 0, 0.0
@@ -198,6 +382,17 @@ def main() -> int:
                                   "kind": "port", "sample": f"{reps} full passes of the same Q512 R8192 D2048 dot "
                                   f"(oracle popcount form, OpenMP over keys); {t_cpu / reps * 1e3:.1f} ms per pass",
                                   "ms_per_call": t_cpu / reps * 1e3, "gpu_output_bit_identical": same}
+    if not args.no_extras and used_core == "mfma":
+        extras = {}
+        for key, fn in (("fc2_like", lambda: _fc2_like(_lib, bsi_ops, args.steps)),
+                        ("opt6.7b_layers_one_row", lambda: _decode_shapes(_lib, bsi_ops)),
+                        ("opt1.3b_prefill", _opt_prefill)):
+            try:
+                extras[key] = fn()
+            except Exception as exc:  # the headline line must not be lost to a side figure
+                extras[key] = {"error": f"{type(exc).__name__}: {exc}"}
+            torch.cuda.empty_cache()
+        result["other_configs"] = extras
     print(json.dumps(result))
     return 0
 

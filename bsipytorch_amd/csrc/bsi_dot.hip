@@ -1839,7 +1839,8 @@ __global__ __launch_bounds__(1024) void dot_mfma_stream_ewah_kernel(
 // in-chunk byte order of planes_to_int8_kernel): one workgroup per query row expands the row's Sa streams into LDS
 // (a wave per stream, all-zero slices skipped) and recombines them 32 elements per thread.  The verbatim planes
 // never exist in memory.
-__global__ __launch_bounds__(256) void ewah_streams_to_int8_kernel(const unsigned long long* __restrict__ comp,
+constexpr int kEwahToInt8Block = 512;  // 8 waves: the (at most 8) streams of a row decode side by side
+__global__ __launch_bounds__(kEwahToInt8Block) void ewah_streams_to_int8_kernel(const unsigned long long* __restrict__ comp,
                                                                     const long long* __restrict__ comp_off,
                                                                     const int* __restrict__ comp_len, int Sa, int W64,
                                                                     int chunks, uint32_t* __restrict__ out32) {
@@ -1850,7 +1851,7 @@ __global__ __launch_bounds__(256) void ewah_streams_to_int8_kernel(const unsigne
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int64_t row = blockIdx.x;
-    for (int s = wave; s < Sa; s += 4) {
+    for (int s = wave; s < Sa; s += kEwahToInt8Block / BSI_WAVE) {
         const unsigned long long* in = comp + comp_off[row * Sa + s];
         const int in_len = comp_len[row * Sa + s];
         const bool zero = ewah_stream_is_zero(in, in_len, W64);
@@ -1860,7 +1861,7 @@ __global__ __launch_bounds__(256) void ewah_streams_to_int8_kernel(const unsigne
     __syncthreads();
     const uint32_t* planes32 = reinterpret_cast<const uint32_t*>(planes);
     const int cols = chunks * 8;
-    for (int col = tid; col < cols; col += 256) {
+    for (int col = tid; col < cols; col += kEwahToInt8Block) {
         uint32_t y[8];
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
@@ -2807,7 +2808,7 @@ extern "C" int bsi_hip_dot_ewah_batch(const uint64_t* comp_words, const int64_t*
         return fail(BSI_ERR_UNSUPPORTED, "%d words per slice do not fit the LDS plane buffer of the stream decoder", W64);
     static LdsOptIn once;
     lds_opt_in(once, reinterpret_cast<const void*>(&ewah_streams_to_int8_kernel), 160 * 1024);
-    hipLaunchKernelGGL(ewah_streams_to_int8_kernel, dim3(static_cast<unsigned>(Q)), dim3(256), lds, st,
+    hipLaunchKernelGGL(ewah_streams_to_int8_kernel, dim3(static_cast<unsigned>(Q)), dim3(kEwahToInt8Block), lds, st,
                        reinterpret_cast<const unsigned long long*>(comp_words), reinterpret_cast<const long long*>(comp_off),
                        comp_len, Sa, W64, chunks, static_cast<uint32_t*>(workspace));
     BSI_LAUNCH_CHECK("ewah_streams_to_int8_kernel");
