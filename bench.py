@@ -336,6 +336,16 @@ def main() -> int:
     buf = torch.ones(1 << 30, dtype=torch.uint8, device="cuda")
     _lib.check(_lib.lib.bsi_hip_probe_stream_read(buf.data_ptr(), buf.numel(), ctypes.byref(v), stream), "probe_read")
     peaks["stream_read_GBs"] = v.value / 1e9
+    # the int8-image kernel's operand path: L2-resident bytes into LDS by LDS-direct loads, every CU at once -- with
+    # eight issuing waves and contiguous pieces (the path's best), and as the kernel's four loader waves issue them
+    _lib.check(_lib.lib.bsi_hip_probe_l2_to_lds(buf.data_ptr(), buf.numel(), 0, ctypes.byref(v), stream), "probe_l2_lds")
+    peaks["l2_to_lds_GBs"] = v.value / 1e9
+    _lib.check(_lib.lib.bsi_hip_probe_l2_to_lds(buf.data_ptr(), buf.numel(), 1, ctypes.byref(v), stream), "probe_l2_lds")
+    peaks["l2_to_lds_GBs_four_loader_waves_row_pieces"] = v.value / 1e9
+    # what the headline kernel's chunk loop has to move along that path: (TM + TN) x D bytes per workgroup
+    loop_bytes = ((R + 127) // 128) * ((Q + 127) // 128) * (128 + 128) * D
+    peaks["headline_loop_bytes_l2_to_lds"] = loop_bytes
+    peaks["headline_loop_floor_us_at_the_loader_rate"] = loop_bytes / v.value * 1e6
     del buf
     result["measured_peaks"] = peaks
     result["roofline"]["frac_of_measured_mfma_peak"] = (int8_ops / (kern_us * 1e-6) / 1e12) / peaks["int8_mfma_TOPS"]

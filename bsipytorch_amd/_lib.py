@@ -79,6 +79,7 @@ PROTOTYPES = {
     "bsi_hip_probe_valu_popcount": [ctypes.POINTER(_d), _vp],
     "bsi_hip_probe_mfma_i8": [ctypes.POINTER(_d), _vp],
     "bsi_hip_probe_stream_read": [_vp, _sz, ctypes.POINTER(_d), _vp],
+    "bsi_hip_probe_l2_to_lds": [_vp, _sz, _i, ctypes.POINTER(_d), _vp],
     "bsi_hip_version": [],
     "bsi_hip_last_error": [],
 }

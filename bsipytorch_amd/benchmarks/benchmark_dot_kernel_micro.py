@@ -97,9 +97,12 @@ def main() -> None:
     p.add_argument("--relu", action="store_true", help="ReLU the queries (about half exact zeros)")
     p.add_argument("--planes_only", action="store_true", help="do not hand the builder's int8 queries to the dot")
     p.add_argument("--report_stats", action="store_true")
+    p.add_argument("--i8_tile", type=int, default=0, choices=[0, 128, 1284, 12864, 64, 6432],
+                   help="force a tile of the int8-image kernel (1284: 128 x 128 on four MFMA waves of 64 x 64); 0 = automatic")
     a = p.parse_args()
     if not torch.cuda.is_available():
         raise RuntimeError("a GPU is required for this microbench")
+    _lib.check(_lib.lib.bsi_hip_set_option(_lib.OPT_I8_TILE, a.i8_tile), "bsi_hip_set_option")
     r = run(a.Q, a.R, a.D, a.decimal_places, a.compress_threshold, a.warmup, a.iters, a.seed, a.core, a.key_sigma,
             a.outliers, a.relu, not a.planes_only, a.report_stats)
     print(f"[Microbench] Q={a.Q} R={a.R} D={a.D} iters={a.iters} core={r['core']} layout={r['layout']}")

@@ -762,6 +762,36 @@ __device__ __forceinline__ void load16_to_lds(bsi_rsrc r, uint32_t lane_off, uin
                                              static_cast<int>(wave_off), 0, 0);
 }
 
+// Peak probe for the int8-image kernel's operand path: every workgroup (one per CU) streams an L2-resident region
+// into LDS with the same LDS-direct buffer loads the kernel's loader waves use, 96 KiB in flight per CU (the kernel's
+// three stages), all CUs at once.  Nothing reads the LDS copy; the figure is what the path from L2 through the CU's
+// vector memory unit into LDS delivers -- with kWaves issuing waves of kSlots loads in flight each, in contiguous
+// 1 KiB pieces or (kRows) in the kernel's own pieces of 8 rows x 128 bytes out of 128 rows.
+constexpr int kProbeLdsWaves = 8, kProbeLdsSlots = 12;
+template <int kWaves, int kSlots, bool kRows>
+__global__ __launch_bounds__(kWaves * 64) void probe_l2_lds_kernel(const unsigned char* __restrict__ buf,
+                                                                   size_t region_bytes, int regions, int passes) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
+    const bsi_rsrc r = make_rsrc(buf + static_cast<size_t>(blockIdx.x % regions) * region_bytes, region_bytes);
+    const int pieces = static_cast<int>(region_bytes / 1024);
+    // kRows: the region is 128 rows of region_bytes / 128 bytes; a piece is 8 rows x 128 bytes (the kernel's stage loads)
+    const uint32_t rowbytes = static_cast<uint32_t>(region_bytes / 128);
+    const uint32_t lane_off = kRows ? static_cast<uint32_t>(lane >> 3) * rowbytes + static_cast<uint32_t>(lane & 7) * 16
+                                    : static_cast<uint32_t>(lane) * 16;
+    int slot = 0;
+    for (int pass = 0; pass < passes; ++pass)
+        for (int p = wave; p < pieces; p += kWaves) {
+            const uint32_t wave_off = kRows ? static_cast<uint32_t>(p & 15) * 8 * rowbytes + static_cast<uint32_t>(p >> 4) * 128
+                                            : static_cast<uint32_t>(p) * 1024;
+            load16_to_lds(r, lane_off, wave_off, lds + (wave * kSlots + slot) * 1024);
+            slot = (slot + 1 == kSlots) ? 0 : slot + 1;
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kSlots - 1) : "memory");
+        }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
 // Tile configuration: TM keys x TN queries per workgroup (128 x 128, 128 x 64, 64 x 64 or 64 x 32; the smaller
 // ones for grids that would leave CUs without a workgroup), MFMA waves arranged 2 (keys) x kWavesN (queries),
 // each WM x WN tiles of 16 x 16; one loader wave per (up to) 64 operand rows.
@@ -784,6 +814,145 @@ struct I8Cfg {
     static constexpr int kEpilogueBytes = 2 * TM * 4;  // the tile's key factors, then its biases (chain modes)
     static constexpr int kLds = 4 * kStage + kScaleBytes + kEpilogueBytes;
 };
+
+// A loader wave of the int8-image kernels (lw = its number among the C::kLoaders loader waves; `consumers` MFMA
+// waves share the workgroup's barriers with it): 8 of the stage's groups of 8 rows (the TM key rows, then the TN
+// query rows: a load moves 1 KiB = 8 rows x 128 bytes), plus the chunk scales of 64 queries once per chunk.
+template <int TM, int TN, bool kSum>
+__device__ __forceinline__ void i8_loader_wave(unsigned char* __restrict__ lds, int lw, int lane,
+                                               const int8_t* __restrict__ A8, const float* __restrict__ qscale,
+                                               int qscale_stride, const int8_t* __restrict__ K8,
+                                               const float* __restrict__ Bw, int Sb, int chunks, int halves, int64_t R,
+                                               int64_t Q, int64_t r0, int64_t q0, size_t rowbytes,
+                                               const float* __restrict__ bias, int ndig, long long dig_stride,
+                                               int key_tiled, const unsigned char* __restrict__ warm,
+                                               long long warm_lines) {
+    using C = I8Cfg<TM, TN>;
+    unsigned char* const scale_lds = lds + 4 * C::kStage;  // [chunk & 3][loader][64] floats
+    // tiled keys: blocks of 64 rows x 128 bytes per half-chunk, 2 chunks of them per 64-row tile; rows past R
+    // are zero padding inside the last block, blocks past the last one read as zero (buffer bounds)
+    const size_t kblock = static_cast<size_t>(chunks) * 2 * 8192;  // bytes of a 64-row tile
+    const bsi_rsrc rk = key_tiled ? make_rsrc(K8 + static_cast<size_t>(r0 / 64) * kblock,
+                                              static_cast<size_t>((R + 63) / 64 - r0 / 64) * kblock)
+                                  : make_rsrc(K8 + static_cast<size_t>(r0) * rowbytes,
+                                              static_cast<size_t>(R - r0) * rowbytes);
+    const bsi_rsrc rq = make_rsrc(A8 + static_cast<size_t>(q0) * rowbytes,
+                                  static_cast<size_t>(Q - q0) * rowbytes +
+                                      (kSum ? static_cast<size_t>(ndig - 1) * static_cast<size_t>(dig_stride) : 0));
+    const bsi_rsrc rs = make_rsrc(qscale + q0 * qscale_stride, static_cast<size_t>(Q - q0) * qscale_stride * 4);
+    if (!kSum) {
+        // The epilogue's operands, staged once per workgroup: the slice-0 weight (key factor) and the bias of the
+        // tile's TM keys, 64 rows per load.  Fetched per lane at the end they are 32 vector-memory instructions
+        // for every MFMA wave, half as many as the whole chunk loop issues, all queued in front of the stores.
+        // Issued first, they have landed before any stage has (loads return in order).  Rows past R, and the
+        // biases of a call without one, read nothing and give 0 (buffer bounds).
+        const bsi_rsrc wrs = make_rsrc(Bw + static_cast<size_t>(r0) * Sb, static_cast<size_t>(R - r0) * Sb * sizeof(float));
+        const bsi_rsrc brs = make_rsrc(bias != nullptr ? bias + r0 : Bw,
+                                       bias != nullptr ? static_cast<size_t>(R - r0) * sizeof(float) : 0);
+        unsigned char* const epi = lds + 4 * C::kStage + C::kScaleBytes;
+        for (int j = lw; j < 2 * (TM / 64); j += C::kLoaders) {
+            const bool is_bias = j >= TM / 64;
+            const int blk = is_bias ? j - TM / 64 : j;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(is_bias ? brs : wrs,
+                                                     BSI_LDS_PTR(epi + (is_bias ? TM * 4 : 0) + blk * 256), 4,
+                                                     (blk * 64 + lane) * (is_bias ? 4 : Sb * 4), 0, 0, 0);
+        }
+    }
+    // the stage has kGroups groups of 8 rows, keys first; loader lw moves groups lw, lw + kLoaders, ... (when
+    // the groups do not divide evenly the last load wraps around and fetches a group a second time, so that
+    // every loader wave has the same number of loads in flight)
+    constexpr int NI = C::kLoads;
+    uint32_t off[NI];
+    bool is_key[NI];  // wave-uniform
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+        const int g = (lw + C::kLoaders * i) % C::kGroups;
+        is_key[i] = g < TM / 8;
+        const int rowl = (is_key[i] ? g : g - TM / 8) * 8 + (lane >> 3);  // row of its operand tile
+        const uint32_t col = static_cast<uint32_t>((lane & 7) ^ ((rowl >> 1) & 7)) * 16;  // logical column landing here
+        const int64_t lim = is_key[i] ? (R - r0) : (Q - q0);              // past the end: clamp (never stored)
+        const int64_t rr = (rowl < lim) ? rowl : (lim - 1);
+        off[i] = static_cast<uint32_t>(rr * rowbytes) + col;
+        if (is_key[i] && key_tiled)
+            off[i] = static_cast<uint32_t>(rowl >> 6) * static_cast<uint32_t>(kblock) +
+                     static_cast<uint32_t>(rowl & 63) * 128 + col;
+    }
+    const uint32_t kstep_bytes = key_tiled ? 8192u : 128u;  // from one half-chunk of a key row to the next
+    // scales: loader wave lw fetches the 64 queries of group lw % (TN / 64) (waves fetching the same group
+    // write their own regions, so that every loader wave has the same number of loads in flight)
+    const int sq = (lw % (TN >= 64 ? TN / 64 : 1)) * 64 + lane;
+    const uint32_t soff = static_cast<uint32_t>(((q0 + sq < Q) ? sq : (Q - 1 - q0)) * qscale_stride * 4);
+    const int sstep = (qscale_stride == 1) ? 0 : 4;
+    // issue() is called for h = 0, 1, 2, ... in order; in the sum mode (next_c, next_dg) follow the chunk and
+    // the digit (counted from the top one) of the half-chunk to come
+    int next_c = 0, next_dg = 0;
+    uint32_t so_k = 0, so_q = 0;
+    auto issue = [&](int h) {  // stage of half-chunk h (clamped to the last) into its ring slot
+        const int hc = h < halves ? h : halves - 1;
+        if (kSum) {
+            if (h < halves) {
+                const uint32_t half = static_cast<uint32_t>(next_c) * 2 + static_cast<uint32_t>(h & 1);
+                so_k = half * kstep_bytes;
+                so_q = half * 128 + static_cast<uint32_t>(ndig - 1 - next_dg) * static_cast<uint32_t>(dig_stride);
+                if (h & 1) {
+                    if (++next_c == chunks) {
+                        next_c = 0;
+                        ++next_dg;
+                    }
+                }
+            }
+        } else {
+            so_q = static_cast<uint32_t>(hc) * 128;
+            so_k = static_cast<uint32_t>(hc) * kstep_bytes;
+        }
+#pragma unroll
+        for (int i = 0; i < NI; ++i)
+            load16_to_lds(is_key[i] ? rk : rq, off[i], is_key[i] ? so_k : so_q,
+                          lds + (h & 3) * C::kStage + ((lw + C::kLoaders * i) % C::kGroups) * 1024);
+        if (!kSum && (h & 1)) {  // with the second half of chunk c = h / 2: its scales
+            const int c = hc >> 1;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                rs, BSI_LDS_PTR(scale_lds + ((c & 3) * C::kLoaders + lw) * 256), 4, static_cast<int>(soff),
+                c * sstep, 0, 0);
+        }
+    };
+    issue(0);
+    issue(1);
+    issue(2);
+    // stage 0 landed (stage 1 + scales + stage 2, 2 NI + 1 instructions, may be in flight)
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NI + (kSum ? 0 : 1)) : "memory");
+    lds_barrier();
+    for (int h = 0; h < halves; ++h) {
+        if (h + 3 < halves) {
+            issue(h + 3);  // its slot was released by the barrier that ended half h - 1
+            // stage h + 1 (and the scales issued right behind it) landed; stages h + 2, h + 3 and one
+            // scale load, 2 NI + 1 instructions, may still be in flight
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NI + (kSum ? 0 : 1)) : "memory");
+        } else if (h + 3 == halves) {
+            // nothing left to issue (a copy of the last stage here, as the prologue does for a single chunk, would
+            // queue 96 KiB of loads in front of every workgroup's output stores); the last stage and its
+            // scales may be in flight
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NI + (kSum ? 0 : 1)) : "memory");
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+        lds_barrier();
+    }
+    if (warm_lines > 0) {
+        // one lane per 128-byte line, 64 lines per load; this loader wave's share of the region.  The values
+        // are summed only so that the loads stay; the store below never happens.
+        const long long waves = static_cast<long long>(gridDim.x) * gridDim.y * C::kLoaders;
+        const long long mine = (static_cast<long long>(blockIdx.y) * gridDim.x + blockIdx.x) * C::kLoaders + lw;
+        const long long per = (warm_lines + waves - 1) / waves;
+        const long long first = mine * per;
+        const long long last = (first + per < warm_lines) ? first + per : warm_lines;
+        unsigned sum = 0;
+        for (long long l = first + lane; l < last; l += 64)
+            sum += *reinterpret_cast<const volatile unsigned*>(warm + l * 128);
+        if (sum == 0x5ca1ab1eu && warm_lines < 0) scale_lds[lane] = 0;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still be writing LDS when the workgroup ends
+}
 
 // One k-step (64 of a chunk's 256 elements) of an MFMA wave: WM WN MFMAs on the operands in (ka, qb), one
 // epilogue element of the previous chunk (held in `prev`) behind each MFMA, and behind the first WM + WN of them
@@ -859,132 +1028,8 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
     unsigned char* const scale_lds = lds + 4 * C::kStage;  // [chunk & 3][loader][64] floats
 
     if (wave >= C::kConsumers) {
-        // ---- loader wave lw: 8 of the stage's groups of 8 rows (the TM key rows, then the TN query rows: a
-        // load moves 1 KiB = 8 rows x 128 bytes), plus the chunk scales of 64 queries once per chunk.
-        const int lw = wave - C::kConsumers;
-        // tiled keys: blocks of 64 rows x 128 bytes per half-chunk, 2 chunks of them per 64-row tile; rows past R
-        // are zero padding inside the last block, blocks past the last one read as zero (buffer bounds)
-        const size_t kblock = static_cast<size_t>(chunks) * 2 * 8192;  // bytes of a 64-row tile
-        const bsi_rsrc rk = key_tiled ? make_rsrc(K8 + static_cast<size_t>(r0 / 64) * kblock,
-                                                  static_cast<size_t>((R + 63) / 64 - r0 / 64) * kblock)
-                                      : make_rsrc(K8 + static_cast<size_t>(r0) * rowbytes,
-                                                  static_cast<size_t>(R - r0) * rowbytes);
-        const bsi_rsrc rq = make_rsrc(A8 + static_cast<size_t>(q0) * rowbytes,
-                                      static_cast<size_t>(Q - q0) * rowbytes +
-                                          (kSum ? static_cast<size_t>(ndig - 1) * static_cast<size_t>(dig_stride) : 0));
-        const bsi_rsrc rs = make_rsrc(qscale + q0 * qscale_stride, static_cast<size_t>(Q - q0) * qscale_stride * 4);
-        if (!kSum) {
-            // The epilogue's operands, staged once per workgroup: the slice-0 weight (key factor) and the bias of the
-            // tile's TM keys, 64 rows per load.  Fetched per lane at the end they are 32 vector-memory instructions
-            // for every MFMA wave, half as many as the whole chunk loop issues, all queued in front of the stores.
-            // Issued first, they have landed before any stage has (loads return in order).  Rows past R, and the
-            // biases of a call without one, read nothing and give 0 (buffer bounds).
-            const bsi_rsrc wrs = make_rsrc(Bw + static_cast<size_t>(r0) * Sb, static_cast<size_t>(R - r0) * Sb * sizeof(float));
-            const bsi_rsrc brs = make_rsrc(bias != nullptr ? bias + r0 : Bw,
-                                           bias != nullptr ? static_cast<size_t>(R - r0) * sizeof(float) : 0);
-            unsigned char* const epi = lds + 4 * C::kStage + C::kScaleBytes;
-            for (int j = lw; j < 2 * (TM / 64); j += C::kLoaders) {
-                const bool is_bias = j >= TM / 64;
-                const int blk = is_bias ? j - TM / 64 : j;
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(is_bias ? brs : wrs,
-                                                         BSI_LDS_PTR(epi + (is_bias ? TM * 4 : 0) + blk * 256), 4,
-                                                         (blk * 64 + lane) * (is_bias ? 4 : Sb * 4), 0, 0, 0);
-            }
-        }
-        // the stage has kGroups groups of 8 rows, keys first; loader lw moves groups lw, lw + kLoaders, ... (when
-        // the groups do not divide evenly the last load wraps around and fetches a group a second time, so that
-        // every loader wave has the same number of loads in flight)
-        constexpr int NI = C::kLoads;
-        uint32_t off[NI];
-        bool is_key[NI];  // wave-uniform
-#pragma unroll
-        for (int i = 0; i < NI; ++i) {
-            const int g = (lw + C::kLoaders * i) % C::kGroups;
-            is_key[i] = g < TM / 8;
-            const int rowl = (is_key[i] ? g : g - TM / 8) * 8 + (lane >> 3);  // row of its operand tile
-            const uint32_t col = static_cast<uint32_t>((lane & 7) ^ ((rowl >> 1) & 7)) * 16;  // logical column landing here
-            const int64_t lim = is_key[i] ? (R - r0) : (Q - q0);              // past the end: clamp (never stored)
-            const int64_t rr = (rowl < lim) ? rowl : (lim - 1);
-            off[i] = static_cast<uint32_t>(rr * rowbytes) + col;
-            if (is_key[i] && key_tiled)
-                off[i] = static_cast<uint32_t>(rowl >> 6) * static_cast<uint32_t>(kblock) +
-                         static_cast<uint32_t>(rowl & 63) * 128 + col;
-        }
-        const uint32_t kstep_bytes = key_tiled ? 8192u : 128u;  // from one half-chunk of a key row to the next
-        // scales: loader wave lw fetches the 64 queries of group lw % (TN / 64) (waves fetching the same group
-        // write their own regions, so that every loader wave has the same number of loads in flight)
-        const int sq = (lw % (TN >= 64 ? TN / 64 : 1)) * 64 + lane;
-        const uint32_t soff = static_cast<uint32_t>(((q0 + sq < Q) ? sq : (Q - 1 - q0)) * qscale_stride * 4);
-        const int sstep = (qscale_stride == 1) ? 0 : 4;
-        // issue() is called for h = 0, 1, 2, ... in order; in the sum mode (next_c, next_dg) follow the chunk and
-        // the digit (counted from the top one) of the half-chunk to come
-        int next_c = 0, next_dg = 0;
-        uint32_t so_k = 0, so_q = 0;
-        auto issue = [&](int h) {  // stage of half-chunk h (clamped to the last) into its ring slot
-            const int hc = h < halves ? h : halves - 1;
-            if (kSum) {
-                if (h < halves) {
-                    const uint32_t half = static_cast<uint32_t>(next_c) * 2 + static_cast<uint32_t>(h & 1);
-                    so_k = half * kstep_bytes;
-                    so_q = half * 128 + static_cast<uint32_t>(ndig - 1 - next_dg) * static_cast<uint32_t>(dig_stride);
-                    if (h & 1) {
-                        if (++next_c == chunks) {
-                            next_c = 0;
-                            ++next_dg;
-                        }
-                    }
-                }
-            } else {
-                so_q = static_cast<uint32_t>(hc) * 128;
-                so_k = static_cast<uint32_t>(hc) * kstep_bytes;
-            }
-#pragma unroll
-            for (int i = 0; i < NI; ++i)
-                load16_to_lds(is_key[i] ? rk : rq, off[i], is_key[i] ? so_k : so_q,
-                              lds + (h & 3) * C::kStage + ((lw + C::kLoaders * i) % C::kGroups) * 1024);
-            if (!kSum && (h & 1)) {  // with the second half of chunk c = h / 2: its scales
-                const int c = hc >> 1;
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(
-                    rs, BSI_LDS_PTR(scale_lds + ((c & 3) * C::kLoaders + lw) * 256), 4, static_cast<int>(soff),
-                    c * sstep, 0, 0);
-            }
-        };
-        issue(0);
-        issue(1);
-        issue(2);
-        // stage 0 landed (stage 1 + scales + stage 2, 2 NI + 1 instructions, may be in flight)
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NI + (kSum ? 0 : 1)) : "memory");
-        lds_barrier();
-        for (int h = 0; h < halves; ++h) {
-            if (h + 3 < halves) {
-                issue(h + 3);  // its slot was released by the barrier that ended half h - 1
-                // stage h + 1 (and the scales issued right behind it) landed; stages h + 2, h + 3 and one
-                // scale load, 2 NI + 1 instructions, may still be in flight
-                asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NI + (kSum ? 0 : 1)) : "memory");
-            } else if (h + 3 == halves) {
-                // nothing left to issue (a copy of the last stage here, as the prologue does for a single chunk, would
-                // queue 96 KiB of loads in front of every workgroup's output stores); the last stage and its
-                // scales may be in flight
-                asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NI + (kSum ? 0 : 1)) : "memory");
-            } else {
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            }
-            lds_barrier();
-        }
-        if (warm_lines > 0) {
-            // one lane per 128-byte line, 64 lines per load; this loader wave's share of the region.  The values
-            // are summed only so that the loads stay; the store below never happens.
-            const long long waves = static_cast<long long>(gridDim.x) * gridDim.y * C::kLoaders;
-            const long long mine = (static_cast<long long>(blockIdx.y) * gridDim.x + blockIdx.x) * C::kLoaders + lw;
-            const long long per = (warm_lines + waves - 1) / waves;
-            const long long first = mine * per;
-            const long long last = (first + per < warm_lines) ? first + per : warm_lines;
-            unsigned sum = 0;
-            for (long long l = first + lane; l < last; l += 64)
-                sum += *reinterpret_cast<const volatile unsigned*>(warm + l * 128);
-            if (sum == 0x5ca1ab1eu && warm_lines < 0) scale_lds[lane] = 0;
-        }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still be writing LDS when the workgroup ends
+        i8_loader_wave<TM, TN, kSum>(lds, wave - C::kConsumers, lane, A8, qscale, qscale_stride, K8, Bw, Sb, chunks, halves, R,
+                                     Q, r0, q0, rowbytes, bias, ndig, dig_stride, key_tiled, warm, warm_lines);
         return;
     }
 
@@ -1241,6 +1286,219 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
                     if (rb + e < R) dst[e] = accf[a][b][e];
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------ int8 image, four MFMA waves of 64 x 64
+//
+// The same workgroup tile (128 keys x 128 queries), ring, loader waves and epilogue as dot_mfma_i8_kernel<128, 128>,
+// with the arithmetic on FOUR MFMA waves of 64 keys x 64 queries (one per SIMD, next to its loader wave) instead of
+// eight of 64 x 32.  An MFMA wave's operand reads are (64 + 64) x 64 bytes per 64 x 64 x 64 MACs instead of
+// (64 + 32) x 64 per 64 x 32 x 64: a third fewer LDS bytes per MAC, on an LDS whose read port the eight-wave kernel
+// keeps as busy as its matrix pipes.  Eight waves of 256 registers hold one int32 accumulator set (64), the fp32
+// chain values (64) and two operand sets (64): there is no second accumulator set to park a finished chunk in, so
+// the chain step of chunk c (one cvt + one fma per output) runs on the accumulators in place, between a tile's last
+// MFMA of chunk c (k-step 3) and its first of chunk c + 1 (k-step 0, which starts from zero and overwrites it):
+// two elements behind each MFMA of k-step 3 from its third MFMA on (tiles 0..6), three behind each of the first
+// twelve MFMAs of the next k-step 0 (tiles 7..15), always tiles whose turn to be overwritten has not come.
+// Where a lane's accumulators go in the [Q, R, chunks] dump (parity checks): element (a, b, e) at
+// base + b * qstep + (a * 16 + e) * chunks, for the query columns of qmask and the first rows[a] key rows of tile a.
+struct I8WDump {
+    int64_t base, qstep;
+    int rows[4];
+    unsigned qmask;
+};
+template <int KS, bool kInts>
+__device__ __forceinline__ void i8w_chain(int first, int count, const v4i (&acc)[4][4], float (&accf)[4][4][4],
+                                          const float (&qs)[4], int* __restrict__ ints_at, const I8WDump& dump,
+                                          int down_shift, int chunks) {
+#pragma unroll
+    for (int i = first; i < first + count; ++i) {
+        const int tile = i >> 2, e = i & 3, a = tile >> 2, b = tile & 3;
+        accf[a][b][e] = fmaf(static_cast<float>(acc[a][b][e]), qs[b], accf[a][b][e]);
+        if (kInts && ints_at != nullptr && ((dump.qmask >> b) & 1u) && e < dump.rows[a])
+            ints_at[dump.base + b * dump.qstep + static_cast<int64_t>(a * 16 + e) * chunks] = acc[a][b][e] >> down_shift;
+    }
+}
+
+// One k-step of a 64 x 64 MFMA wave: 16 MFMAs (tile t = 4 a + b), the reads of the next k-step's eight operand
+// tiles behind the first eight, and the chain elements that fall to this k-step (see above).  qs_cur / ints_cur:
+// scales and accumulator dump of the chunk being computed (used by k-step 3); qs_prev / ints_prev: of the chunk
+// before it (used by k-step 0).
+template <int KS, bool kInts>
+__device__ __forceinline__ void i8w_kstep(const v4i (&ka)[4], const v4i (&qb)[4], v4i (&ka_n)[4], v4i (&qb_n)[4],
+                                          const unsigned char* __restrict__ krow_n,
+                                          const unsigned char* __restrict__ qrow_n, v4i (&acc)[4][4],
+                                          float (&accf)[4][4][4], const float (&qs_cur)[4], const float (&qs_prev)[4],
+                                          int* __restrict__ ints_cur, int* __restrict__ ints_prev, const I8WDump& dump,
+                                          int down_shift, int chunks) {
+#pragma unroll
+    for (int t = 0; t < 16; ++t) {
+        const int a = t >> 2, b = t & 3;
+        const v4i c0 = (KS == 0) ? (v4i){0, 0, 0, 0} : acc[a][b];
+        acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ka[a], qb[b], c0, 0, 0, 0);
+        // read number t of the next k-step, in the order its MFMAs first need them: ka[0], qb[0..3], ka[1..3]
+        if (t == 0) ka_n[0] = *reinterpret_cast<const v4i*>(krow_n);
+        else if (t <= 4) qb_n[t - 1] = *reinterpret_cast<const v4i*>(qrow_n + (t - 1) * 16 * 128);
+        else if (t < 8) ka_n[t - 4] = *reinterpret_cast<const v4i*>(krow_n + (t - 4) * 16 * 128);
+        if (KS == 0 && t < 12)  // elements 28 + 3 t .. + 2 of the previous chunk: tiles 7 .. 15, none of them below t + 1
+            i8w_chain<KS, kInts>(28 + 3 * t, 3, acc, accf, qs_prev, ints_prev, dump, down_shift, chunks);
+        if (KS == 3 && t >= 2)  // elements 2 (t - 2), + 1 of this chunk: tiles 0 .. 6, finished two MFMAs ago or earlier
+            i8w_chain<KS, kInts>(2 * (t - 2), 2, acc, accf, qs_cur, ints_cur, dump, down_shift, chunks);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
+constexpr int kI8WConsumers = 4;
+constexpr int kI8WBlock = (kI8WConsumers + I8Cfg<128, 128>::kLoaders) * 64;
+
+template <bool kInts>
+__global__ __launch_bounds__(kI8WBlock) void dot_mfma_i8w_kernel(
+    const int8_t* __restrict__ A8, const float* __restrict__ qscale, int qscale_stride, const int8_t* __restrict__ K8,
+    const float* __restrict__ Bw, int Sb, int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv,
+    int64_t R_total, float* __restrict__ out, int* __restrict__ chunk_ints, const float* __restrict__ bias,
+    int key_tiled, const unsigned char* __restrict__ warm, long long warm_lines) {
+    constexpr int TM = 128, TN = 128;
+    using C = I8Cfg<TM, TN>;
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];  // C::kLds
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int64_t r0 = static_cast<int64_t>(blockIdx.x) * TM;
+    const int64_t q0 = static_cast<int64_t>(blockIdx.y) * TN;
+    const size_t rowbytes = static_cast<size_t>(chunks) * 256;
+    const int halves = chunks * 2;
+    unsigned char* const scale_lds = lds + 4 * C::kStage;
+
+    if (wave >= kI8WConsumers) {
+        i8_loader_wave<TM, TN, false>(lds, wave - kI8WConsumers, lane, A8, qscale, qscale_stride, K8, Bw, Sb, chunks, halves,
+                                      R, Q, r0, q0, rowbytes, bias, 1, 0, key_tiled, warm, warm_lines);
+        return;
+    }
+
+    // ---- MFMA waves: wr = half of the keys, wq = half of the queries
+    const int wr = wave & 1, wq = wave >> 1;
+    const int ln = lane & 15, lg = lane >> 4;
+    const int krow_off = (wr * 64 + ln) * 128;
+    const int qrow_off = C::kOperandK + (wq * 64 + ln) * 128;
+    int pcol[2];
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) pcol[kk] = ((kk * 4 + lg) ^ (ln >> 1)) * 16;
+    float accf[4][4][4];
+    v4i acc[4][4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            acc[a][b] = (v4i){0, 0, 0, 0};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) accf[a][b][e] = 0.0f;
+        }
+    const float down = __uint_as_float(static_cast<uint32_t>(127 - down_shift) << 23);
+    I8WDump dump;
+    {
+        const int64_t rl = r0 + wr * 64 + lg * 4, ql = q0 + wq * 64 + ln;  // the lane's first key row and query column
+        dump.base = (ql * R + rl) * chunks;
+        dump.qstep = 16 * R * chunks;
+        dump.qmask = 0;
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            const int64_t left = R - (rl + a * 16);
+            dump.rows[a] = static_cast<int>(left < 0 ? 0 : (left < 4 ? left : 4));
+        }
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+            if (kInts && ql + b * 16 < Q) dump.qmask |= 1u << b;
+    }
+    // chunk scales of the lane's four query columns, from the loaders' ring: region wq holds queries 64 wq .. + 63
+    const unsigned char* sread = scale_lds + wq * 256 + ln * 4;
+    float qsa[4], qsb[4];  // scales of even / odd chunks (all zero before the first chunk: its "previous" chain adds 0)
+#pragma unroll
+    for (int b = 0; b < 4; ++b) qsa[b] = qsb[b] = 0.0f;
+#define BSI_I8W_SCALES(dst, c)                                                                         \
+    {                                                                                                  \
+        _Pragma("unroll") for (int b = 0; b < 4; ++b) dst[b] =                                         \
+            *reinterpret_cast<const float*>(sread + ((c) & 3) * (C::kLoaders * 256) + b * 64);         \
+    }
+    v4i ka[2][4], qb[2][4];  // operand sets of even / odd k-steps
+#define BSI_I8W_KSTEP(KS, nslot, qc, qp, ic, ip)                                                                    \
+    i8w_kstep<KS, kInts>(ka[(KS) & 1], qb[(KS) & 1], ka[((KS) + 1) & 1], qb[((KS) + 1) & 1],                        \
+                         lds + (nslot) * C::kStage + krow_off + pcol[((KS) + 1) & 1],                               \
+                         lds + (nslot) * C::kStage + qrow_off + pcol[((KS) + 1) & 1], acc, accf, qc, qp, ic, ip,    \
+                         dump, down_shift, chunks);
+    // a chunk whose halves sit in ring slots s0, s0 + 1; nslot: slot of the next chunk's first half; qc / qp: this
+    // chunk's and the previous chunk's scales.  This chunk's scales have landed with its second half, which the
+    // first barrier announces.
+#define BSI_I8W_CHUNK(s0, nslot, qc, qp, ic, ip, c)                                                                 \
+    BSI_I8W_KSTEP(0, s0, qc, qp, ic, ip);                                                                           \
+    lds_barrier();                                                                                                  \
+    BSI_I8W_SCALES(qc, c);                                                                                          \
+    BSI_I8W_KSTEP(1, (s0) + 1, qc, qp, ic, ip);                                                                     \
+    BSI_I8W_KSTEP(2, (s0) + 1, qc, qp, ic, ip);                                                                     \
+    lds_barrier();                                                                                                  \
+    BSI_I8W_KSTEP(3, nslot, qc, qp, ic, ip);
+
+    lds_barrier();  // stage 0 is there
+#pragma unroll
+    for (int t = 0; t < 4; ++t) ka[0][t] = *reinterpret_cast<const v4i*>(lds + krow_off + t * 16 * 128 + pcol[0]);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) qb[0][t] = *reinterpret_cast<const v4i*>(lds + qrow_off + t * 16 * 128 + pcol[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    int c = 0;
+    for (; c + 1 < chunks; c += 2) {
+        // even chunk c: ring slots 0 and 1, scales qsa; the chain elements of chunk c - 1 left for its k-step 0 use qsb
+        BSI_I8W_CHUNK(0, 2, qsa, qsb, chunk_ints + c, (c > 0 ? chunk_ints + (c - 1) : nullptr), c);
+        // odd chunk c + 1: ring slots 2 and 3, scales qsb
+        BSI_I8W_CHUNK(2, 0, qsb, qsa, chunk_ints + c + 1, chunk_ints + c, c + 1);
+    }
+    bool last_even = false;
+    if (c < chunks) {  // odd number of chunks: one more even chunk
+        BSI_I8W_CHUNK(0, 2, qsa, qsb, chunk_ints + c, (c > 0 ? chunk_ints + (c - 1) : nullptr), c);
+        last_even = true;
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the last k-step read ahead into a stage nothing uses
+#undef BSI_I8W_CHUNK
+#undef BSI_I8W_KSTEP
+#undef BSI_I8W_SCALES
+    // the chain elements of the last chunk that its k-step 3 left (28 .. 63)
+    if (last_even) i8w_chain<0, kInts>(28, 36, acc, accf, qsa, chunk_ints + (chunks - 1), dump, down_shift, chunks);
+    else i8w_chain<0, kInts>(28, 36, acc, accf, qsb, chunk_ints + (chunks - 1), dump, down_shift, chunks);
+    // key factors and biases from the copy the loader waves staged in LDS
+    float bs[4][4], bi[4][4];
+    {
+        const float* epi = reinterpret_cast<const float*>(lds + 4 * C::kStage + C::kScaleBytes);
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            const int rl = wr * 64 + a * 16 + lg * 4;
+            const float4 w4 = *reinterpret_cast<const float4*>(epi + rl);
+            const float4 b4 = *reinterpret_cast<const float4*>(epi + TM + rl);
+            bs[a][0] = w4.x, bs[a][1] = w4.y, bs[a][2] = w4.z, bs[a][3] = w4.w;
+            bi[a][0] = b4.x, bi[a][1] = b4.y, bi[a][2] = b4.z, bi[a][3] = b4.w;
+        }
+    }
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+        const int64_t rb = r0 + wr * 64 + a * 16 + lg * 4;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const int64_t q = q0 + wq * 64 + b * 16 + ln;
+            float v[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                v[e] = ((accf[a][b][e] * down) * bs[a][e]) * scale_inv;
+                if (bias != nullptr) v[e] = v[e] + bi[a][e];
+            }
+            if (q >= Q) continue;
+            float* dst = out + static_cast<size_t>(q) * R_total + rb;
+            if (rb + 3 < R && ((reinterpret_cast<uintptr_t>(dst) & 15) == 0)) {
+                *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (rb + e < R) dst[e] = v[e];
             }
         }
     }
@@ -2242,6 +2500,25 @@ static void launch_mfma_i8_t(int ndig, long long dig_stride, const long long* ke
                                             R_total, out, chunk_ints, bias, st, 1, 0, nullptr, key_tiled);
 }
 
+// The 128 x 128 tile on four MFMA waves of 64 x 64 (chain modes only).
+static void launch_mfma_i8w(const int8_t* A8, const float* qscale, int stride, const int8_t* K8, const float* Bw, int Sb,
+                            int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv, int64_t R_total, float* out,
+                            int32_t* chunk_ints, const float* bias, hipStream_t st, int key_tiled) {
+    using C = I8Cfg<128, 128>;
+    const dim3 grid(static_cast<unsigned>((R + 127) / 128), static_cast<unsigned>((Q + 127) / 128));
+    static LdsOptIn once0, once1;
+    lds_opt_in(once0, reinterpret_cast<const void*>(&dot_mfma_i8w_kernel<false>), C::kLds);
+    lds_opt_in(once1, reinterpret_cast<const void*>(&dot_mfma_i8w_kernel<true>), C::kLds);
+    const unsigned char* warm = static_cast<const unsigned char*>(g_warm_ptr);
+    const long long warm_lines = static_cast<long long>(g_warm_bytes / 128);
+    if (chunk_ints)
+        hipLaunchKernelGGL((dot_mfma_i8w_kernel<true>), grid, dim3(kI8WBlock), C::kLds, st, A8, qscale, stride, K8, Bw, Sb,
+                           chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias, key_tiled, warm, warm_lines);
+    else
+        hipLaunchKernelGGL((dot_mfma_i8w_kernel<false>), grid, dim3(kI8WBlock), C::kLds, st, A8, qscale, stride, K8, Bw, Sb,
+                           chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias, key_tiled, warm, warm_lines);
+}
+
 // Tile choice.  The 128 x 128 tile moves the fewest operand bytes per MAC and is the fastest whenever its grid
 // covers the 256 CUs (one workgroup per CU at a time) -- measured up to several rounds of 256.  A smaller grid
 // leaves CUs idle that smaller tiles would use: a workgroup's time per half-chunk is about 1 : 0.63 : 0.35 : 0.31
@@ -2268,8 +2545,13 @@ static void launch_mfma_i8(const int8_t* A8, const float* qscale, int stride, co
                            float* out, int32_t* chunk_ints, const float* bias, hipStream_t st, int key_tiled = 0,
                            int ndig = 0, long long dig_stride = 0, const long long* key_indices = nullptr) {
     const int tile = choose_i8_tile(R, Q);
+    if (tile == 1284 && ndig == 0) {
+        launch_mfma_i8w(A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias,
+                        st, key_tiled);
+        return;
+    }
 #define BSI_I8_ARGS ndig, dig_stride, key_indices, key_tiled, A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias, st
-    if (tile == 128) launch_mfma_i8_t<128, 128>(BSI_I8_ARGS);
+    if (tile == 128 || tile == 1284) launch_mfma_i8_t<128, 128>(BSI_I8_ARGS);
     else if (tile == 12864) launch_mfma_i8_t<128, 64>(BSI_I8_ARGS);
     else if (tile == 64) launch_mfma_i8_t<64, 64>(BSI_I8_ARGS);
     else launch_mfma_i8_t<64, 32>(BSI_I8_ARGS);
@@ -2363,8 +2645,8 @@ extern "C" int bsi_hip_set_option(int option, int value) {
             g_digits_route = value;
             return BSI_OK;
         case BSI_OPT_I8_TILE:
-            BSI_REQUIRE(value == 0 || value == 128 || value == 12864 || value == 64 || value == 6432,
-                        "tile must be 0, 128, 12864, 64 or 6432");
+            BSI_REQUIRE(value == 0 || value == 128 || value == 1284 || value == 12864 || value == 64 || value == 6432,
+                        "tile must be 0, 128, 1284, 12864, 64 or 6432");
             g_i8_tile = value;
             return BSI_OK;
         case BSI_OPT_BUILD_ITEMS:
@@ -2945,6 +3227,49 @@ extern "C" int bsi_hip_dot_digits(const int8_t* A_digits, int nq, const float* A
                        reinterpret_cast<const int*>(workspace), nq, nk, Q, R, preshift, Aw, Sa, Bw, Sb,
                        reinterpret_cast<const long long*>(key_indices), scale_inv, R_total, bias, out);
     BSI_LAUNCH_CHECK("digits_combine_kernel");
+    return BSI_OK;
+}
+
+extern "C" int bsi_hip_probe_l2_to_lds(const void* buf, size_t bytes, int loader_pattern, double* bytes_per_s, void* stream) {
+    BSI_REQUIRE(buf && bytes_per_s, "null pointer");
+    constexpr size_t kRegion = 256 * 1024;
+    constexpr int kRegions = 8, kPasses = 64;
+    BSI_REQUIRE(bytes >= kRegion * kRegions, "the probe streams %zu bytes of the buffer", kRegion * kRegions);
+    hipStream_t st = as_stream(stream);
+    int dev = 0, cus = 0;
+    BSI_HIP_CHECK(hipGetDevice(&dev));
+    BSI_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    const int lds = kProbeLdsWaves * kProbeLdsSlots * 1024;
+    static LdsOptIn once0, once1;
+    lds_opt_in(once0, reinterpret_cast<const void*>(&probe_l2_lds_kernel<8, 12, false>), lds);
+    lds_opt_in(once1, reinterpret_cast<const void*>(&probe_l2_lds_kernel<4, 24, true>), lds);
+    hipEvent_t e0, e1;
+    BSI_HIP_CHECK(hipEventCreate(&e0));
+    if (hipError_t ec = hipEventCreate(&e1); ec != hipSuccess) {
+        (void)hipEventDestroy(e0);
+        return fail(BSI_ERR_HIP, "hipEventCreate failed: %s", hipGetErrorString(ec));
+    }
+    float best = 1e30f;
+    hipError_t err = hipSuccess;
+    for (int rep = 0; rep < 4 && err == hipSuccess; ++rep) {  // the first repetition also brings the regions into L2
+        (void)hipEventRecord(e0, st);
+        if (loader_pattern)
+            hipLaunchKernelGGL((probe_l2_lds_kernel<4, 24, true>), dim3(static_cast<unsigned>(cus)), dim3(4 * 64), lds, st,
+                               static_cast<const unsigned char*>(buf), kRegion, kRegions, kPasses);
+        else
+            hipLaunchKernelGGL((probe_l2_lds_kernel<8, 12, false>), dim3(static_cast<unsigned>(cus)), dim3(8 * 64), lds, st,
+                               static_cast<const unsigned char*>(buf), kRegion, kRegions, kPasses);
+        (void)hipEventRecord(e1, st);
+        err = hipEventSynchronize(e1);
+        float ms = 0.0f;
+        if (err == hipSuccess) err = hipEventElapsedTime(&ms, e0, e1);
+        if (rep > 0 && ms < best) best = ms;
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    if (err != hipSuccess) return fail(BSI_ERR_HIP, "probe timing failed: %s", hipGetErrorString(err));
+    BSI_LAUNCH_CHECK("probe_l2_lds_kernel");
+    *bytes_per_s = static_cast<double>(cus) * kRegion * kPasses / (best * 1e-3);
     return BSI_OK;
 }
 
