@@ -2011,13 +2011,16 @@ __global__ __launch_bounds__(1024) void dot_mfma_stream_ewah_kernel(
     const int64_t tile = blockIdx.x;
     const unsigned long long* ksrc = B64 + static_cast<size_t>(tile) * chunks * (6 * 64) + lane;
 
-    // ---- inline EWAH decode: the group's streams round-robin over the waves
+    // ---- inline EWAH decode: the group's streams round-robin over the waves.  Three kinds of stream: all zero
+    // (nothing to do), verbatim (one marker followed by the W64 words of the slice: the words are read where they
+    // lie, straight from the stream, when their chunk comes up), anything else (expanded into LDS planes now).
     for (int s = wave; s < nstreams; s += nwaves) {
         const unsigned long long* in = comp + comp_off[q0 * Sa + s];
         const int in_len = comp_len[q0 * Sa + s];
         const bool zero = ewah_stream_is_zero(in, in_len, W64);
-        if (lane == 0) present[s] = zero ? 0 : 1;
-        if (!zero) ewah_expand_wave(in, in_len, W64, planes + static_cast<size_t>(s) * sstride, wpad, lane);
+        const bool verbatim = !zero && in_len == W64 + 1 && in[0] == (static_cast<unsigned long long>(W64) << 33);
+        if (lane == 0) present[s] = zero ? 0 : (verbatim ? 2 : 1);
+        if (!zero && !verbatim) ewah_expand_wave(in, in_len, W64, planes + static_cast<size_t>(s) * sstride, wpad, lane);
     }
     __syncthreads();
 
@@ -2029,12 +2032,21 @@ __global__ __launch_bounds__(1024) void dot_mfma_stream_ewah_kernel(
     const int sstep = (qscale_stride == 1) ? 0 : 1;
     const float* myscale = qscale + (q0 + (cn < nq ? cn : 0)) * qscale_stride;
     float accf = 0.0f;
-    // which of the lane's query's planes hold anything (bit t of the mask: row t of the 8 x 8 transposes)
-    unsigned have = 0;
+    // the planes of the lane's query (row t of the 8 x 8 transposes): expanded in LDS (have), verbatim in the stream (verb)
+    unsigned have = 0, verb = 0;
+    const unsigned long long* vptr[8];
 #pragma unroll
     for (int t = 0; t < 8; ++t) {
         const int j = t - (8 - Sa);
-        if (ln < nq && j >= 0 && present[ln * Sa + j]) have |= 1u << t;
+        vptr[t] = comp;
+        if (ln < nq && j >= 0) {
+            const int cls = present[ln * Sa + j];
+            if (cls == 1) have |= 1u << t;
+            if (cls == 2) {
+                verb |= 1u << t;
+                vptr[t] = comp + comp_off[(q0 + ln) * Sa + j] + 1;  // past the marker
+            }
+        }
     }
     const unsigned long long* myplanes = planes + static_cast<size_t>(ln < nq ? ln : 0) * Sa * sstride;
 
@@ -2052,7 +2064,9 @@ __global__ __launch_bounds__(1024) void dot_mfma_stream_ewah_kernel(
 #pragma unroll
             for (int t = 0; t < 8; ++t) {
                 const int j = t - (8 - Sa);
-                const unsigned long long w = ((have >> t) & 1u) ? myplanes[static_cast<size_t>(j) * sstride + c * 4 + lg] : 0ULL;
+                unsigned long long w = 0ULL;
+                if ((verb >> t) & 1u) w = (c * 4 + lg < W64) ? vptr[t][c * 4 + lg] : 0ULL;
+                else if ((have >> t) & 1u) w = myplanes[static_cast<size_t>(j) * sstride + c * 4 + lg];
                 qlo[t] = static_cast<uint32_t>(w);
                 qhi[t] = static_cast<uint32_t>(w >> 32);
             }
