@@ -28,6 +28,8 @@
 // kernel (bsi_ops/csrc/cuda/bsi_cuda_kernels_dot.cuh:1447-1540).
 #include "bsi_common.h"
 
+#include <type_traits>
+
 namespace bsi {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
@@ -800,6 +802,7 @@ static std::atomic<int> g_digits_route{0};  // bsi_hip_dot_digits: 0 = by cost, 
 
 template <int TM, int TN>
 struct I8Cfg {
+    static constexpr int kTM = TM, kTN = TN;
     static constexpr int kWM = TM / 32;                // 16-key tiles per wave (2 waves along the keys)
     static constexpr int kWN = 2;                      // 16-query tiles per wave
     static constexpr int kWavesN = TN / 32;            // waves along the queries
@@ -818,7 +821,7 @@ struct I8Cfg {
 // A loader wave of the int8-image kernels (lw = its number among the C::kLoaders loader waves; `consumers` MFMA
 // waves share the workgroup's barriers with it): 8 of the stage's groups of 8 rows (the TM key rows, then the TN
 // query rows: a load moves 1 KiB = 8 rows x 128 bytes), plus the chunk scales of 64 queries once per chunk.
-template <int TM, int TN, bool kSum>
+template <typename C, bool kSum>
 __device__ __forceinline__ void i8_loader_wave(unsigned char* __restrict__ lds, int lw, int lane,
                                                const int8_t* __restrict__ A8, const float* __restrict__ qscale,
                                                int qscale_stride, const int8_t* __restrict__ K8,
@@ -827,7 +830,7 @@ __device__ __forceinline__ void i8_loader_wave(unsigned char* __restrict__ lds, 
                                                const float* __restrict__ bias, int ndig, long long dig_stride,
                                                int key_tiled, const unsigned char* __restrict__ warm,
                                                long long warm_lines) {
-    using C = I8Cfg<TM, TN>;
+    constexpr int TM = C::kTM, TN = C::kTN;
     unsigned char* const scale_lds = lds + 4 * C::kStage;  // [chunk & 3][loader][64] floats
     // tiled keys: blocks of 64 rows x 128 bytes per half-chunk, 2 chunks of them per 64-row tile; rows past R
     // are zero padding inside the last block, blocks past the last one read as zero (buffer bounds)
@@ -954,6 +957,18 @@ __device__ __forceinline__ void i8_loader_wave(unsigned char* __restrict__ lds, 
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still be writing LDS when the workgroup ends
 }
 
+// The 128 x 128 tile with EIGHT loader waves of four loads per stage (the stage loads run faster the more waves
+// issue them); everything else as I8Cfg<128, 128>.
+struct I8CfgL8 {
+    static constexpr int kTM = 128, kTN = 128;
+    static constexpr int kGroups = 32, kLoaders = 8, kLoads = 4;
+    static constexpr int kOperandK = 128 * 128;
+    static constexpr int kStage = 256 * 128;
+    static constexpr int kScaleBytes = 4 * kLoaders * 256;
+    static constexpr int kEpilogueBytes = 2 * 128 * 4;
+    static constexpr int kLds = 4 * kStage + kScaleBytes + kEpilogueBytes;
+};
+
 // One k-step (64 of a chunk's 256 elements) of an MFMA wave: WM WN MFMAs on the operands in (ka, qb), one
 // epilogue element of the previous chunk (held in `prev`) behind each MFMA, and behind the first WM + WN of them
 // the reads of the NEXT k-step's operands into (ka_n, qb_n), so that the LDS latency of every k-step hides
@@ -985,12 +1000,52 @@ __device__ __forceinline__ void i8_kstep(const v4i (&ka)[WM], const v4i (&qb)[WN
                 if (kInts && ints_prev != nullptr && int_off[ea][eb] >= 0 && e < int_rows[ea])
                     ints_prev[int_off[ea][eb] + static_cast<int64_t>(e) * chunks] = prev[ea][eb][e] >> down_shift;
             }
-            // read number t of the next k-step, in the order its MFMAs first need them: ka[0], qb[0..], ka[1..]
-            if (t == 0) ka_n[0] = *reinterpret_cast<const v4i*>(krow_n);
-            else if (t <= WN) qb_n[t - 1] = *reinterpret_cast<const v4i*>(qrow_n + (t - 1) * 16 * 128);
-            else if (t < WM + WN) ka_n[t - WN] = *reinterpret_cast<const v4i*>(krow_n + (t - WN) * 16 * 128);
+            // reads 2 t and 2 t + 1 of the next k-step, in the order its MFMAs first need them: ka[0], qb[0..],
+            // ka[1..].  Two per MFMA: the last of them is then issued more than half a k-step before the barrier
+            // that may follow this k-step, which has to wait for all of them before it releases their stage.
+#pragma unroll
+            for (int r = 2 * t; r < 2 * t + 2; ++r) {
+                if (r == 0) ka_n[0] = *reinterpret_cast<const v4i*>(krow_n);
+                else if (r <= WN) qb_n[r - 1] = *reinterpret_cast<const v4i*>(qrow_n + (r - 1) * 16 * 128);
+                else if (r < WM + WN) ka_n[r - WN] = *reinterpret_cast<const v4i*>(krow_n + (r - WN) * 16 * 128);
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
+}
+
+// The output tile of an MFMA wave (WM x WN tiles of 16 keys x 16 queries; lane (ln, lg) holds keys 4 lg .. + 3 of
+// query ln of each) stored in whole 128-byte lines.  Stored as it lies, a store instruction writes 64 bytes per query
+// (4 lanes x 16 bytes): half a line.  Here neighbouring query lanes first swap one of two vertically adjacent tiles
+// (a, a + 1), so that the even lane holds keys 0 .. 15 of both queries and the odd lane keys 16 .. 31; a store then
+// writes, for one query of the pair, 8 lanes x 16 bytes = the 32 consecutive keys of a line.  Only for a tile that
+// lies wholly inside the output and whose lines are aligned; returns false (nothing stored) otherwise.
+template <int WM, int WN>
+__device__ __forceinline__ bool i8_store_lines(const float (&v)[WM][WN][4], float* __restrict__ out, int64_t R_total,
+                                               int64_t rw, int64_t qw, int64_t R, int64_t Q, int ln, int lg) {
+    static_assert(WM % 2 == 0, "tiles are paired along the keys");
+    const bool whole = rw + WM * 16 <= R && qw + WN * 16 <= Q && (R_total & 31) == 0 && (rw & 31) == 0 &&
+                       (reinterpret_cast<uintptr_t>(out) & 127) == 0;
+    if (!whole) return false;
+    const bool odd = (ln & 1) != 0;
+#pragma unroll
+    for (int a = 0; a < WM; a += 2)
+#pragma unroll
+        for (int b = 0; b < WN; ++b) {
+            float x[4], y[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float give = odd ? v[a][b][e] : v[a + 1][b][e];
+                // quad_perm [1, 0, 3, 2]: the value of the neighbouring query lane
+                const float got = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(give), 0xB1, 0xF, 0xF, false));
+                x[e] = odd ? got : v[a][b][e];       // the pair's even query: keys 16 (odd lane) + 4 lg ..
+                y[e] = odd ? v[a + 1][b][e] : got;   // the pair's odd query
+            }
+            const int64_t qe = qw + b * 16 + (ln & ~1);
+            float* dst = out + static_cast<size_t>(qe) * R_total + rw + a * 16 + (odd ? 16 : 0) + lg * 4;
+            *reinterpret_cast<float4*>(dst) = make_float4(x[0], x[1], x[2], x[3]);
+            *reinterpret_cast<float4*>(dst + R_total) = make_float4(y[0], y[1], y[2], y[3]);
+        }
+    return true;
 }
 
 template <int TM, int TN, int kMode>
@@ -1028,7 +1083,7 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
     unsigned char* const scale_lds = lds + 4 * C::kStage;  // [chunk & 3][loader][64] floats
 
     if (wave >= C::kConsumers) {
-        i8_loader_wave<TM, TN, kSum>(lds, wave - C::kConsumers, lane, A8, qscale, qscale_stride, K8, Bw, Sb, chunks, halves, R,
+        i8_loader_wave<C, kSum>(lds, wave - C::kConsumers, lane, A8, qscale, qscale_stride, K8, Bw, Sb, chunks, halves, R,
                                      Q, r0, q0, rowbytes, bias, ndig, dig_stride, key_tiled, warm, warm_lines);
         return;
     }
@@ -1264,8 +1319,7 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
         }
     }
 #pragma unroll
-    for (int a = 0; a < WM; ++a) {
-        const int64_t rb = r0 + wr * (WM * 16) + a * 16 + lg * 4;
+    for (int a = 0; a < WM; ++a)
 #pragma unroll
         for (int b = 0; b < WN; ++b)
 #pragma unroll
@@ -1275,6 +1329,10 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
                 if (bias != nullptr) v = v + bi[a][e];
                 accf[a][b][e] = v;
             }
+    if (i8_store_lines<WM, WN>(accf, out, R_total, r0 + wr * (WM * 16), q0 + wq * (WN * 16), R, Q, ln, lg)) return;
+#pragma unroll
+    for (int a = 0; a < WM; ++a) {
+        const int64_t rb = r0 + wr * (WM * 16) + a * 16 + lg * 4;
 #pragma unroll
         for (int b = 0; b < WN; ++b) {
             const int64_t q = q0 + wq * (WN * 16) + b * 16 + ln;
@@ -1291,77 +1349,89 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
     }
 }
 
-// ------------------------------------------------------------------ int8 image, four MFMA waves of 64 x 64
+// ------------------------------------------------------------------ int8 image, one accumulator set per MFMA wave
 //
-// The same workgroup tile (128 keys x 128 queries), ring, loader waves and epilogue as dot_mfma_i8_kernel<128, 128>,
-// with the arithmetic on FOUR MFMA waves of 64 keys x 64 queries (one per SIMD, next to its loader wave) instead of
-// eight of 64 x 32.  An MFMA wave's operand reads are (64 + 64) x 64 bytes per 64 x 64 x 64 MACs instead of
-// (64 + 32) x 64 per 64 x 32 x 64: a third fewer LDS bytes per MAC, on an LDS whose read port the eight-wave kernel
-// keeps as busy as its matrix pipes.  Eight waves of 256 registers hold one int32 accumulator set (64), the fp32
-// chain values (64) and two operand sets (64): there is no second accumulator set to park a finished chunk in, so
-// the chain step of chunk c (one cvt + one fma per output) runs on the accumulators in place, between a tile's last
-// MFMA of chunk c (k-step 3) and its first of chunk c + 1 (k-step 0, which starts from zero and overwrites it):
-// two elements behind each MFMA of k-step 3 from its third MFMA on (tiles 0..6), three behind each of the first
-// twelve MFMAs of the next k-step 0 (tiles 7..15), always tiles whose turn to be overwritten has not come.
-// Where a lane's accumulators go in the [Q, R, chunks] dump (parity checks): element (a, b, e) at
-// base + b * qstep + (a * 16 + e) * chunks, for the query columns of qmask and the first rows[a] key rows of tile a.
-struct I8WDump {
-    int64_t base, qstep;
-    int rows[4];
+// The same workgroup tile (128 keys x 128 queries), ring and epilogue as dot_mfma_i8_kernel<128, 128>, with MFMA waves
+// that keep ONE int32 accumulator set instead of two.  Without a second set to park a finished chunk in, the chain
+// step of chunk c (one cvt + one fma per output) runs on the accumulators in place, between a tile's last MFMA of
+// chunk c (k-step 3) and its first of chunk c + 1 (k-step 0, which starts from zero and overwrites it): two
+// elements behind each MFMA of k-step 3 from its third MFMA on, three behind each of the first MFMAs of the next
+// k-step 0, always of tiles whose turn to be overwritten has not come.  The 32 registers this frees per wave buy one
+// of two things (WN = 16-query tiles per MFMA wave):
+//   WN = 4  four MFMA waves of 64 keys x 64 queries (one per SIMD) + four loader waves, 256 registers each: an MFMA
+//           wave's operand reads are (64 + 64) x 64 bytes per 64 x 64 x 64 MACs instead of (64 + 32) x 64 per
+//           64 x 32 x 64, a third fewer LDS bytes per MAC;
+//   WN = 2  eight MFMA waves of 64 x 32 + EIGHT loader waves, 128 registers each: twice the waves issuing the stage
+//           loads, which is what sets the pace of the chunk loop.
+template <int WN>
+struct I8WDump {  // where a lane's accumulators go in the [Q, R, chunks] dump (parity checks): element (a, b, e) at
+    int64_t base, qstep;  // base + b * qstep + (a * 16 + e) * chunks, for the query columns of qmask and the
+    int rows[4];          // first rows[a] key rows of tile a
     unsigned qmask;
 };
-template <int KS, bool kInts>
-__device__ __forceinline__ void i8w_chain(int first, int count, const v4i (&acc)[4][4], float (&accf)[4][4][4],
-                                          const float (&qs)[4], int* __restrict__ ints_at, const I8WDump& dump,
+template <int WN, bool kInts>
+__device__ __forceinline__ void i8w_chain(int first, int count, const v4i (&acc)[4][WN], float (&accf)[4][WN][4],
+                                          const float (&qs)[WN], int* __restrict__ ints_at, const I8WDump<WN>& dump,
                                           int down_shift, int chunks) {
 #pragma unroll
     for (int i = first; i < first + count; ++i) {
-        const int tile = i >> 2, e = i & 3, a = tile >> 2, b = tile & 3;
+        if (i >= 16 * WN) break;
+        const int tile = i >> 2, e = i & 3, a = tile / WN, b = tile % WN;
         accf[a][b][e] = fmaf(static_cast<float>(acc[a][b][e]), qs[b], accf[a][b][e]);
         if (kInts && ints_at != nullptr && ((dump.qmask >> b) & 1u) && e < dump.rows[a])
             ints_at[dump.base + b * dump.qstep + static_cast<int64_t>(a * 16 + e) * chunks] = acc[a][b][e] >> down_shift;
     }
 }
 
-// One k-step of a 64 x 64 MFMA wave: 16 MFMAs (tile t = 4 a + b), the reads of the next k-step's eight operand
-// tiles behind the first eight, and the chain elements that fall to this k-step (see above).  qs_cur / ints_cur:
+// One k-step of such an MFMA wave: 4 WN MFMAs (tile t = WN a + b), the reads of the next k-step's 4 + WN operand
+// tiles behind the first of them, and the chain elements that fall to this k-step (see above).  qs_cur / ints_cur:
 // scales and accumulator dump of the chunk being computed (used by k-step 3); qs_prev / ints_prev: of the chunk
 // before it (used by k-step 0).
-template <int KS, bool kInts>
-__device__ __forceinline__ void i8w_kstep(const v4i (&ka)[4], const v4i (&qb)[4], v4i (&ka_n)[4], v4i (&qb_n)[4],
+template <int WN, int KS, bool kInts>
+__device__ __forceinline__ void i8w_kstep(const v4i (&ka)[4], const v4i (&qb)[WN], v4i (&ka_n)[4], v4i (&qb_n)[WN],
                                           const unsigned char* __restrict__ krow_n,
-                                          const unsigned char* __restrict__ qrow_n, v4i (&acc)[4][4],
-                                          float (&accf)[4][4][4], const float (&qs_cur)[4], const float (&qs_prev)[4],
-                                          int* __restrict__ ints_cur, int* __restrict__ ints_prev, const I8WDump& dump,
+                                          const unsigned char* __restrict__ qrow_n, v4i (&acc)[4][WN],
+                                          float (&accf)[4][WN][4], const float (&qs_cur)[WN], const float (&qs_prev)[WN],
+                                          int* __restrict__ ints_cur, int* __restrict__ ints_prev, const I8WDump<WN>& dump,
                                           int down_shift, int chunks) {
+    constexpr int NT = 4 * WN;            // tiles of the wave
+    constexpr int kLate = 2 * (NT - 2);   // chain elements k-step 3 takes care of; the rest fall to the next k-step 0
 #pragma unroll
-    for (int t = 0; t < 16; ++t) {
-        const int a = t >> 2, b = t & 3;
+    for (int t = 0; t < NT; ++t) {
+        const int a = t / WN, b = t % WN;
         const v4i c0 = (KS == 0) ? (v4i){0, 0, 0, 0} : acc[a][b];
         acc[a][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ka[a], qb[b], c0, 0, 0, 0);
-        // read number t of the next k-step, in the order its MFMAs first need them: ka[0], qb[0..3], ka[1..3]
+        // read number t of the next k-step, in the order its MFMAs first need them: ka[0], qb[0 ..], ka[1 ..]
         if (t == 0) ka_n[0] = *reinterpret_cast<const v4i*>(krow_n);
-        else if (t <= 4) qb_n[t - 1] = *reinterpret_cast<const v4i*>(qrow_n + (t - 1) * 16 * 128);
-        else if (t < 8) ka_n[t - 4] = *reinterpret_cast<const v4i*>(krow_n + (t - 4) * 16 * 128);
-        if (KS == 0 && t < 12)  // elements 28 + 3 t .. + 2 of the previous chunk: tiles 7 .. 15, none of them below t + 1
-            i8w_chain<KS, kInts>(28 + 3 * t, 3, acc, accf, qs_prev, ints_prev, dump, down_shift, chunks);
-        if (KS == 3 && t >= 2)  // elements 2 (t - 2), + 1 of this chunk: tiles 0 .. 6, finished two MFMAs ago or earlier
-            i8w_chain<KS, kInts>(2 * (t - 2), 2, acc, accf, qs_cur, ints_cur, dump, down_shift, chunks);
+        else if (t <= WN) qb_n[t - 1] = *reinterpret_cast<const v4i*>(qrow_n + (t - 1) * 16 * 128);
+        else if (t < 4 + WN) ka_n[t - WN] = *reinterpret_cast<const v4i*>(krow_n + (t - WN) * 16 * 128);
+        if (KS == 0 && kLate + 3 * t < 4 * NT)  // three elements of the previous chunk, of tiles above t
+            i8w_chain<WN, kInts>(kLate + 3 * t, 3, acc, accf, qs_prev, ints_prev, dump, down_shift, chunks);
+        if (KS == 3 && t >= 2)  // two elements of this chunk, of tiles finished two MFMAs ago or earlier
+            i8w_chain<WN, kInts>(2 * (t - 2), 2, acc, accf, qs_cur, ints_cur, dump, down_shift, chunks);
         __builtin_amdgcn_sched_barrier(0);
     }
 }
 
-constexpr int kI8WConsumers = 4;
-constexpr int kI8WBlock = (kI8WConsumers + I8Cfg<128, 128>::kLoaders) * 64;
+template <int WN>
+struct I8WCfg {
+    using Tile = typename std::conditional<WN == 4, I8Cfg<128, 128>, I8CfgL8>::type;  // LDS layout and loader waves
+    static constexpr int kWavesN = 128 / (16 * WN);      // MFMA waves along the queries (2 along the keys)
+    static constexpr int kConsumers = 2 * kWavesN;
+    static constexpr int kBlock = (kConsumers + Tile::kLoaders) * 64;
+};
 
-template <bool kInts>
-__global__ __launch_bounds__(kI8WBlock) void dot_mfma_i8w_kernel(
+template <int WN, bool kInts>
+__global__ __launch_bounds__((I8WCfg<WN>::kBlock)) void dot_mfma_i8w_kernel(
     const int8_t* __restrict__ A8, const float* __restrict__ qscale, int qscale_stride, const int8_t* __restrict__ K8,
     const float* __restrict__ Bw, int Sb, int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv,
     int64_t R_total, float* __restrict__ out, int* __restrict__ chunk_ints, const float* __restrict__ bias,
     int key_tiled, const unsigned char* __restrict__ warm, long long warm_lines) {
     constexpr int TM = 128, TN = 128;
-    using C = I8Cfg<TM, TN>;
+    using W = I8WCfg<WN>;
+    using C = typename W::Tile;
+    constexpr int kNE = 16 * WN;          // chain elements per lane and chunk
+    constexpr int kLate = 2 * (4 * WN - 2);
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];  // C::kLds
 
     const int tid = threadIdx.x;
@@ -1373,34 +1443,34 @@ __global__ __launch_bounds__(kI8WBlock) void dot_mfma_i8w_kernel(
     const int halves = chunks * 2;
     unsigned char* const scale_lds = lds + 4 * C::kStage;
 
-    if (wave >= kI8WConsumers) {
-        i8_loader_wave<TM, TN, false>(lds, wave - kI8WConsumers, lane, A8, qscale, qscale_stride, K8, Bw, Sb, chunks, halves,
-                                      R, Q, r0, q0, rowbytes, bias, 1, 0, key_tiled, warm, warm_lines);
+    if (wave >= W::kConsumers) {
+        i8_loader_wave<C, false>(lds, wave - W::kConsumers, lane, A8, qscale, qscale_stride, K8, Bw, Sb, chunks, halves, R, Q,
+                                 r0, q0, rowbytes, bias, 1, 0, key_tiled, warm, warm_lines);
         return;
     }
 
-    // ---- MFMA waves: wr = half of the keys, wq = half of the queries
+    // ---- MFMA waves: wr = half of the keys, wq = group of 16 WN queries
     const int wr = wave & 1, wq = wave >> 1;
     const int ln = lane & 15, lg = lane >> 4;
     const int krow_off = (wr * 64 + ln) * 128;
-    const int qrow_off = C::kOperandK + (wq * 64 + ln) * 128;
+    const int qrow_off = C::kOperandK + (wq * (16 * WN) + ln) * 128;
     int pcol[2];
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) pcol[kk] = ((kk * 4 + lg) ^ (ln >> 1)) * 16;
-    float accf[4][4][4];
-    v4i acc[4][4];
+    float accf[4][WN][4];
+    v4i acc[4][WN];
 #pragma unroll
     for (int a = 0; a < 4; ++a)
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
+        for (int b = 0; b < WN; ++b) {
             acc[a][b] = (v4i){0, 0, 0, 0};
 #pragma unroll
             for (int e = 0; e < 4; ++e) accf[a][b][e] = 0.0f;
         }
     const float down = __uint_as_float(static_cast<uint32_t>(127 - down_shift) << 23);
-    I8WDump dump;
+    I8WDump<WN> dump;
     {
-        const int64_t rl = r0 + wr * 64 + lg * 4, ql = q0 + wq * 64 + ln;  // the lane's first key row and query column
+        const int64_t rl = r0 + wr * 64 + lg * 4, ql = q0 + wq * (16 * WN) + ln;  // the lane's first key row and query column
         dump.base = (ql * R + rl) * chunks;
         dump.qstep = 16 * R * chunks;
         dump.qmask = 0;
@@ -1410,25 +1480,26 @@ __global__ __launch_bounds__(kI8WBlock) void dot_mfma_i8w_kernel(
             dump.rows[a] = static_cast<int>(left < 0 ? 0 : (left < 4 ? left : 4));
         }
 #pragma unroll
-        for (int b = 0; b < 4; ++b)
+        for (int b = 0; b < WN; ++b)
             if (kInts && ql + b * 16 < Q) dump.qmask |= 1u << b;
     }
-    // chunk scales of the lane's four query columns, from the loaders' ring: region wq holds queries 64 wq .. + 63
-    const unsigned char* sread = scale_lds + wq * 256 + ln * 4;
-    float qsa[4], qsb[4];  // scales of even / odd chunks (all zero before the first chunk: its "previous" chain adds 0)
+    // chunk scales of the lane's query columns, from the loaders' ring: 64 queries per region, region g = queries 64 g ..
+    const int qfirst = wq * (16 * WN);
+    const unsigned char* sread = scale_lds + (qfirst >> 6) * 256 + ((qfirst & 63) + ln) * 4;
+    float qsa[WN], qsb[WN];  // scales of even / odd chunks (all zero before the first chunk: its "previous" chain adds 0)
 #pragma unroll
-    for (int b = 0; b < 4; ++b) qsa[b] = qsb[b] = 0.0f;
+    for (int b = 0; b < WN; ++b) qsa[b] = qsb[b] = 0.0f;
 #define BSI_I8W_SCALES(dst, c)                                                                         \
     {                                                                                                  \
-        _Pragma("unroll") for (int b = 0; b < 4; ++b) dst[b] =                                         \
+        _Pragma("unroll") for (int b = 0; b < WN; ++b) dst[b] =                                        \
             *reinterpret_cast<const float*>(sread + ((c) & 3) * (C::kLoaders * 256) + b * 64);         \
     }
-    v4i ka[2][4], qb[2][4];  // operand sets of even / odd k-steps
+    v4i ka[2][4], qb[2][WN];  // operand sets of even / odd k-steps
 #define BSI_I8W_KSTEP(KS, nslot, qc, qp, ic, ip)                                                                    \
-    i8w_kstep<KS, kInts>(ka[(KS) & 1], qb[(KS) & 1], ka[((KS) + 1) & 1], qb[((KS) + 1) & 1],                        \
-                         lds + (nslot) * C::kStage + krow_off + pcol[((KS) + 1) & 1],                               \
-                         lds + (nslot) * C::kStage + qrow_off + pcol[((KS) + 1) & 1], acc, accf, qc, qp, ic, ip,    \
-                         dump, down_shift, chunks);
+    i8w_kstep<WN, KS, kInts>(ka[(KS) & 1], qb[(KS) & 1], ka[((KS) + 1) & 1], qb[((KS) + 1) & 1],                    \
+                             lds + (nslot) * C::kStage + krow_off + pcol[((KS) + 1) & 1],                           \
+                             lds + (nslot) * C::kStage + qrow_off + pcol[((KS) + 1) & 1], acc, accf, qc, qp, ic, ip, \
+                             dump, down_shift, chunks);
     // a chunk whose halves sit in ring slots s0, s0 + 1; nslot: slot of the next chunk's first half; qc / qp: this
     // chunk's and the previous chunk's scales.  This chunk's scales have landed with its second half, which the
     // first barrier announces.
@@ -1445,7 +1516,7 @@ __global__ __launch_bounds__(kI8WBlock) void dot_mfma_i8w_kernel(
 #pragma unroll
     for (int t = 0; t < 4; ++t) ka[0][t] = *reinterpret_cast<const v4i*>(lds + krow_off + t * 16 * 128 + pcol[0]);
 #pragma unroll
-    for (int t = 0; t < 4; ++t) qb[0][t] = *reinterpret_cast<const v4i*>(lds + qrow_off + t * 16 * 128 + pcol[0]);
+    for (int t = 0; t < WN; ++t) qb[0][t] = *reinterpret_cast<const v4i*>(lds + qrow_off + t * 16 * 128 + pcol[0]);
     __builtin_amdgcn_sched_barrier(0);
     int c = 0;
     for (; c + 1 < chunks; c += 2) {
@@ -1463,9 +1534,9 @@ __global__ __launch_bounds__(kI8WBlock) void dot_mfma_i8w_kernel(
 #undef BSI_I8W_CHUNK
 #undef BSI_I8W_KSTEP
 #undef BSI_I8W_SCALES
-    // the chain elements of the last chunk that its k-step 3 left (28 .. 63)
-    if (last_even) i8w_chain<0, kInts>(28, 36, acc, accf, qsa, chunk_ints + (chunks - 1), dump, down_shift, chunks);
-    else i8w_chain<0, kInts>(28, 36, acc, accf, qsb, chunk_ints + (chunks - 1), dump, down_shift, chunks);
+    // the chain elements of the last chunk that its k-step 3 left
+    if (last_even) i8w_chain<WN, kInts>(kLate, kNE - kLate, acc, accf, qsa, chunk_ints + (chunks - 1), dump, down_shift, chunks);
+    else i8w_chain<WN, kInts>(kLate, kNE - kLate, acc, accf, qsb, chunk_ints + (chunks - 1), dump, down_shift, chunks);
     // key factors and biases from the copy the loader waves staged in LDS
     float bs[4][4], bi[4][4];
     {
@@ -1480,25 +1551,30 @@ __global__ __launch_bounds__(kI8WBlock) void dot_mfma_i8w_kernel(
         }
     }
 #pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < WN; ++b)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float v = ((accf[a][b][e] * down) * bs[a][e]) * scale_inv;
+                if (bias != nullptr) v = v + bi[a][e];
+                accf[a][b][e] = v;
+            }
+    if (i8_store_lines<4, WN>(accf, out, R_total, r0 + wr * 64, q0 + wq * (16 * WN), R, Q, ln, lg)) return;
+#pragma unroll
     for (int a = 0; a < 4; ++a) {
         const int64_t rb = r0 + wr * 64 + a * 16 + lg * 4;
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
-            const int64_t q = q0 + wq * 64 + b * 16 + ln;
-            float v[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                v[e] = ((accf[a][b][e] * down) * bs[a][e]) * scale_inv;
-                if (bias != nullptr) v[e] = v[e] + bi[a][e];
-            }
+        for (int b = 0; b < WN; ++b) {
+            const int64_t q = q0 + wq * (16 * WN) + b * 16 + ln;
             if (q >= Q) continue;
             float* dst = out + static_cast<size_t>(q) * R_total + rb;
             if (rb + 3 < R && ((reinterpret_cast<uintptr_t>(dst) & 15) == 0)) {
-                *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+                *reinterpret_cast<float4*>(dst) = make_float4(accf[a][b][0], accf[a][b][1], accf[a][b][2], accf[a][b][3]);
             } else {
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
-                    if (rb + e < R) dst[e] = v[e];
+                    if (rb + e < R) dst[e] = accf[a][b][e];
             }
         }
     }
@@ -2514,22 +2590,25 @@ static void launch_mfma_i8_t(int ndig, long long dig_stride, const long long* ke
                                             R_total, out, chunk_ints, bias, st, 1, 0, nullptr, key_tiled);
 }
 
-// The 128 x 128 tile on four MFMA waves of 64 x 64 (chain modes only).
+// The 128 x 128 tile on MFMA waves with one accumulator set (chain modes only): WN = 4, four MFMA waves of 64 x 64 and
+// four loader waves (tile 1284); WN = 2, eight MFMA waves of 64 x 32 and eight loader waves (tile 1288).
+template <int WN>
 static void launch_mfma_i8w(const int8_t* A8, const float* qscale, int stride, const int8_t* K8, const float* Bw, int Sb,
                             int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv, int64_t R_total, float* out,
                             int32_t* chunk_ints, const float* bias, hipStream_t st, int key_tiled) {
-    using C = I8Cfg<128, 128>;
+    using W = I8WCfg<WN>;
+    using C = typename W::Tile;
     const dim3 grid(static_cast<unsigned>((R + 127) / 128), static_cast<unsigned>((Q + 127) / 128));
     static LdsOptIn once0, once1;
-    lds_opt_in(once0, reinterpret_cast<const void*>(&dot_mfma_i8w_kernel<false>), C::kLds);
-    lds_opt_in(once1, reinterpret_cast<const void*>(&dot_mfma_i8w_kernel<true>), C::kLds);
+    lds_opt_in(once0, reinterpret_cast<const void*>(&dot_mfma_i8w_kernel<WN, false>), C::kLds);
+    lds_opt_in(once1, reinterpret_cast<const void*>(&dot_mfma_i8w_kernel<WN, true>), C::kLds);
     const unsigned char* warm = static_cast<const unsigned char*>(g_warm_ptr);
     const long long warm_lines = static_cast<long long>(g_warm_bytes / 128);
     if (chunk_ints)
-        hipLaunchKernelGGL((dot_mfma_i8w_kernel<true>), grid, dim3(kI8WBlock), C::kLds, st, A8, qscale, stride, K8, Bw, Sb,
+        hipLaunchKernelGGL((dot_mfma_i8w_kernel<WN, true>), grid, dim3(W::kBlock), C::kLds, st, A8, qscale, stride, K8, Bw, Sb,
                            chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias, key_tiled, warm, warm_lines);
     else
-        hipLaunchKernelGGL((dot_mfma_i8w_kernel<false>), grid, dim3(kI8WBlock), C::kLds, st, A8, qscale, stride, K8, Bw, Sb,
+        hipLaunchKernelGGL((dot_mfma_i8w_kernel<WN, false>), grid, dim3(W::kBlock), C::kLds, st, A8, qscale, stride, K8, Bw, Sb,
                            chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias, key_tiled, warm, warm_lines);
 }
 
@@ -2559,13 +2638,17 @@ static void launch_mfma_i8(const int8_t* A8, const float* qscale, int stride, co
                            float* out, int32_t* chunk_ints, const float* bias, hipStream_t st, int key_tiled = 0,
                            int ndig = 0, long long dig_stride = 0, const long long* key_indices = nullptr) {
     const int tile = choose_i8_tile(R, Q);
-    if (tile == 1284 && ndig == 0) {
-        launch_mfma_i8w(A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias,
-                        st, key_tiled);
+    if ((tile == 1284 || tile == 1288) && ndig == 0) {
+        if (tile == 1284)
+            launch_mfma_i8w<4>(A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints,
+                               bias, st, key_tiled);
+        else
+            launch_mfma_i8w<2>(A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints,
+                               bias, st, key_tiled);
         return;
     }
 #define BSI_I8_ARGS ndig, dig_stride, key_indices, key_tiled, A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias, st
-    if (tile == 128 || tile == 1284) launch_mfma_i8_t<128, 128>(BSI_I8_ARGS);
+    if (tile == 128 || tile == 1284 || tile == 1288) launch_mfma_i8_t<128, 128>(BSI_I8_ARGS);
     else if (tile == 12864) launch_mfma_i8_t<128, 64>(BSI_I8_ARGS);
     else if (tile == 64) launch_mfma_i8_t<64, 64>(BSI_I8_ARGS);
     else launch_mfma_i8_t<64, 32>(BSI_I8_ARGS);
@@ -2659,8 +2742,9 @@ extern "C" int bsi_hip_set_option(int option, int value) {
             g_digits_route = value;
             return BSI_OK;
         case BSI_OPT_I8_TILE:
-            BSI_REQUIRE(value == 0 || value == 128 || value == 1284 || value == 12864 || value == 64 || value == 6432,
-                        "tile must be 0, 128, 1284, 12864, 64 or 6432");
+            BSI_REQUIRE(value == 0 || value == 128 || value == 1284 || value == 1288 || value == 12864 || value == 64 ||
+                            value == 6432,
+                        "tile must be 0, 128, 1284, 1288, 12864, 64 or 6432");
             g_i8_tile = value;
             return BSI_OK;
         case BSI_OPT_BUILD_ITEMS:
