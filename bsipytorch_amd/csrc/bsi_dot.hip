@@ -831,10 +831,19 @@ __device__ __forceinline__ void i8_loader_wave(unsigned char* __restrict__ lds, 
                                                int key_tiled, const unsigned char* __restrict__ warm,
                                                long long warm_lines) {
     constexpr int TM = C::kTM, TN = C::kTN;
+    constexpr int L = C::kLoaders, NI = C::kLoads, KG = TM / 8, QG = TN / 8;
+    // When the key groups and the query groups both divide evenly among the loader waves, every loader moves KG / L
+    // key groups, then QG / L query groups: which operand a load belongs to is then known at compile time.
+    constexpr bool kEven = (KG % L == 0) && (QG % L == 0);
+    static_assert(!kEven || NI == KG / L + QG / L, "loads per loader wave");
     unsigned char* const scale_lds = lds + 4 * C::kStage;  // [chunk & 3][loader][64] floats
+    // The prologue below is kept short on purpose: it runs on one wave per SIMD while the whole workgroup waits for
+    // the first stage.  No row is clamped: a load that starts past its operand's end reads nothing (buffer bounds),
+    // and whatever such a row or query leaves in LDS only reaches outputs past R or Q, which are never stored.
     // tiled keys: blocks of 64 rows x 128 bytes per half-chunk, 2 chunks of them per 64-row tile; rows past R
-    // are zero padding inside the last block, blocks past the last one read as zero (buffer bounds)
-    const size_t kblock = static_cast<size_t>(chunks) * 2 * 8192;  // bytes of a 64-row tile
+    // are zero padding inside the last block
+    const uint32_t rowbytes32 = static_cast<uint32_t>(chunks) << 8;
+    const uint32_t kblock = static_cast<uint32_t>(chunks) << 14;  // bytes of a 64-row tile of the tiled image
     const bsi_rsrc rk = key_tiled ? make_rsrc(K8 + static_cast<size_t>(r0 / 64) * kblock,
                                               static_cast<size_t>((R + 63) / 64 - r0 / 64) * kblock)
                                   : make_rsrc(K8 + static_cast<size_t>(r0) * rowbytes,
@@ -842,49 +851,36 @@ __device__ __forceinline__ void i8_loader_wave(unsigned char* __restrict__ lds, 
     const bsi_rsrc rq = make_rsrc(A8 + static_cast<size_t>(q0) * rowbytes,
                                   static_cast<size_t>(Q - q0) * rowbytes +
                                       (kSum ? static_cast<size_t>(ndig - 1) * static_cast<size_t>(dig_stride) : 0));
-    const bsi_rsrc rs = make_rsrc(qscale + q0 * qscale_stride, static_cast<size_t>(Q - q0) * qscale_stride * 4);
-    if (!kSum) {
-        // The epilogue's operands, staged once per workgroup: the slice-0 weight (key factor) and the bias of the
-        // tile's TM keys, 64 rows per load.  Fetched per lane at the end they are 32 vector-memory instructions
-        // for every MFMA wave, half as many as the whole chunk loop issues, all queued in front of the stores.
-        // Issued first, they have landed before any stage has (loads return in order).  Rows past R, and the
-        // biases of a call without one, read nothing and give 0 (buffer bounds).
-        const bsi_rsrc wrs = make_rsrc(Bw + static_cast<size_t>(r0) * Sb, static_cast<size_t>(R - r0) * Sb * sizeof(float));
-        const bsi_rsrc brs = make_rsrc(bias != nullptr ? bias + r0 : Bw,
-                                       bias != nullptr ? static_cast<size_t>(R - r0) * sizeof(float) : 0);
-        unsigned char* const epi = lds + 4 * C::kStage + C::kScaleBytes;
-        for (int j = lw; j < 2 * (TM / 64); j += C::kLoaders) {
-            const bool is_bias = j >= TM / 64;
-            const int blk = is_bias ? j - TM / 64 : j;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(is_bias ? brs : wrs,
-                                                     BSI_LDS_PTR(epi + (is_bias ? TM * 4 : 0) + blk * 256), 4,
-                                                     (blk * 64 + lane) * (is_bias ? 4 : Sb * 4), 0, 0, 0);
-        }
-    }
-    // the stage has kGroups groups of 8 rows, keys first; loader lw moves groups lw, lw + kLoaders, ... (when
-    // the groups do not divide evenly the last load wraps around and fetches a group a second time, so that
-    // every loader wave has the same number of loads in flight)
-    constexpr int NI = C::kLoads;
-    uint32_t off[NI];
+    // A load moves group g of the stage: 8 rows x 128 bytes; lane = (row lr of the group, 16-byte column lc), and the
+    // logical column that lands in LDS column lc of row 8 g + lr is lc ^ (((8 g + lr) >> 1) & 7) = lc ^ (4 (g & 1) +
+    // (lr >> 1)).  Per lane: the offset inside the group, for either parity of g and for either layout; per load
+    // (scalar): the offset of its group.
+    const uint32_t lr = static_cast<uint32_t>(lane) >> 3, lc = static_cast<uint32_t>(lane) & 7;
+    uint32_t voff[NI], goff[NI];
     bool is_key[NI];  // wave-uniform
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
-        const int g = (lw + C::kLoaders * i) % C::kGroups;
-        is_key[i] = g < TM / 8;
-        const int rowl = (is_key[i] ? g : g - TM / 8) * 8 + (lane >> 3);  // row of its operand tile
-        const uint32_t col = static_cast<uint32_t>((lane & 7) ^ ((rowl >> 1) & 7)) * 16;  // logical column landing here
-        const int64_t lim = is_key[i] ? (R - r0) : (Q - q0);              // past the end: clamp (never stored)
-        const int64_t rr = (rowl < lim) ? rowl : (lim - 1);
-        off[i] = static_cast<uint32_t>(rr * rowbytes) + col;
-        if (is_key[i] && key_tiled)
-            off[i] = static_cast<uint32_t>(rowl >> 6) * static_cast<uint32_t>(kblock) +
-                     static_cast<uint32_t>(rowl & 63) * 128 + col;
+        int g, gg;  // group of the stage, group of its operand
+        if (kEven) {
+            is_key[i] = i < KG / L;
+            gg = is_key[i] ? lw + L * i : lw + L * (i - KG / L);
+            g = is_key[i] ? gg : gg + KG;
+        } else {  // the last load wraps around and fetches a group a second time: the same number of loads per wave
+            g = (lw + L * i) % C::kGroups;
+            is_key[i] = g < KG;
+            gg = is_key[i] ? g : g - KG;
+        }
+        const uint32_t col = (lc ^ (static_cast<uint32_t>(gg & 1) * 4 + (lr >> 1))) * 16;
+        const bool tiled = is_key[i] && key_tiled;
+        voff[i] = (tiled ? lr * 128 : lr * rowbytes32) + col;
+        goff[i] = tiled ? static_cast<uint32_t>(gg >> 3) * kblock + static_cast<uint32_t>(gg & 7) * 1024
+                        : static_cast<uint32_t>(gg) * 8 * rowbytes32;
     }
     const uint32_t kstep_bytes = key_tiled ? 8192u : 128u;  // from one half-chunk of a key row to the next
     // scales: loader wave lw fetches the 64 queries of group lw % (TN / 64) (waves fetching the same group
     // write their own regions, so that every loader wave has the same number of loads in flight)
-    const int sq = (lw % (TN >= 64 ? TN / 64 : 1)) * 64 + lane;
-    const uint32_t soff = static_cast<uint32_t>(((q0 + sq < Q) ? sq : (Q - 1 - q0)) * qscale_stride * 4);
+    const bsi_rsrc rs = make_rsrc(qscale + q0 * qscale_stride, static_cast<size_t>(Q - q0) * qscale_stride * 4);
+    const uint32_t soff = static_cast<uint32_t>((lw % (TN >= 64 ? TN / 64 : 1)) * 64 + lane) * static_cast<uint32_t>(qscale_stride) * 4;
     const int sstep = (qscale_stride == 1) ? 0 : 4;
     // issue() is called for h = 0, 1, 2, ... in order; in the sum mode (next_c, next_dg) follow the chunk and
     // the digit (counted from the top one) of the half-chunk to come
@@ -909,9 +905,11 @@ __device__ __forceinline__ void i8_loader_wave(unsigned char* __restrict__ lds, 
             so_k = static_cast<uint32_t>(hc) * kstep_bytes;
         }
 #pragma unroll
-        for (int i = 0; i < NI; ++i)
-            load16_to_lds(is_key[i] ? rk : rq, off[i], is_key[i] ? so_k : so_q,
-                          lds + (h & 3) * C::kStage + ((lw + C::kLoaders * i) % C::kGroups) * 1024);
+        for (int i = 0; i < NI; ++i) {
+            const int g = kEven ? (i < KG / L ? lw + L * i : KG + lw + L * (i - KG / L)) : (lw + L * i) % C::kGroups;
+            load16_to_lds(is_key[i] ? rk : rq, voff[i], goff[i] + (is_key[i] ? so_k : so_q),
+                          lds + (h & 3) * C::kStage + g * 1024);
+        }
         if (!kSum && (h & 1)) {  // with the second half of chunk c = h / 2: its scales
             const int c = hc >> 1;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(
@@ -922,8 +920,29 @@ __device__ __forceinline__ void i8_loader_wave(unsigned char* __restrict__ lds, 
     issue(0);
     issue(1);
     issue(2);
-    // stage 0 landed (stage 1 + scales + stage 2, 2 NI + 1 instructions, may be in flight)
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NI + (kSum ? 0 : 1)) : "memory");
+    // The epilogue's operands, staged once per workgroup behind the first three stages: the slice-0 weight (key
+    // factor) and the bias of the tile's TM keys, 64 rows per load.  (Fetched per lane at the end they are 32
+    // vector-memory instructions for every MFMA wave, all queued in front of the output stores.)  Every loader wave
+    // issues kEpi of them -- wrapping around where they do not divide evenly -- so that the waits below count the
+    // same for all.  Rows past R, and the biases of a call without one, read nothing and give 0 (buffer bounds).
+    constexpr int kEpi = kSum ? 0 : (2 * (TM / 64) + L - 1) / L;
+    if (!kSum) {
+        const bsi_rsrc wrs = make_rsrc(Bw + static_cast<size_t>(r0) * Sb, static_cast<size_t>(R - r0) * Sb * sizeof(float));
+        const bsi_rsrc brs = make_rsrc(bias != nullptr ? bias + r0 : Bw,
+                                       bias != nullptr ? static_cast<size_t>(R - r0) * sizeof(float) : 0);
+        unsigned char* const epi = lds + 4 * C::kStage + C::kScaleBytes;
+#pragma unroll
+        for (int k = 0; k < kEpi; ++k) {
+            const int j = (lw + L * k) % (2 * (TM / 64));
+            const bool is_bias = j >= TM / 64;
+            const int blk = is_bias ? j - TM / 64 : j;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(is_bias ? brs : wrs,
+                                                     BSI_LDS_PTR(epi + (is_bias ? TM * 4 : 0) + blk * 256), 4,
+                                                     (blk * 64 + lane) * (is_bias ? 4 : Sb * 4), 0, 0, 0);
+        }
+    }
+    // stage 0 landed (stage 1 + scales + stage 2 + the epilogue operands may be in flight)
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NI + (kSum ? 0 : 1) + kEpi) : "memory");
     lds_barrier();
     for (int h = 0; h < halves; ++h) {
         if (h + 3 < halves) {
@@ -1042,8 +1061,9 @@ __device__ __forceinline__ bool i8_store_lines(const float (&v)[WM][WN][4], floa
             }
             const int64_t qe = qw + b * 16 + (ln & ~1);
             float* dst = out + static_cast<size_t>(qe) * R_total + rw + a * 16 + (odd ? 16 : 0) + lg * 4;
-            *reinterpret_cast<float4*>(dst) = make_float4(x[0], x[1], x[2], x[3]);
-            *reinterpret_cast<float4*>(dst + R_total) = make_float4(y[0], y[1], y[2], y[3]);
+            typedef float v4f __attribute__((ext_vector_type(4)));
+            __builtin_nontemporal_store((v4f){x[0], x[1], x[2], x[3]}, reinterpret_cast<v4f*>(dst));
+            __builtin_nontemporal_store((v4f){y[0], y[1], y[2], y[3]}, reinterpret_cast<v4f*>(dst + R_total));
         }
     return true;
 }
@@ -3338,9 +3358,12 @@ extern "C" int bsi_hip_probe_l2_to_lds(const void* buf, size_t bytes, int loader
     BSI_HIP_CHECK(hipGetDevice(&dev));
     BSI_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
     const int lds = kProbeLdsWaves * kProbeLdsSlots * 1024;
-    static LdsOptIn once0, once1;
+    BSI_REQUIRE(loader_pattern >= 0 && loader_pattern <= 3, "loader_pattern must be 0, 1, 2 or 3");
+    static LdsOptIn once0, once1, once2, once3;
     lds_opt_in(once0, reinterpret_cast<const void*>(&probe_l2_lds_kernel<8, 12, false>), lds);
     lds_opt_in(once1, reinterpret_cast<const void*>(&probe_l2_lds_kernel<4, 24, true>), lds);
+    lds_opt_in(once2, reinterpret_cast<const void*>(&probe_l2_lds_kernel<4, 24, false>), lds);
+    lds_opt_in(once3, reinterpret_cast<const void*>(&probe_l2_lds_kernel<8, 12, true>), lds);
     hipEvent_t e0, e1;
     BSI_HIP_CHECK(hipEventCreate(&e0));
     if (hipError_t ec = hipEventCreate(&e1); ec != hipSuccess) {
@@ -3351,8 +3374,14 @@ extern "C" int bsi_hip_probe_l2_to_lds(const void* buf, size_t bytes, int loader
     hipError_t err = hipSuccess;
     for (int rep = 0; rep < 4 && err == hipSuccess; ++rep) {  // the first repetition also brings the regions into L2
         (void)hipEventRecord(e0, st);
-        if (loader_pattern)
+        if (loader_pattern == 1)
             hipLaunchKernelGGL((probe_l2_lds_kernel<4, 24, true>), dim3(static_cast<unsigned>(cus)), dim3(4 * 64), lds, st,
+                               static_cast<const unsigned char*>(buf), kRegion, kRegions, kPasses);
+        else if (loader_pattern == 2)
+            hipLaunchKernelGGL((probe_l2_lds_kernel<4, 24, false>), dim3(static_cast<unsigned>(cus)), dim3(4 * 64), lds, st,
+                               static_cast<const unsigned char*>(buf), kRegion, kRegions, kPasses);
+        else if (loader_pattern == 3)
+            hipLaunchKernelGGL((probe_l2_lds_kernel<8, 12, true>), dim3(static_cast<unsigned>(cus)), dim3(8 * 64), lds, st,
                                static_cast<const unsigned char*>(buf), kRegion, kRegions, kPasses);
         else
             hipLaunchKernelGGL((probe_l2_lds_kernel<8, 12, false>), dim3(static_cast<unsigned>(cus)), dim3(8 * 64), lds, st,

@@ -373,7 +373,8 @@ int bsi_hip_probe_stream_read(const void* buf_device, size_t bytes, double* byte
  * 2 MiB are read) into LDS with LDS-direct 16-byte buffer loads, 96 KiB in flight per CU, all CUs at once; the result
  * is the aggregate rate over all CUs in bytes per second.  loader_pattern = 0: eight issuing waves per CU, contiguous
  * 1 KiB pieces (the path's best); 1: four issuing waves and pieces of 8 rows x 128 bytes out of 2 KiB rows, as the
- * kernel's four loader waves issue them.  Synchronises. */
+ * loader waves fetch a row-major operand; 2: four issuing waves, contiguous pieces; 3: eight issuing waves, row
+ * pieces.  Synchronises. */
 int bsi_hip_probe_l2_to_lds(const void* buf_device, size_t bytes, int loader_pattern, double* bytes_per_s, void* stream);
 
 #ifdef __cplusplus
