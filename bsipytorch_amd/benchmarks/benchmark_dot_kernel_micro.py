@@ -97,8 +97,8 @@ def main() -> None:
     p.add_argument("--relu", action="store_true", help="ReLU the queries (about half exact zeros)")
     p.add_argument("--planes_only", action="store_true", help="do not hand the builder's int8 queries to the dot")
     p.add_argument("--report_stats", action="store_true")
-    p.add_argument("--i8_tile", type=int, default=0, choices=[0, 128, 1284, 1288, 12864, 64, 6432],
-                   help="force a tile of the int8-image kernel (1284 / 1288: 128 x 128 on four MFMA waves of 64 x 64 / eight of 64 x 32 with eight loader waves); 0 = automatic")
+    p.add_argument("--i8_tile", type=int, default=0, choices=[0, 128, 1284, 12864, 64, 6432],
+                   help="force a tile of the int8-image kernel (1284: 128 x 128 on four MFMA waves of 64 x 64); 0 = automatic")
     a = p.parse_args()
     if not torch.cuda.is_available():
         raise RuntimeError("a GPU is required for this microbench")

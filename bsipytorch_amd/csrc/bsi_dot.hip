@@ -976,18 +976,6 @@ __device__ __forceinline__ void i8_loader_wave(unsigned char* __restrict__ lds, 
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still be writing LDS when the workgroup ends
 }
 
-// The 128 x 128 tile with EIGHT loader waves of four loads per stage (the stage loads run faster the more waves
-// issue them); everything else as I8Cfg<128, 128>.
-struct I8CfgL8 {
-    static constexpr int kTM = 128, kTN = 128;
-    static constexpr int kGroups = 32, kLoaders = 8, kLoads = 4;
-    static constexpr int kOperandK = 128 * 128;
-    static constexpr int kStage = 256 * 128;
-    static constexpr int kScaleBytes = 4 * kLoaders * 256;
-    static constexpr int kEpilogueBytes = 2 * 128 * 4;
-    static constexpr int kLds = 4 * kStage + kScaleBytes + kEpilogueBytes;
-};
-
 // One k-step (64 of a chunk's 256 elements) of an MFMA wave: WM WN MFMAs on the operands in (ka, qb), one
 // epilogue element of the previous chunk (held in `prev`) behind each MFMA, and behind the first WM + WN of them
 // the reads of the NEXT k-step's operands into (ka_n, qb_n), so that the LDS latency of every k-step hides
@@ -1265,25 +1253,30 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
                 }
             }
 #pragma unroll
+            for (int a = 0; a < WM; ++a)
+#pragma unroll
+                for (int b = 0; b < WN; ++b)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        float v = static_cast<float>(static_cast<double>(acc0[a][b][e]) * qf[b] * static_cast<double>(kfv[a][e])) * scale_inv;
+                        if (bias != nullptr) v = v + biv[a][e];
+                        accf[a][b][e] = v;
+                    }
+            if (i8_store_lines<WM, WN>(accf, out, R_total, r0 + wr * (WM * 16), q0 + wq * (WN * 16), R, Q, ln, lg)) return;
+#pragma unroll
             for (int a = 0; a < WM; ++a) {
                 const int64_t rb = r0 + wr * (WM * 16) + a * 16 + lg * 4;
 #pragma unroll
                 for (int b = 0; b < WN; ++b) {
                     const int64_t q = q0 + wq * (WN * 16) + b * 16 + ln;
                     if (q >= Q) continue;
-                    float v[4];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        v[e] = static_cast<float>(static_cast<double>(acc0[a][b][e]) * qf[b] * static_cast<double>(kfv[a][e])) * scale_inv;
-                        if (bias != nullptr) v[e] = v[e] + biv[a][e];
-                    }
                     float* dst = out + static_cast<size_t>(q) * R_total + rb;
                     if (rb + 3 < R && ((reinterpret_cast<uintptr_t>(dst) & 15) == 0)) {
-                        *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+                        *reinterpret_cast<float4*>(dst) = make_float4(accf[a][b][0], accf[a][b][1], accf[a][b][2], accf[a][b][3]);
                     } else {
 #pragma unroll
                         for (int e = 0; e < 4; ++e)
-                            if (rb + e < R) dst[e] = v[e];
+                            if (rb + e < R) dst[e] = accf[a][b][e];
                     }
                 }
             }
@@ -1376,13 +1369,11 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
 // step of chunk c (one cvt + one fma per output) runs on the accumulators in place, between a tile's last MFMA of
 // chunk c (k-step 3) and its first of chunk c + 1 (k-step 0, which starts from zero and overwrites it): two
 // elements behind each MFMA of k-step 3 from its third MFMA on, three behind each of the first MFMAs of the next
-// k-step 0, always of tiles whose turn to be overwritten has not come.  The 32 registers this frees per wave buy one
-// of two things (WN = 16-query tiles per MFMA wave):
-//   WN = 4  four MFMA waves of 64 keys x 64 queries (one per SIMD) + four loader waves, 256 registers each: an MFMA
-//           wave's operand reads are (64 + 64) x 64 bytes per 64 x 64 x 64 MACs instead of (64 + 32) x 64 per
-//           64 x 32 x 64, a third fewer LDS bytes per MAC;
-//   WN = 2  eight MFMA waves of 64 x 32 + EIGHT loader waves, 128 registers each: twice the waves issuing the stage
-//           loads, which is what sets the pace of the chunk loop.
+// k-step 0, always of tiles whose turn to be overwritten has not come.  The 32 registers this frees per wave let four
+// MFMA waves of 64 keys x 64 queries (WN = 4 query tiles; one wave per SIMD, 256 registers each) do the work of eight
+// of 64 x 32: an MFMA wave's operand reads are (64 + 64) x 64 bytes per 64 x 64 x 64 MACs instead of (64 + 32) x 64
+// per 64 x 32 x 64, a third fewer LDS bytes per MAC.  (The same scheme on eight MFMA waves of 64 x 32 with eight
+// loader waves needs 16 waves of at most 128 registers; it spills and is slower, so it is not built.)
 template <int WN>
 struct I8WDump {  // where a lane's accumulators go in the [Q, R, chunks] dump (parity checks): element (a, b, e) at
     int64_t base, qstep;  // base + b * qstep + (a * 16 + e) * chunks, for the query columns of qmask and the
@@ -1435,7 +1426,8 @@ __device__ __forceinline__ void i8w_kstep(const v4i (&ka)[4], const v4i (&qb)[WN
 
 template <int WN>
 struct I8WCfg {
-    using Tile = typename std::conditional<WN == 4, I8Cfg<128, 128>, I8CfgL8>::type;  // LDS layout and loader waves
+    static_assert(WN == 4, "four MFMA waves of 64 x 64");
+    using Tile = I8Cfg<128, 128>;  // LDS layout and loader waves
     static constexpr int kWavesN = 128 / (16 * WN);      // MFMA waves along the queries (2 along the keys)
     static constexpr int kConsumers = 2 * kWavesN;
     static constexpr int kBlock = (kConsumers + Tile::kLoaders) * 64;
@@ -2610,8 +2602,8 @@ static void launch_mfma_i8_t(int ndig, long long dig_stride, const long long* ke
                                             R_total, out, chunk_ints, bias, st, 1, 0, nullptr, key_tiled);
 }
 
-// The 128 x 128 tile on MFMA waves with one accumulator set (chain modes only): WN = 4, four MFMA waves of 64 x 64 and
-// four loader waves (tile 1284); WN = 2, eight MFMA waves of 64 x 32 and eight loader waves (tile 1288).
+// The 128 x 128 tile on four MFMA waves of 64 x 64 with one accumulator set, and four loader waves (tile 1284; chain
+// modes only).
 template <int WN>
 static void launch_mfma_i8w(const int8_t* A8, const float* qscale, int stride, const int8_t* K8, const float* Bw, int Sb,
                             int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv, int64_t R_total, float* out,
@@ -2658,17 +2650,13 @@ static void launch_mfma_i8(const int8_t* A8, const float* qscale, int stride, co
                            float* out, int32_t* chunk_ints, const float* bias, hipStream_t st, int key_tiled = 0,
                            int ndig = 0, long long dig_stride = 0, const long long* key_indices = nullptr) {
     const int tile = choose_i8_tile(R, Q);
-    if ((tile == 1284 || tile == 1288) && ndig == 0) {
-        if (tile == 1284)
-            launch_mfma_i8w<4>(A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints,
-                               bias, st, key_tiled);
-        else
-            launch_mfma_i8w<2>(A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints,
-                               bias, st, key_tiled);
+    if (tile == 1284 && ndig == 0) {
+        launch_mfma_i8w<4>(A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias,
+                           st, key_tiled);
         return;
     }
 #define BSI_I8_ARGS ndig, dig_stride, key_indices, key_tiled, A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias, st
-    if (tile == 128 || tile == 1284 || tile == 1288) launch_mfma_i8_t<128, 128>(BSI_I8_ARGS);
+    if (tile == 128 || tile == 1284) launch_mfma_i8_t<128, 128>(BSI_I8_ARGS);
     else if (tile == 12864) launch_mfma_i8_t<128, 64>(BSI_I8_ARGS);
     else if (tile == 64) launch_mfma_i8_t<64, 64>(BSI_I8_ARGS);
     else launch_mfma_i8_t<64, 32>(BSI_I8_ARGS);
@@ -2762,9 +2750,8 @@ extern "C" int bsi_hip_set_option(int option, int value) {
             g_digits_route = value;
             return BSI_OK;
         case BSI_OPT_I8_TILE:
-            BSI_REQUIRE(value == 0 || value == 128 || value == 1284 || value == 1288 || value == 12864 || value == 64 ||
-                            value == 6432,
-                        "tile must be 0, 128, 1284, 1288, 12864, 64 or 6432");
+            BSI_REQUIRE(value == 0 || value == 128 || value == 1284 || value == 12864 || value == 64 || value == 6432,
+                        "tile must be 0, 128, 1284, 12864, 64 or 6432");
             g_i8_tile = value;
             return BSI_OK;
         case BSI_OPT_BUILD_ITEMS:

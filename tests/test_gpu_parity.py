@@ -421,7 +421,7 @@ def _oracle_case(oracle, Q, R, d, seed, qkind="randn", ksigma=0.02, bits_q=7, bi
 
 
 # forms of the `tiled` argument that select the cached int8 key image, and the tile each one forces (0: automatic)
-_I8_TILES = {"int8": 0, "int8-128": 128, "int8-1284": 1284, "int8-1288": 1288, "int8-12864": 12864, "int8-64": 64, "int8-6432": 6432}
+_I8_TILES = {"int8": 0, "int8-128": 128, "int8-1284": 1284, "int8-12864": 12864, "int8-64": 64, "int8-6432": 6432}
 
 
 def _run_dot(hip, qb, kb, Q, R, W, Sa, Sb, core, tiled, with_ints8, want_ints=True, R_total=None):
@@ -497,8 +497,7 @@ DOT_SHAPES = [
                                               (0, True, True), (2, "int8-128", True), (0, "int8-64", False),
                                               (2, "int8-12864", True), (0, "int8-12864", False),
                                               (2, "int8-6432", True), (0, "int8-6432", False),
-                                              (2, "int8-1284", True), (0, "int8-1284", False),
-                                              (2, "int8-1288", True), (0, "int8-1288", False)])
+                                              (2, "int8-1284", True), (0, "int8-1284", False)])
 def test_dot_bit_exact(hip, oracle, Q, R, d, kind, core, tiled, ints8):
     x, k, qb, kb, want_ints, want_out = _oracle_case(oracle, Q, R, d, seed=Q + R + d, qkind=kind)
     W = (d + 63) // 64
@@ -568,7 +567,7 @@ def test_hybrid_query_dot_decodes_inline(ops, oracle, monkeypatch):
 
 
 @pytest.mark.parametrize("Sa,Sb", [(8, 8), (5, 4), (2, 2), (7, 5), (3, 7)])
-@pytest.mark.parametrize("core,tiled", [(1, False), (2, True), (2, "int8-128"), (2, "int8-1284"), (2, "int8-1288"), (2, "int8-12864"), (2, "int8-64"), (2, "int8-6432")])
+@pytest.mark.parametrize("core,tiled", [(1, False), (2, True), (2, "int8-128"), (2, "int8-1284"), (2, "int8-12864"), (2, "int8-64"), (2, "int8-6432")])
 def test_dot_other_bit_widths(hip, oracle, Sa, Sb, core, tiled):
     Q, R, d = 19, 35, 1024
     x, k, qb, kb, want_ints, want_out = _oracle_case(oracle, Q, R, d, seed=Sa * 10 + Sb, ksigma=0.05, bits_q=Sa, bits_k=Sb)
@@ -636,7 +635,7 @@ def test_dot_row_stride_and_untouched_columns(hip, oracle):
 
 def test_dot_row_stride_int8_image_and_few_rows(hip, oracle):
     x, k, qb, kb, want_ints, want_out = _oracle_case(oracle, 70, 150, 1024, seed=8)
-    for tiled in ("int8-128", "int8-1284", "int8-1288", "int8-12864", "int8-64", "int8-6432"):
+    for tiled in ("int8-128", "int8-1284", "int8-12864", "int8-64", "int8-6432"):
         _, out = _run_dot(hip, qb, kb, 70, 150, 16, 7, 6, 2, tiled=tiled, with_ints8=True, want_ints=False, R_total=163)
         np.testing.assert_array_equal(out[:, :150], want_out)
         assert np.isnan(out[:, 150:]).all()
@@ -646,7 +645,7 @@ def test_dot_row_stride_int8_image_and_few_rows(hip, oracle):
     assert np.isnan(out[:, 150:]).all()
 
 
-@pytest.mark.parametrize("tile", ["int8-128", "int8-1284", "int8-1288", "int8-12864", "int8-64", "int8-6432"])
+@pytest.mark.parametrize("tile", ["int8-128", "int8-1284", "int8-12864", "int8-64", "int8-6432"])
 @pytest.mark.parametrize("d", [256, 512, 768, 1280, 1792, 2304, 4352])
 def test_dot_int8_image_short_and_odd_chunk_counts(hip, oracle, d, tile):
     """1, 2, 3, 5, 7, 9 and 17 chunks through every tile of the int8-image kernel: the loader's prologue (three stages
@@ -680,7 +679,7 @@ def test_dot_int8_image_short_and_odd_chunk_counts(hip, oracle, d, tile):
     np.testing.assert_array_equal(outb.cpu().numpy(), want_out + bias[None, :])
 
 
-@pytest.mark.parametrize("Q,tiled", [(70, "int8-128"), (70, "int8-1284"), (70, "int8-1288"), (70, "int8-12864"), (70, "int8-64"), (70, "int8-6432"), (9, True), (70, True), (70, False)])
+@pytest.mark.parametrize("Q,tiled", [(70, "int8-128"), (70, "int8-1284"), (70, "int8-12864"), (70, "int8-64"), (70, "int8-6432"), (9, True), (70, True), (70, False)])
 def test_dot_bias_entry_point(hip, oracle, Q, tiled):
     """bsi_hip_dot_bias == bsi_hip_dot followed by a float addition of the bias row, bit for bit, whether the
     kernel adds it in its epilogue (int8 image, few rows) or the library appends an addition kernel."""
