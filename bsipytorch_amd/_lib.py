@@ -9,7 +9,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libbsi_hip.so")
+# BSI_HIP_LIBRARY names another build of the same library (the timeline build, say); it must exist like the default.
+LIB_PATH = os.environ.get("BSI_HIP_LIBRARY") or os.path.join(_HERE, "libbsi_hip.so")
 
 BSI_OK = 0
 DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
@@ -80,6 +81,7 @@ PROTOTYPES = {
     "bsi_hip_probe_mfma_i8": [ctypes.POINTER(_d), _vp],
     "bsi_hip_probe_stream_read": [_vp, _sz, ctypes.POINTER(_d), _vp],
     "bsi_hip_probe_l2_to_lds": [_vp, _sz, _i, ctypes.POINTER(_d), _vp],
+    "bsi_hip_timeline_read": [ctypes.POINTER(ctypes.c_ulonglong), _i],
     "bsi_hip_version": [],
     "bsi_hip_last_error": [],
 }

@@ -818,6 +818,23 @@ struct I8Cfg {
     static constexpr int kLds = 4 * kStage + kScaleBytes + kEpilogueBytes;
 };
 
+// Timeline build (make TIMELINE=1, -DBSI_TIMELINE): one MFMA wave and one loader wave of every workgroup of
+// dot_mfma_i8_kernel stamp the 100 MHz wall clock at the points below, 8 slots per workgroup (the first
+// kTimelineWorkgroups of the grid); bsi_hip_timeline_read copies them out.  The ordinary build has none of this.
+constexpr int kTimelineWorkgroups = 8192;
+constexpr int kStampMfmaEntry = 0, kStampFirstStage = 1, kStampLoopDone = 2, kStampStored = 3, kStampLoaderEntry = 4,
+              kStampLoaderDone = 5, kStampFirstIssue = 6, kStampThreeIssued = 7;
+#ifdef BSI_TIMELINE
+__device__ unsigned long long g_timeline[kTimelineWorkgroups * 8];
+#define BSI_STAMP(slot)                                                                    \
+    {                                                                                      \
+        const unsigned wg_ = blockIdx.y * gridDim.x + blockIdx.x;                          \
+        if (lane == 0 && wg_ < kTimelineWorkgroups) g_timeline[wg_ * 8 + (slot)] = wall_clock64(); \
+    }
+#else
+#define BSI_STAMP(slot)
+#endif
+
 // A loader wave of the int8-image kernels (lw = its number among the C::kLoaders loader waves; `consumers` MFMA
 // waves share the workgroup's barriers with it): 8 of the stage's groups of 8 rows (the TM key rows, then the TN
 // query rows: a load moves 1 KiB = 8 rows x 128 bytes), plus the chunk scales of 64 queries once per chunk.
@@ -917,9 +934,11 @@ __device__ __forceinline__ void i8_loader_wave(unsigned char* __restrict__ lds, 
                 c * sstep, 0, 0);
         }
     };
+    if (lw == 0) BSI_STAMP(kStampFirstIssue);
     issue(0);
     issue(1);
     issue(2);
+    if (lw == 0) BSI_STAMP(kStampThreeIssued);
     // The epilogue's operands, staged once per workgroup behind the first three stages: the slice-0 weight (key
     // factor) and the bias of the tile's TM keys, 64 rows per load.  (Fetched per lane at the end they are 32
     // vector-memory instructions for every MFMA wave, all queued in front of the output stores.)  Every loader wave
@@ -1091,10 +1110,13 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
     unsigned char* const scale_lds = lds + 4 * C::kStage;  // [chunk & 3][loader][64] floats
 
     if (wave >= C::kConsumers) {
+        if (wave == C::kConsumers) BSI_STAMP(kStampLoaderEntry);
         i8_loader_wave<C, kSum>(lds, wave - C::kConsumers, lane, A8, qscale, qscale_stride, K8, Bw, Sb, chunks, halves, R,
                                      Q, r0, q0, rowbytes, bias, ndig, dig_stride, key_tiled, warm, warm_lines);
+        if (wave == C::kConsumers) BSI_STAMP(kStampLoaderDone);
         return;
     }
+    if (wave == 0) BSI_STAMP(kStampMfmaEntry);
 
     // ---- MFMA waves
     const int wr = wave & 1, wq = wave >> 1;  // half of the keys, group of 32 queries
@@ -1161,6 +1183,7 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
     BSI_I8_KSTEP(3, nslot, acc, prev, qs, ip);
 
     lds_barrier();  // stage 0 is there
+    if (wave == 0) BSI_STAMP(kStampFirstStage);
 #pragma unroll
     for (int t = 0; t < WM; ++t) ka[0][t] = *reinterpret_cast<const v4i*>(lds + krow_off + t * 16 * 128 + pcol[0]);
 #pragma unroll
@@ -1205,6 +1228,7 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
     // the last k-step read ahead into a stage that does not exist (the loaders fill it with a copy of the last
     // one); nothing uses those operands
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    if (wave == 0) BSI_STAMP(kStampLoopDone);
 #undef BSI_I8_HORNER
 #undef BSI_I8_CHUNK
 #undef BSI_I8_KSTEP
@@ -1342,24 +1366,29 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
                 if (bias != nullptr) v = v + bi[a][e];
                 accf[a][b][e] = v;
             }
-    if (i8_store_lines<WM, WN>(accf, out, R_total, r0 + wr * (WM * 16), q0 + wq * (WN * 16), R, Q, ln, lg)) return;
+    if (!i8_store_lines<WM, WN>(accf, out, R_total, r0 + wr * (WM * 16), q0 + wq * (WN * 16), R, Q, ln, lg)) {
 #pragma unroll
-    for (int a = 0; a < WM; ++a) {
-        const int64_t rb = r0 + wr * (WM * 16) + a * 16 + lg * 4;
+        for (int a = 0; a < WM; ++a) {
+            const int64_t rb = r0 + wr * (WM * 16) + a * 16 + lg * 4;
 #pragma unroll
-        for (int b = 0; b < WN; ++b) {
-            const int64_t q = q0 + wq * (WN * 16) + b * 16 + ln;
-            if (q >= Q) continue;
-            float* dst = out + static_cast<size_t>(q) * R_total + rb;
-            if (rb + 3 < R && ((reinterpret_cast<uintptr_t>(dst) & 15) == 0)) {
-                *reinterpret_cast<float4*>(dst) = make_float4(accf[a][b][0], accf[a][b][1], accf[a][b][2], accf[a][b][3]);
-            } else {
+            for (int b = 0; b < WN; ++b) {
+                const int64_t q = q0 + wq * (WN * 16) + b * 16 + ln;
+                if (q >= Q) continue;
+                float* dst = out + static_cast<size_t>(q) * R_total + rb;
+                if (rb + 3 < R && ((reinterpret_cast<uintptr_t>(dst) & 15) == 0)) {
+                    *reinterpret_cast<float4*>(dst) = make_float4(accf[a][b][0], accf[a][b][1], accf[a][b][2], accf[a][b][3]);
+                } else {
 #pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (rb + e < R) dst[e] = accf[a][b][e];
+                    for (int e = 0; e < 4; ++e)
+                        if (rb + e < R) dst[e] = accf[a][b][e];
+                }
             }
         }
     }
+#ifdef BSI_TIMELINE
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the stamp below: the outputs have left the wave
+    if (wave == 0) BSI_STAMP(kStampStored);
+#endif
 }
 
 // ------------------------------------------------------------------ int8 image, one accumulator set per MFMA wave
@@ -3385,6 +3414,21 @@ extern "C" int bsi_hip_probe_l2_to_lds(const void* buf, size_t bytes, int loader
     BSI_LAUNCH_CHECK("probe_l2_lds_kernel");
     *bytes_per_s = static_cast<double>(cus) * kRegion * kPasses / (best * 1e-3);
     return BSI_OK;
+}
+
+extern "C" int bsi_hip_timeline_read(unsigned long long* stamps_host, int workgroups) {
+    BSI_REQUIRE(stamps_host && workgroups >= 1 && workgroups <= kTimelineWorkgroups, "workgroups must be 1 .. %d",
+                kTimelineWorkgroups);
+#ifdef BSI_TIMELINE
+    BSI_HIP_CHECK(hipDeviceSynchronize());
+    BSI_HIP_CHECK(hipMemcpyFromSymbol(stamps_host, HIP_SYMBOL(g_timeline), sizeof(unsigned long long) * 8 * workgroups));
+    void* dev = nullptr;  // cleared, so that the next read shows which workgroups have run since
+    BSI_HIP_CHECK(hipGetSymbolAddress(&dev, HIP_SYMBOL(g_timeline)));
+    BSI_HIP_CHECK(hipMemset(dev, 0, sizeof(unsigned long long) * 8 * kTimelineWorkgroups));
+    return BSI_OK;
+#else
+    return fail(BSI_ERR_INVALID, "this library was built without the timeline stamps (make TIMELINE=1 builds one with)");
+#endif
 }
 
 extern "C" int bsi_hip_dot_timed(const uint64_t* A, const int8_t* A_ints8, const float* A_chunk_scales,

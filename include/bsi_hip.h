@@ -369,6 +369,13 @@ int bsi_hip_dot_timed(const uint64_t* A, const int8_t* A_ints8, const float* A_c
 int bsi_hip_probe_valu_popcount(double* lane_ops_per_s, void* stream);
 int bsi_hip_probe_mfma_i8(double* ops_per_s, void* stream);
 int bsi_hip_probe_stream_read(const void* buf_device, size_t bytes, double* bytes_per_s, void* stream);
+/* Timeline build only (make -C bsipytorch_amd/csrc TIMELINE=1 -> libbsi_hip_timeline.so; the ordinary library returns
+ * BSI_ERR_INVALID): copies out the wall-clock stamps (100 MHz ticks) that the last int8-image chunk-scale dot left,
+ * 8 per workgroup for the first `workgroups` workgroups of its grid, in the order: MFMA wave entered, first stage in
+ * LDS, chunk loop done, outputs stored, loader wave entered, loader wave done, first stage load issued, three stages
+ * issued; a workgroup that has not run since the last read gives zeros (the read clears the stamps).  Synchronises the
+ * device.  No counterpart in the reference: a measuring aid. */
+int bsi_hip_timeline_read(unsigned long long* stamps_host, int workgroups);
 /* What the int8-image kernel's operand path delivers: every CU streams an L2-resident part of buf_device (at least
  * 2 MiB are read) into LDS with LDS-direct 16-byte buffer loads, 96 KiB in flight per CU, all CUs at once; the result
  * is the aggregate rate over all CUs in bytes per second.  loader_pattern = 0: eight issuing waves per CU, contiguous
