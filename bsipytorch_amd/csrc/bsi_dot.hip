@@ -800,15 +800,24 @@ __global__ __launch_bounds__(kWaves * 64) void probe_l2_lds_kernel(const unsigne
 static std::atomic<int> g_i8_tile{0};  // 0 = by grid size; 128, 12864 (128 keys x 64 queries) or 64 force a tile
 static std::atomic<int> g_digits_route{0};  // bsi_hip_dot_digits: 0 = by cost, 1 = stacked digits + combine pass, 2 = in-accumulator
 
+#ifndef BSI_I8_WN_RULE
+#define BSI_I8_WN_RULE ((TM == 128 && TN == 128) ? 2 : 1)
+#endif
 template <int TM, int TN>
 struct I8Cfg {
     static constexpr int kTM = TM, kTN = TN;
     static constexpr int kWM = TM / 32;                // 16-key tiles per wave (2 waves along the keys)
-    static constexpr int kWN = 2;                      // 16-query tiles per wave
-    static constexpr int kWavesN = TN / 32;            // waves along the queries
+    // 16-query tiles per wave: two for the 128 x 128 tile (eight MFMA waves of 64 x 32), one for the smaller tiles, which
+    // would otherwise run on four MFMA waves or fewer -- one per SIMD, and a single wave cannot issue its MFMAs, the chain
+    // and the operand reads fast enough to keep its SIMD's matrix pipe busy
+    static constexpr int kWN = BSI_I8_WN_RULE;
+    static constexpr int kWavesN = TN / (16 * kWN);    // waves along the queries
     static constexpr int kConsumers = 2 * kWavesN;
     static constexpr int kGroups = (TM + TN) / 8;      // groups of 8 operand rows (1 KiB per half-chunk) in a stage
-    static constexpr int kLoaders = (kGroups + 7) / 8;  // a loader wave moves up to 8 groups per stage
+    // loader waves: one per SIMD (the more waves issue a stage's loads, the faster it comes) -- but two for the
+    // 64 x 64 tile, measured: on one machine 512 x 2048 x 8192 takes 17.4 us with two and 18.7 with four (with four
+    // or with eight MFMA waves alike), while the 64 x 32 and 128 x 64 tiles gain 5 to 10 % from four
+    static constexpr int kLoaders = (TM == 64 && TN == 64) ? 2 : 4;
     static constexpr int kLoads = (kGroups + kLoaders - 1) / kLoaders;  // loads per loader wave and stage
     static constexpr int kBlock = (kConsumers + kLoaders) * 64;
     static constexpr int kOperandK = TM * 128;         // bytes of the key tile of one half-chunk
@@ -849,10 +858,9 @@ __device__ __forceinline__ void i8_loader_wave(unsigned char* __restrict__ lds, 
                                                long long warm_lines) {
     constexpr int TM = C::kTM, TN = C::kTN;
     constexpr int L = C::kLoaders, NI = C::kLoads, KG = TM / 8, QG = TN / 8;
-    // When the key groups and the query groups both divide evenly among the loader waves, every loader moves KG / L
-    // key groups, then QG / L query groups: which operand a load belongs to is then known at compile time.
-    constexpr bool kEven = (KG % L == 0) && (QG % L == 0);
-    static_assert(!kEven || NI == KG / L + QG / L, "loads per loader wave");
+    // The key groups and the query groups both divide evenly among the loader waves: every loader moves KG / L key
+    // groups, then QG / L query groups, so which operand a load belongs to is known at compile time.
+    static_assert(KG % L == 0 && QG % L == 0 && NI == KG / L + QG / L, "loads per loader wave");
     unsigned char* const scale_lds = lds + 4 * C::kStage;  // [chunk & 3][loader][64] floats
     // The prologue below is kept short on purpose: it runs on one wave per SIMD while the whole workgroup waits for
     // the first stage.  No row is clamped: a load that starts past its operand's end reads nothing (buffer bounds),
@@ -874,19 +882,11 @@ __device__ __forceinline__ void i8_loader_wave(unsigned char* __restrict__ lds, 
     // (scalar): the offset of its group.
     const uint32_t lr = static_cast<uint32_t>(lane) >> 3, lc = static_cast<uint32_t>(lane) & 7;
     uint32_t voff[NI], goff[NI];
-    bool is_key[NI];  // wave-uniform
+    bool is_key[NI];  // known at compile time once the loops are unrolled
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
-        int g, gg;  // group of the stage, group of its operand
-        if (kEven) {
-            is_key[i] = i < KG / L;
-            gg = is_key[i] ? lw + L * i : lw + L * (i - KG / L);
-            g = is_key[i] ? gg : gg + KG;
-        } else {  // the last load wraps around and fetches a group a second time: the same number of loads per wave
-            g = (lw + L * i) % C::kGroups;
-            is_key[i] = g < KG;
-            gg = is_key[i] ? g : g - KG;
-        }
+        is_key[i] = i < KG / L;
+        const int gg = is_key[i] ? lw + L * i : lw + L * (i - KG / L);  // group of its operand
         const uint32_t col = (lc ^ (static_cast<uint32_t>(gg & 1) * 4 + (lr >> 1))) * 16;
         const bool tiled = is_key[i] && key_tiled;
         voff[i] = (tiled ? lr * 128 : lr * rowbytes32) + col;
@@ -923,7 +923,7 @@ __device__ __forceinline__ void i8_loader_wave(unsigned char* __restrict__ lds, 
         }
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
-            const int g = kEven ? (i < KG / L ? lw + L * i : KG + lw + L * (i - KG / L)) : (lw + L * i) % C::kGroups;
+            const int g = i < KG / L ? lw + L * i : KG + lw + L * (i - KG / L);  // group of the stage
             load16_to_lds(is_key[i] ? rk : rq, voff[i], goff[i] + (is_key[i] ? so_k : so_q),
                           lds + (h & 3) * C::kStage + g * 1024);
         }
@@ -1011,7 +1011,7 @@ __device__ __forceinline__ void i8_kstep(const v4i (&ka)[WM], const v4i (&qb)[WN
                                          const float (&qs_prev)[WN], int* __restrict__ ints_prev,
                                          const int64_t (&int_off)[WM][WN], const int (&int_rows)[WM], int down_shift,
                                          int chunks) {
-    static_assert(WM + WN <= WM * WN, "one operand read behind each MFMA of a k-step");
+    static_assert(WM + WN <= 2 * WM * WN, "two operand reads behind each MFMA of a k-step");
 #pragma unroll
     for (int a = 0; a < WM; ++a)
 #pragma unroll
@@ -1153,9 +1153,9 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
             int_off[a][b] = (kInts && q < Q && r < R) ? (q * R + r) * chunks : -1;
         }
     }
-    // chunk scales of the lane's query columns, from the loaders' ring: region wq / 2 holds queries
-    // 64 (wq / 2) .. + 63 (WN = 2: a wave spans 32 queries)
-    const unsigned char* sread = scale_lds + (wq >> 1) * 256 + ((wq & 1) * 32 + ln) * 4;
+    // chunk scales of the lane's query columns, from the loaders' ring: region g holds queries 64 g .. + 63
+    const int qfirst = wq * (WN * 16);
+    const unsigned char* sread = scale_lds + (qfirst >> 6) * 256 + ((qfirst & 63) + ln) * 4;
     float qsa[WN], qsb[WN];  // scales of even / odd chunks
 #pragma unroll
     for (int b = 0; b < WN; ++b) qsa[b] = qsb[b] = 0.0f;
