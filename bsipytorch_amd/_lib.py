@@ -19,6 +19,7 @@ LAYOUT_CANONICAL, LAYOUT_TILED16, LAYOUT_INT8, LAYOUT_INT8_TILED = 0, 1, 2, 3
 OPT_I8_TILE = 1
 OPT_DIGITS_ROUTE = 2
 OPT_BUILD_ITEMS = 3
+OPT_OUTPUT_STORES = 4
 
 _vp = ctypes.c_void_p
 _i = ctypes.c_int

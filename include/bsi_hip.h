@@ -177,13 +177,17 @@ int bsi_hip_planes_to_int8_tiled(const uint64_t* words_device, int64_t rows, int
 
 /* Tuning knobs (process-wide, not thread-safe; set before launching).  No counterpart in the reference,
  * whose kernel selection is read from environment variables on every call (bsi_cuda_kernels_dot.cuh:2642). */
-#define BSI_OPT_I8_TILE 1 /* tile of the int8-image kernel: 128 (128 keys x 128 queries), 12864 (128 x 64), 64 (64 x 64)
-                             or 6432 (64 x 32); 0 (default) = chosen per call from the grid each tile would give on
-                             the 256 CUs */
+#define BSI_OPT_I8_TILE 1 /* tile of the int8-image kernel: 128 (128 keys x 128 queries), 12864 (128 x 64), 64 (64 x 64),
+                             6432 (64 x 32) or 1284 (128 x 128 on four MFMA waves of 64 x 64 with one accumulator set);
+                             0 (default) = chosen per call from the grid each tile would give on the 256 CUs */
 #define BSI_OPT_DIGITS_ROUTE 2 /* bsi_hip_dot_digits: 1 = stacked digits and a combine pass, 2 = digits recombined in the
                                   accumulator where the int32 bound allows; 0 (default) = the cheaper by a cost estimate */
 #define BSI_OPT_BUILD_ITEMS 3 /* (row, chunk) items per wave of the fused chunk-scale builder: 1, 2, 4 or 8; 0 (default)
                                  = chosen per call from the number of items */
+#define BSI_OPT_OUTPUT_STORES 4 /* how the int8-image kernels store whole output tiles: 1 = plain stores (the output stays
+                                   in the caches for the next kernel), 2 = nontemporal stores (it leaves them as it is
+                                   written); 0 (default) = plain from the linear-layer entry points (bsi_hip_dot_bias,
+                                   bsi_hip_dot_bias_warm, bsi_hip_linear), nontemporal from the other dot entry points */
 int bsi_hip_set_option(int option, int value);
 
 /* Bytes of device workspace bsi_hip_dot needs for this shape and core (0 when none). */

@@ -679,6 +679,40 @@ def test_dot_int8_image_short_and_odd_chunk_counts(hip, oracle, d, tile):
     np.testing.assert_array_equal(outb.cpu().numpy(), want_out + bias[None, :])
 
 
+@pytest.mark.parametrize("tile", ["int8-128", "int8-1284", "int8-12864", "int8-64", "int8-6432"])
+@pytest.mark.parametrize("stores", [0, 1, 2])
+def test_dot_whole_tiles_stored_in_lines(hip, oracle, tile, stores):
+    """Output tiles that lie wholly inside an aligned output are stored in whole 128-byte lines after a lane exchange,
+    with plain or nontemporal stores (BSI_OPT_OUTPUT_STORES; 0 = plain from the layer entry point bsi_hip_dot_bias,
+    nontemporal from bsi_hip_dot).  The last key tile and the last query tile are ragged and take the element path;
+    every combination must give the oracle's bits, through both entry points."""
+    Q, R, d, W = 200, 416, 1024, 16  # 416 = 13 x 32: the lines are aligned, the last tile of 64 or 128 keys is not whole
+    x, k, qb, kb, want_ints, want_out = _oracle_case(oracle, Q, R, d, seed=77)
+    bias = np.random.default_rng(2).standard_normal(R).astype(np.float32)
+    L = hip.lib
+    A, scales, Bc, Bw, bd = dev(qb["words"]), dev(qb["scales"]), dev(kb["words"]), dev(kb["slice_weights"]), dev(bias)
+    a8 = torch.zeros((Q, 4 * 256), dtype=torch.int8, device="cuda")
+    hip.check(L.bsi_hip_planes_to_int8(A.data_ptr(), Q, 7, W, a8.data_ptr(), st()), "p2i8")
+    B = torch.zeros((R, 4 * 256), dtype=torch.int8, device="cuda")
+    hip.check(L.bsi_hip_planes_to_int8(Bc.data_ptr(), R, 6, W, B.data_ptr(), st()), "image")
+    hip.check(L.bsi_hip_set_option(hip.OPT_I8_TILE, _I8_TILES[tile]), "opt")
+    hip.check(L.bsi_hip_set_option(hip.OPT_OUTPUT_STORES, stores), "opt")
+    try:
+        out = torch.full((Q, R), float("nan"), dtype=torch.float32, device="cuda")
+        hip.check(L.bsi_hip_dot(A.data_ptr(), a8.data_ptr(), scales.data_ptr(), 4, 7, W, B.data_ptr(), 2, Bw.data_ptr(), 6,
+                                R, Q, float(np.float32(1e-4)), R, out.data_ptr(), None, 2, None, 0, st()), "dot")
+        outb = torch.full((Q, R), float("nan"), dtype=torch.float32, device="cuda")
+        hip.check(L.bsi_hip_dot_bias(A.data_ptr(), a8.data_ptr(), scales.data_ptr(), 4, 7, W, B.data_ptr(), 2,
+                                     Bw.data_ptr(), 6, R, Q, float(np.float32(1e-4)), R, bd.data_ptr(), outb.data_ptr(),
+                                     2, None, 0, st()), "dot_bias")
+        torch.cuda.synchronize()
+    finally:
+        hip.check(L.bsi_hip_set_option(hip.OPT_I8_TILE, 0), "opt")
+        hip.check(L.bsi_hip_set_option(hip.OPT_OUTPUT_STORES, 0), "opt")
+    np.testing.assert_array_equal(out.cpu().numpy(), want_out)
+    np.testing.assert_array_equal(outb.cpu().numpy(), want_out + bias[None, :])
+
+
 @pytest.mark.parametrize("Q,tiled", [(70, "int8-128"), (70, "int8-1284"), (70, "int8-12864"), (70, "int8-64"), (70, "int8-6432"), (9, True), (70, True), (70, False)])
 def test_dot_bias_entry_point(hip, oracle, Q, tiled):
     """bsi_hip_dot_bias == bsi_hip_dot followed by a float addition of the bias row, bit for bit, whether the
