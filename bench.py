@@ -189,6 +189,43 @@ def _decode_shapes(_lib, bsi_ops):
     return rows
 
 
+def _headline_rotating(_lib, bsi_ops):
+    """The headline shape (Q512 R8192 D2048) on a rotation of keysets whose int8 images add up to more than the 256 MB
+    memory-side cache, so that every launch reads its 16 MiB key image from HBM, next to the resident figure taken the
+    same way (launches recorded into one HIP graph and replayed)."""
+    import torch
+
+    Qh, Rh, Dh = 512, 8192, 2048
+    image_bytes = Rh * Dh
+    n_sets = -(-640 * 1024 * 1024 // image_bytes)
+    gen = torch.Generator(device="cuda").manual_seed(7)
+    keysets = []
+    for _ in range(n_sets):
+        Kd = torch.randn(Rh, Dh, device="cuda", generator=gen) * 0.02
+        keysets.append(bsi_ops.build_bsi_keys_cuda(Kd, 2, 0.5)[0])
+        del Kd
+    x = torch.randn(Qh, Dh, device="cuda", generator=gen)
+    qcap = bsi_ops.build_bsi_queries_cuda_batch_packed(x, 2, 0.5)
+    W, chunks = Dh // 64, Dh // 256
+    out = torch.empty((Qh, Rh), dtype=torch.float32, device="cuda")
+
+    def launch(kc):
+        kptr, klayout = bsi_ops.key_operand(kc, Qh, SA, _lib.CORE_MFMA)
+
+        def f():
+            _lib.check(_lib.lib.bsi_hip_dot(qcap.words.data_ptr(), qcap.ints8.data_ptr(), qcap.chunk_scales.data_ptr(),
+                                            chunks, SA, W, kptr, klayout, kc.slice_weights.data_ptr(), SB, Rh, Qh, 1e-4, Rh,
+                                            out.data_ptr(), None, _lib.CORE_MFMA, None, 0, bsi_ops._stream()), "bsi_hip_dot")
+        return f
+
+    resident = _graph_timed_us([launch(keysets[0])], rounds=32)
+    rotating = _graph_timed_us([launch(kc) for kc in keysets], rounds=2)
+    ops = 2.0 * Qh * Rh * Dh
+    return {"workload": "Q512 R8192 D2048, launches replayed from a HIP graph", "keysets_in_rotation": n_sets,
+            "key_image_bytes": image_bytes, "us_resident": resident, "us_rotating": rotating,
+            "frac_of_int8_mfma_peak_rotating": ops / (rotating * 1e-6) / 1e12 / MFMA_I8_PEAK_TOPS}
+
+
 def _opt_prefill():
     """OPT-1.3B-shaped prefill (24 layers, hidden 2048, 32 heads, FFN 8192, vocab 50272, batch 1 x 512 tokens, every
     decoder linear layer BSI): tokens/s eager and as a replayed HIP graph, and the dot's share of the forward."""
@@ -395,6 +432,7 @@ def main() -> int:
     if not args.no_extras and used_core == "mfma":
         extras = {}
         for key, fn in (("fc2_like", lambda: _fc2_like(_lib, bsi_ops, args.steps)),
+                        ("headline_on_rotating_keysets", lambda: _headline_rotating(_lib, bsi_ops)),
                         ("opt6.7b_layers_one_row", lambda: _decode_shapes(_lib, bsi_ops)),
                         ("opt1.3b_prefill", _opt_prefill)):
             try:
