@@ -831,8 +831,10 @@ struct I8Cfg {
 // dot_mfma_i8_kernel stamp the 100 MHz wall clock at the points below, 8 slots per workgroup (the first
 // kTimelineWorkgroups of the grid); bsi_hip_timeline_read copies them out.  The ordinary build has none of this.
 constexpr int kTimelineWorkgroups = 8192;
-constexpr int kStampMfmaEntry = 0, kStampFirstStage = 1, kStampLoopDone = 2, kStampStored = 3, kStampLoaderEntry = 4,
-              kStampLoaderDone = 5, kStampFirstIssue = 6, kStampThreeIssued = 7;
+enum TimelineStamp {
+    kStampMfmaEntry = 0, kStampFirstStage = 1, kStampLoopDone = 2, kStampStored = 3, kStampLoaderEntry = 4,
+    kStampLoaderDone = 5, kStampFirstIssue = 6, kStampThreeIssued = 7
+};
 #ifdef BSI_TIMELINE
 __device__ unsigned long long g_timeline[kTimelineWorkgroups * 8];
 #define BSI_STAMP(slot)                                                                    \
