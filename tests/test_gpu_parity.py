@@ -705,12 +705,24 @@ def test_dot_whole_tiles_stored_in_lines(hip, oracle, tile, stores):
         hip.check(L.bsi_hip_dot_bias(A.data_ptr(), a8.data_ptr(), scales.data_ptr(), 4, 7, W, B.data_ptr(), 2,
                                      Bw.data_ptr(), 6, R, Q, float(np.float32(1e-4)), R, bd.data_ptr(), outb.data_ptr(),
                                      2, None, 0, st()), "dot_bias")
+        # an output whose base is not on a 128-byte line (64 bytes off), and one 4 bytes off: the element paths
+        off = []
+        for shift in (16, 1):
+            flat = torch.full((Q * R + 32,), float("nan"), dtype=torch.float32, device="cuda")
+            hip.check(L.bsi_hip_dot(A.data_ptr(), a8.data_ptr(), scales.data_ptr(), 4, 7, W, B.data_ptr(), 2, Bw.data_ptr(),
+                                    6, R, Q, float(np.float32(1e-4)), R, flat.data_ptr() + 4 * shift, None, 2, None, 0, st()),
+                      "dot")
+            off.append((shift, flat))
         torch.cuda.synchronize()
     finally:
         hip.check(L.bsi_hip_set_option(hip.OPT_I8_TILE, 0), "opt")
         hip.check(L.bsi_hip_set_option(hip.OPT_OUTPUT_STORES, 0), "opt")
     np.testing.assert_array_equal(out.cpu().numpy(), want_out)
     np.testing.assert_array_equal(outb.cpu().numpy(), want_out + bias[None, :])
+    for shift, flat in off:
+        got = flat.cpu().numpy()
+        np.testing.assert_array_equal(got[shift:shift + Q * R].reshape(Q, R), want_out)
+        assert np.isnan(got[:shift]).all() and np.isnan(got[shift + Q * R:]).all()
 
 
 @pytest.mark.parametrize("Q,tiled", [(70, "int8-128"), (70, "int8-1284"), (70, "int8-12864"), (70, "int8-64"), (70, "int8-6432"), (9, True), (70, True), (70, False)])
