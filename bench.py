@@ -401,6 +401,23 @@ def main() -> int:
         e1.record()
         torch.cuda.synchronize()
         dense[f"torch_matmul_{name}_us"] = e0.elapsed_time(e1) / 20 * 1e3
+    # the vendor library's int8 GEMM of the shape (int32 output, no chunk scales): the same matrix-core instruction
+    # class as the BSI dot's core, without its fp32 chain
+    try:
+        a8 = torch.randint(-64, 63, (Q, D), dtype=torch.int8, device="cuda")
+        b8 = torch.randint(-32, 31, (R, D), dtype=torch.int8, device="cuda")
+        for _ in range(5):
+            torch._int_mm(a8, b8.t())
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(20):
+            torch._int_mm(a8, b8.t())
+        e1.record()
+        torch.cuda.synchronize()
+        dense["torch_int_mm_int8_us"] = e0.elapsed_time(e1) / 20 * 1e3
+    except Exception as exc:  # not every build of torch has it
+        dense["torch_int_mm_int8_us"] = None
+        dense["torch_int_mm_error"] = f"{type(exc).__name__}: {exc}"[:200]
     result["dense_baseline"] = dense
 
     if not args.no_cpu:
