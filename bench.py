@@ -28,7 +28,7 @@ Q, R, D = 512, 8192, 2048
 # HBM bytes per launch of the dot kernel on this workload: an OFFLINE figure, from rocprofv3 FETCH_SIZE and WRITE_SIZE
 # runs of this script scaled by a 256 MiB copy (profiles/dot_mfma_i8_kernel_fc1_Q512_R8192_D2048_hbm_traffic.txt).
 # Hardware counters cannot be read from inside the process, so it is not re-measured by a run of this script.
-MEASURED_TRAFFIC_BYTES = {"mfma": 42466000}
+MEASURED_TRAFFIC_BYTES = {"mfma": 42439000}
 TRAFFIC_SOURCE = "offline: profiles/dot_mfma_i8_kernel_fc1_Q512_R8192_D2048_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)"
 SA, SB = 7, 6
 
