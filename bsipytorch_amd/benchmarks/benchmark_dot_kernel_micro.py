@@ -18,7 +18,7 @@ from bsipytorch_amd import _lib, bsi_ops
 
 
 def run(Q, R, D, decimal_places=2, compress_threshold=0.5, warmup=10, iters=50, seed=123, core="auto",
-        key_sigma=0.02, outliers=False, relu=False, use_ints8=True, report_stats=False):
+        key_sigma=0.02, outliers=False, relu=False, use_ints8=True, report_stats=False, image_fill="built"):
     torch.manual_seed(seed)
     K = torch.randn(R, D, dtype=torch.float32) * key_sigma
     X = torch.randn(Q, D, dtype=torch.float32)
@@ -30,6 +30,8 @@ def run(Q, R, D, decimal_places=2, compress_threshold=0.5, warmup=10, iters=50, 
     qcap = bsi_ops.build_bsi_queries_cuda_batch_packed(X.cuda(), decimal_places, float(compress_threshold))
     if report_stats:
         print("[Keys]", bsi_ops.bsi_keys_cuda_stats(kcap))
+    if image_fill != "built":
+        _refill_images(qcap, kcap, image_fill)
     chunks = (W + 3) // 4
     if not (qcap.fixed and kcap.fixed):
         return _run_weighted(qcap, kcap, Q, R, D, W, key_bytes, warmup, iters)
@@ -57,6 +59,24 @@ def run(Q, R, D, decimal_places=2, compress_threshold=0.5, warmup=10, iters=50, 
             "avg_dot_us": t * 1e6, "dot_q_us": t * 1e6 / Q, "dot_s_ns": t * 1e9 / (Q * R),
             "effective_bitop_TOPS": bit_ops / t / 1e12, "int8_TOPS": 2.0 * Q * R * D / t / 1e12,
             "algorithmic_GBps": alg_bytes / t / 1e9, "key_plane_GBps": key_bytes / t / 1e9, "iters": iters}
+
+
+def _refill_images(qcap, kcap, fill):
+    """Overwrite the int8 images the matrix-core kernel reads, for timing only (the output is then not the dot of
+    the inputs).  The kernel does the same instructions on any data, so a change of its time with the data is the
+    shader clock following the power the operands draw: "zero" toggles nothing, "random" is uniform bytes,
+    "magnitude" keeps the built values without their signs (no runs of one-bits from sign extension)."""
+    if qcap.ints8 is None or kcap.ints8 is None:
+        raise RuntimeError("--image_fill needs fixed-bit operands with int8 images")
+    for cap in (qcap, kcap):
+        if fill == "zero":
+            cap.ints8.zero_()
+        elif fill == "random":
+            cap.ints8.copy_(torch.randint(-128, 128, cap.ints8.shape, dtype=torch.int8, device=cap.ints8.device))
+        elif fill == "magnitude":
+            cap.ints8.copy_(cap.ints8.abs())
+        else:
+            raise ValueError(fill)
 
 
 def _run_weighted(qcap, kcap, Q, R, D, W, key_bytes, warmup, iters):
@@ -99,12 +119,14 @@ def main() -> None:
     p.add_argument("--report_stats", action="store_true")
     p.add_argument("--i8_tile", type=int, default=0, choices=[0, 128, 1284, 12864, 64, 6432],
                    help="force a tile of the int8-image kernel (1284: 128 x 128 on four MFMA waves of 64 x 64); 0 = automatic")
+    p.add_argument("--image_fill", default="built", choices=["built", "zero", "random", "magnitude"],
+                   help="timing only: overwrite the int8 images (the clock follows the power the data draws)")
     a = p.parse_args()
     if not torch.cuda.is_available():
         raise RuntimeError("a GPU is required for this microbench")
     _lib.check(_lib.lib.bsi_hip_set_option(_lib.OPT_I8_TILE, a.i8_tile), "bsi_hip_set_option")
     r = run(a.Q, a.R, a.D, a.decimal_places, a.compress_threshold, a.warmup, a.iters, a.seed, a.core, a.key_sigma,
-            a.outliers, a.relu, not a.planes_only, a.report_stats)
+            a.outliers, a.relu, not a.planes_only, a.report_stats, a.image_fill)
     print(f"[Microbench] Q={a.Q} R={a.R} D={a.D} iters={a.iters} core={r['core']} layout={r['layout']}")
     print(f"[Kernel] avg_dot_ms={r['avg_dot_us'] / 1e3:.4f}  dot_q_us={r['dot_q_us']:.3f}  dot_s_ns={r['dot_s_ns']:.4f}")
     print(json.dumps(r))
