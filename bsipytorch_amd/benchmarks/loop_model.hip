@@ -11,12 +11,22 @@
 // the shader clock the two counters imply.  Machines whose shader clock settles lower under this load show fewer cycles
 // per stage for the same time: part of the stage's way is clocked by the memory side, not by the CU.
 //
+// Two more parts.  (1) The matrix pipes by themselves: back-to-back v_mfma_i32_16x16x64_i8 and v_mfma_i32_32x32x32_i8 on
+// independent accumulators, one and two waves per SIMD -- the rate the chip sustains at the clock it holds under that
+// load, to set next to the published peak (which assumes 2.4 GHz).  (2) The same loop for a workgroup tile of 256 keys x
+// 128 queries on v_mfma_i32_32x32x32_i8: eight waves of 64 x 64 at up to 256 registers each (no room for loader waves),
+// two int32 accumulator sets (the 32-deep k-step halves the operand registers, which makes room for the second set), the
+// chain spread evenly (two elements per MFMA), four operand reads per k-step, and every wave issuing an eighth of
+// each 48 KiB stage itself as inline assembly (loads the compiler knows to write LDS make it wait before LDS reads).
+//
 //   make -C bsipytorch_amd/csrc ../benchmarks/loop_model && bsipytorch_amd/benchmarks/loop_model
 #include <hip/hip_runtime.h>
 
+#include <cstdint>
 #include <cstdio>
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
 typedef __amdgpu_buffer_rsrc_t rsrc_t;
 
 #define CHECK(x)                                                                          \
@@ -122,6 +132,205 @@ __global__ __launch_bounds__(768) void loop_model(int* sink, int ksteps, unsigne
     }
 }
 
+
+// ---------------------------------------------------------------- the matrix pipes by themselves
+template <bool k32>
+__global__ __launch_bounds__(512) void mfma_only(int* sink, int iters, unsigned long long* cycles) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];  // only to keep one workgroup per CU
+    v4i a, b;
+    unsigned s = (threadIdx.x + 1u + blockIdx.x * 977u) * 2654435761u;
+    for (int j = 0; j < 4; ++j) {  // pseudo-random int8 operands of the kernel's value range
+        s = s * 1664525u + 1013904223u;
+        a[j] = static_cast<int>(s & 0x3f3f3f3fu);
+        s = s * 1664525u + 1013904223u;
+        b[j] = static_cast<int>(s ^ (s >> 7));
+    }
+    if (threadIdx.x == 9999) lds[0] = 1;
+    const unsigned long long t0 = __builtin_readcyclecounter(), w0 = wall_clock64();
+    int r = 0;
+    if (!k32) {
+        v4i c[8];
+        for (int j = 0; j < 8; ++j) c[j] = (v4i){0, 0, 0, 0};
+        for (int i = 0; i < iters; ++i) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) c[j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(j & 1 ? a : b, j & 2 ? a : b, c[j], 0, 0, 0);
+        }
+        for (int j = 0; j < 8; ++j) r += c[j][j & 3];
+    } else {
+        v16i c[4];
+        for (int j = 0; j < 4; ++j)
+            for (int e = 0; e < 16; ++e) c[j][e] = 0;
+        for (int i = 0; i < iters; ++i) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) c[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(j & 1 ? a : b, j & 2 ? a : b, c[j], 0, 0, 0);
+        }
+        for (int j = 0; j < 4; ++j) r += c[j][j];
+    }
+    const unsigned long long t1 = __builtin_readcyclecounter(), w1 = wall_clock64();
+    if (r == 0x7FFFFFFF) sink[0] = r;  // never
+    if ((threadIdx.x & 63) == 0) {
+        atomicMax(&cycles[0], t1 - t0);
+        atomicMax(&cycles[2], w1 - w0);
+    }
+}
+
+template <bool k32>
+static int run_mfma_only(int* sink, unsigned long long* cycles, int cus, int waves_per_simd) {
+    CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&mfma_only<k32>), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes));
+    const int iters = 4096;
+    unsigned long long h[4] = {0, 0, 0, 0};
+    for (int rep = 0; rep < 2; ++rep) {
+        CHECK(hipMemset(cycles, 0, 32));
+        hipLaunchKernelGGL((mfma_only<k32>), dim3(cus), dim3(256 * waves_per_simd), kLdsBytes, 0, sink, iters, cycles);
+        CHECK(hipDeviceSynchronize());
+        CHECK(hipMemcpy(h, cycles, 32, hipMemcpyDeviceToHost));
+    }
+    const double n = iters * (k32 ? 4.0 : 8.0) * waves_per_simd, ns = static_cast<double>(h[2]) * 10.0 / n;
+    printf("%s back to back, %d wave(s) per SIMD: %5.1f cycles and %5.2f ns per MFMA = %.2f POP/s over %d SIMDs  [shader clock %.2f GHz]\n",
+           k32 ? "v_mfma_i32_32x32x32_i8" : "v_mfma_i32_16x16x64_i8", waves_per_simd, static_cast<double>(h[0]) / n, ns,
+           2.0 * (k32 ? 32768.0 : 16384.0) * cus * 4 / ns / 1e6, cus * 4, static_cast<double>(h[0]) / (static_cast<double>(h[2]) * 10.0));
+    return 0;
+}
+
+// ---------------------------------------------------------------- 256 x 128 on v_mfma_i32_32x32x32_i8, self-loading
+constexpr int kStageX = 48 * 1024;  // (256 + 128) rows x 128 bytes: a half-chunk of the 256 x 128 tile
+constexpr int kLdsX = 3 * kStageX + 8192;
+constexpr size_t kRegionX = 384 * 1024;
+
+__device__ __forceinline__ v4i raw_rsrc(const void* base, size_t bytes) {
+    const uint64_t b = reinterpret_cast<uint64_t>(base);
+    return (v4i){static_cast<int>(__builtin_amdgcn_readfirstlane(static_cast<uint32_t>(b))),
+                 static_cast<int>(__builtin_amdgcn_readfirstlane(static_cast<uint32_t>(b >> 32) & 0xFFFFu)),
+                 static_cast<int>(__builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bytes))), 0x00020000};
+}
+// 64 lanes x 16 bytes from the buffer (byte offset voff per lane + soff) to LDS address lds_addr + 16 lane
+__device__ __forceinline__ void dma16(v4i rsrc, uint32_t voff, uint32_t soff, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds" ::"v"(voff), "s"(rsrc), "s"(soff), "s"(lds_addr) : "memory");
+}
+
+// kLoads: LDS-direct loads per wave and stage (6 = a wave's eighth of 48 KiB); kBarrier: a workgroup barrier per stage;
+// kSpread: the loads issued 2, 1, 2, 1 behind the four k-steps of a stage (true) or 3 + 3 behind the first and third
+template <int kLoads, bool kBarrier, bool kSpread>
+__global__ __launch_bounds__(512) void loop_model_x(int* sink, int stages, unsigned long long* cycles, const unsigned char* buf) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    for (int i = threadIdx.x; i < kStageX / 4; i += 512) reinterpret_cast<int*>(lds)[i] = (i * 2654435761u) & 0x3f3f3f3f;
+    __syncthreads();
+    const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) unsigned char*)lds));
+    const v4i r = raw_rsrc(buf + (blockIdx.x % 8) * kRegionX, kRegionX);
+    uint32_t goff = wave * 6 * 1024;
+    const int wr = wave & 3, wq = wave >> 2, l32 = lane & 31, lh = lane >> 5;
+    const int krow = wr * 64 + l32, qrow = 256 + wq * 64 + l32;
+    // operand of tile t (32 rows further), k-step ks: 16-byte column (2 ks + lh) ^ ((row >> 1) & 7) of the row
+    auto kaddr = [&](int t, int ks) { const int row = krow + t * 32; return lds + row * 128 + (((2 * ks + lh) ^ (row >> 1)) & 7) * 16; };
+    auto qaddr = [&](int t, int ks) { const int row = qrow + t * 32; return lds + row * 128 + (((2 * ks + lh) ^ (row >> 1)) & 7) * 16; };
+    v4i ka[2][2], qb[2][2];
+    v16i acc[2][2][2];
+    float accf[2][2][16];
+    for (int a = 0; a < 2; ++a) {
+        ka[0][a] = ka[1][a] = *reinterpret_cast<const v4i*>(kaddr(a, 0));
+        qb[0][a] = qb[1][a] = *reinterpret_cast<const v4i*>(qaddr(a, 0));
+        for (int b = 0; b < 2; ++b)
+            for (int e = 0; e < 16; ++e) {
+                acc[0][a][b][e] = a + b + e;
+                acc[1][a][b][e] = a - b + e;
+                accf[a][b][e] = 0.f;
+            }
+    }
+    const float sc = 1.0f + (lane & 3);
+    const unsigned long long t0 = __builtin_readcyclecounter(), w0 = wall_clock64();
+    int slot = 1;
+    for (int st = 0; st < stages; st += 4) {  // two chunks = four stages per trip; the int32 set is the chunk's parity
+#pragma unroll
+        for (int s4 = 0; s4 < 4; ++s4) {
+            const int set = s4 >> 1;
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {  // k-steps of 32 within the stage
+                v4i(&kc)[2] = ka[ks & 1];
+                v4i(&qc)[2] = qb[ks & 1];
+                v4i(&kn)[2] = ka[(ks & 1) ^ 1];
+                v4i(&qn)[2] = qb[(ks & 1) ^ 1];
+                const bool first = (s4 & 1) == 0 && ks == 0;  // first k-step of a chunk: accumulate onto zero
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const int a = t >> 1, b = t & 1;
+                    if (first)
+                        acc[set][a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kc[a], qc[b], (v16i){0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}, 0, 0, 0);
+                    else
+                        acc[set][a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kc[a], qc[b], acc[set][a][b], 0, 0, 0);
+                    // the chain of the other set (the previous chunk): 64 elements over 32 MFMAs
+                    const int m = ((s4 & 1) * 4 + ks) * 4 + t;
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) {
+                        const int el = m * 2 + j, ta = el >> 5, tb = (el >> 4) & 1, e = el & 15;
+                        accf[ta][tb][e] = fmaf(static_cast<float>(acc[set ^ 1][ta][tb][e]), sc, accf[ta][tb][e]);
+                    }
+                    const int nks = (ks + 1) & 3;
+                    const v4i rd = *reinterpret_cast<const v4i*>(t < 2 ? kaddr(t, nks) : qaddr(t - 2, nks));
+                    if (t < 2) kn[t] = rd;
+                    else qn[t - 2] = rd;
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                if (kLoads) {
+                    const uint32_t base = lds0 + slot * kStageX + wave * 6 * 1024;
+                    if (kSpread) {
+                        const int n = (ks & 1) ? 1 : 2, at = (ks >> 1) * 3 + (ks & 1) * 2;
+#pragma unroll
+                        for (int i = 0; i < n; ++i)
+                            if (at + i < kLoads) dma16(r, lane * 16, goff + (at + i) * 1024, base + (at + i) * 1024);
+                    } else if (ks == 0 || ks == 2) {
+#pragma unroll
+                        for (int i = 0; i < 3; ++i)
+                            if ((ks >> 1) * 3 + i < kLoads) dma16(r, lane * 16, goff + ((ks >> 1) * 3 + i) * 1024, base + ((ks >> 1) * 3 + i) * 1024);
+                    }
+                }
+            }
+            if (kLoads) {
+                goff += 48 * 1024;
+                if (goff + 6 * 1024 > kRegionX) goff = wave * 6 * 1024;
+                slot = (slot == 2) ? 1 : 2;
+            }
+            if (kBarrier) {
+                if (kLoads) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoads) : "memory");
+                asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            }
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    const unsigned long long t1 = __builtin_readcyclecounter(), w1 = wall_clock64();
+    int sum = 0;
+    float fs = 0;
+    for (int a = 0; a < 2; ++a)
+        for (int b = 0; b < 2; ++b)
+            for (int e = 0; e < 16; ++e) {
+                sum += acc[0][a][b][e] + acc[1][a][b][e];
+                fs += accf[a][b][e];
+            }
+    if (sum == 0x7FFFFFFF || fs == 1.2345f) sink[0] = sum;  // never
+    if (lane == 0) {
+        atomicMax(&cycles[0], t1 - t0);
+        atomicMax(&cycles[2], w1 - w0);
+    }
+}
+
+template <int kLoads, bool kBarrier, bool kSpread = false>
+static int run_x(int* sink, unsigned long long* cycles, const unsigned char* buf, int cus, const char* name) {
+    CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&loop_model_x<kLoads, kBarrier, kSpread>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, kLdsX));
+    const int stages = 2048;
+    unsigned long long h[4] = {0, 0, 0, 0};
+    for (int rep = 0; rep < 2; ++rep) {
+        CHECK(hipMemset(cycles, 0, 32));
+        hipLaunchKernelGGL((loop_model_x<kLoads, kBarrier, kSpread>), dim3(cus), dim3(512), kLdsX, 0, sink, stages, cycles, buf);
+        CHECK(hipDeviceSynchronize());
+        CHECK(hipMemcpy(h, cycles, 32, hipMemcpyDeviceToHost));
+    }
+    const double per_stage = static_cast<double>(h[0]) / stages;
+    printf("%-58s %5.1f cycles per MFMA and SIMD  %5.0f cycles = %.3f us per 48 KiB stage  [shader clock %.2f GHz]\n", name, per_stage / 32.0,
+           per_stage, static_cast<double>(h[2]) / 100.0 / stages, static_cast<double>(h[0]) / (static_cast<double>(h[2]) * 10.0));
+    return 0;
+}
+
 template <bool kLoaders, bool kBarrier, int kReads = 6, int kPrio = 0, bool kMfma = true, int kFlight = 16>
 static int run(int* sink, unsigned long long* cycles, const unsigned char* buf, int cus, const char* name) {
     CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&loop_model<kLoaders, kBarrier, kReads, kPrio, kMfma, kFlight>),
@@ -154,9 +363,15 @@ int main() {
     CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, 0));
     CHECK(hipMalloc(&sink, 64));
     CHECK(hipMalloc(&cycles, 32));
-    CHECK(hipMalloc(&buf, 8 * kRegion));
-    CHECK(hipMemset(buf, 1, 8 * kRegion));
+    CHECK(hipMalloc(&buf, 8 * kRegionX));
+    CHECK(hipMemset(buf, 1, 8 * kRegionX));
     int rc = 0;
+    printf("the matrix pipes by themselves (16 and 32 cycles are the pipe's time per instruction):\n");
+    rc |= run_mfma_only<false>(sink, cycles, cus, 1);
+    rc |= run_mfma_only<false>(sink, cycles, cus, 2);
+    rc |= run_mfma_only<true>(sink, cycles, cus, 1);
+    rc |= run_mfma_only<true>(sink, cycles, cus, 2);
+    printf("the kernel's loop: 128 x 128 tile, eight MFMA waves of 64 x 32 on 16x16x64, four loader waves, 32 KiB stages:\n");
     rc |= run<false, false>(sink, cycles, buf, cus, "MFMA waves alone");
     rc |= run<true, false>(sink, cycles, buf, cus, "+ loader waves streaming, no barrier");
     rc |= run<false, true>(sink, cycles, buf, cus, "+ a barrier per half-chunk, no loads");
@@ -167,5 +382,11 @@ int main() {
     rc |= run<true, false, 6, 0, true, 40>(sink, cycles, buf, cus, "loaders with up to 48 loads in flight each, no barrier");
     rc |= run<true, false, 6, 3>(sink, cycles, buf, cus, "loader waves at s_setprio 3, no barrier");
     rc |= run<true, true, 6, 3>(sink, cycles, buf, cus, "loader waves at s_setprio 3, barrier per half-chunk");
+    printf("a 256 x 128 tile: eight self-loading waves of 64 x 64 on 32x32x32 (32 cycles per MFMA = the pipe's rate), 48 KiB stages:\n");
+    rc |= run_x<0, false>(sink, cycles, buf, cus, "arithmetic alone (MFMAs, chain, operand reads)");
+    rc |= run_x<0, true>(sink, cycles, buf, cus, "+ a barrier per stage");
+    rc |= run_x<6, false>(sink, cycles, buf, cus, "+ six loads per wave and stage (3 + 3), no barrier");
+    rc |= run_x<6, true>(sink, cycles, buf, cus, "+ the loads (3 + 3) and the barrier");
+    rc |= run_x<6, true, true>(sink, cycles, buf, cus, "+ the loads (2, 1, 2, 1 behind the k-steps) and the barrier");
     return rc;
 }
