@@ -41,21 +41,38 @@ typedef __amdgpu_buffer_rsrc_t rsrc_t;
 constexpr int kLdsBytes = 136 * 1024;   // 32 KiB of operands + a 96 KiB ring for the loaders + slack: one workgroup per CU
 constexpr size_t kRegion = 256 * 1024;  // what a workgroup's loaders stream, over and over (8 regions: L2-resident)
 
-template <bool kLoaders, bool kBarrier, int kReads, int kPrio, bool kMfma, int kFlight>
+// Bounded wait until an LDS counter reaches a target (the bound only matters if the model is wrong: no wave may spin for ever).
+__device__ __forceinline__ void wait_counter(const volatile unsigned* counter, unsigned target) {
+    for (int spin = 0; spin < (1 << 16); ++spin) {
+        if (*counter >= target) return;
+        __builtin_amdgcn_s_sleep(1);
+    }
+}
+
+// kSync: 0 = the two kinds of waves never meet; 1 = one workgroup barrier per half-chunk (the kernel); 2 = counters in
+// LDS instead: per ring slot, how many loader waves have landed their part of the stage in it and how many MFMA waves
+// have read it for the last time -- an MFMA wave then waits for data only, never for another MFMA wave.
+template <bool kLoaders, int kSync, int kReads, int kPrio, bool kMfma, int kFlight>
 __global__ __launch_bounds__(768) void loop_model(int* sink, int ksteps, unsigned long long* cycles,
                                                   const unsigned char* buf) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     for (int i = threadIdx.x; i < 32768 / 4; i += 768) reinterpret_cast<int*>(lds)[i] = (i * 2654435761u) & 0x3f3f3f3f;
+    volatile unsigned* const landed = reinterpret_cast<volatile unsigned*>(lds + 32768 + 96 * 1024);  // [4] per ring slot
+    volatile unsigned* const freed = landed + 4;                                                      // [4]
+    if (threadIdx.x < 8) landed[threadIdx.x] = 0;
     __syncthreads();
+    constexpr bool kBarrier = (kSync == 1);
     if (wave >= 8) {  // loader waves: 8 loads of 1 KiB per half-chunk each
-        if (!kLoaders && !kBarrier) return;
+        if (!kLoaders && kSync == 0) return;
         const rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char*>(buf) + (blockIdx.x % 8) * kRegion, 0,
                                                            static_cast<int>(kRegion), 0x00020000);
         unsigned off = 0;
         if (kPrio) __builtin_amdgcn_s_setprio(kPrio);
         const unsigned long long t0 = __builtin_readcyclecounter(), w0 = wall_clock64();
         for (int h = 0; h < ksteps / 2; ++h) {
+            // flags: the slot of stage h was read for the last time (as stage h - 4) by all eight MFMA waves
+            if (kSync == 2 && h >= 4) wait_counter(&freed[h & 3], 8u * static_cast<unsigned>(h >> 2));
             if (kLoaders) {
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
@@ -67,9 +84,16 @@ __global__ __launch_bounds__(768) void loop_model(int* sink, int ksteps, unsigne
                 }
                 asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kFlight) : "memory");
             }
+            // flags: with stages h and h - 1 in flight, this wave's part of stage h - 2 has landed
+            if (kSync == 2 && h >= 2 && lane == 0) atomicAdd(const_cast<unsigned*>(&landed[(h - 2) & 3]), 1u);
             if (kBarrier) asm volatile("s_barrier" ::: "memory");
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (kSync == 2 && lane == 0) {
+            const int n = ksteps / 2;
+            atomicAdd(const_cast<unsigned*>(&landed[(n - 2) & 3]), 1u);
+            atomicAdd(const_cast<unsigned*>(&landed[(n - 1) & 3]), 1u);
+        }
         const unsigned long long t1 = __builtin_readcyclecounter(), w1 = wall_clock64();
         if (lane == 0) {
             atomicMax(&cycles[1], t1 - t0);
@@ -115,6 +139,13 @@ __global__ __launch_bounds__(768) void loop_model(int* sink, int ksteps, unsigne
                 __builtin_amdgcn_sched_barrier(0);
             }
             if (kBarrier && half == 0) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            if (kSync == 2 && half == 0) {
+                // the last reads of stage h = ks / 2 are done: its slot is free; the next k-step reads stage h + 1
+                const int h = ks >> 1;
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                if (lane == 0) atomicAdd(const_cast<unsigned*>(&freed[h & 3]), 1u);
+                if (h + 1 < ksteps / 2) wait_counter(&landed[(h + 1) & 3], 4u * static_cast<unsigned>(((h + 1) >> 2) + 1));
+            }
         }
     }
     const unsigned long long t1 = __builtin_readcyclecounter(), w1 = wall_clock64();
@@ -331,15 +362,15 @@ static int run_x(int* sink, unsigned long long* cycles, const unsigned char* buf
     return 0;
 }
 
-template <bool kLoaders, bool kBarrier, int kReads = 6, int kPrio = 0, bool kMfma = true, int kFlight = 16>
+template <bool kLoaders, int kSync, int kReads = 6, int kPrio = 0, bool kMfma = true, int kFlight = 16>
 static int run(int* sink, unsigned long long* cycles, const unsigned char* buf, int cus, const char* name) {
-    CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&loop_model<kLoaders, kBarrier, kReads, kPrio, kMfma, kFlight>),
+    CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&loop_model<kLoaders, kSync, kReads, kPrio, kMfma, kFlight>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes));
     const int ksteps = 4096;
     unsigned long long h[4] = {0, 0, 0, 0};
     for (int rep = 0; rep < 2; ++rep) {  // the first repetition brings the regions into L2
         CHECK(hipMemset(cycles, 0, 32));
-        hipLaunchKernelGGL((loop_model<kLoaders, kBarrier, kReads, kPrio, kMfma, kFlight>), dim3(cus), dim3(768), kLdsBytes, 0,
+        hipLaunchKernelGGL((loop_model<kLoaders, kSync, kReads, kPrio, kMfma, kFlight>), dim3(cus), dim3(768), kLdsBytes, 0,
                            sink, ksteps, cycles, buf);
         CHECK(hipDeviceSynchronize());
         CHECK(hipMemcpy(h, cycles, 32, hipMemcpyDeviceToHost));
@@ -372,16 +403,17 @@ int main() {
     rc |= run_mfma_only<true>(sink, cycles, cus, 1);
     rc |= run_mfma_only<true>(sink, cycles, cus, 2);
     printf("the kernel's loop: 128 x 128 tile, eight MFMA waves of 64 x 32 on 16x16x64, four loader waves, 32 KiB stages:\n");
-    rc |= run<false, false>(sink, cycles, buf, cus, "MFMA waves alone");
-    rc |= run<true, false>(sink, cycles, buf, cus, "+ loader waves streaming, no barrier");
-    rc |= run<false, true>(sink, cycles, buf, cus, "+ a barrier per half-chunk, no loads");
-    rc |= run<true, true>(sink, cycles, buf, cus, "+ loader waves and the barrier per half-chunk");
-    rc |= run<true, false, 4>(sink, cycles, buf, cus, "loaders, no barrier, 4 operand reads per k-step");
-    rc |= run<true, false, 0>(sink, cycles, buf, cus, "loaders, no barrier, no operand reads");
-    rc |= run<true, false, 0, 0, false>(sink, cycles, buf, cus, "loaders next to sleeping waves");
-    rc |= run<true, false, 6, 0, true, 40>(sink, cycles, buf, cus, "loaders with up to 48 loads in flight each, no barrier");
-    rc |= run<true, false, 6, 3>(sink, cycles, buf, cus, "loader waves at s_setprio 3, no barrier");
-    rc |= run<true, true, 6, 3>(sink, cycles, buf, cus, "loader waves at s_setprio 3, barrier per half-chunk");
+    rc |= run<false, 0>(sink, cycles, buf, cus, "MFMA waves alone");
+    rc |= run<true, 0>(sink, cycles, buf, cus, "+ loader waves streaming, no barrier");
+    rc |= run<false, 1>(sink, cycles, buf, cus, "+ a barrier per half-chunk, no loads");
+    rc |= run<true, 1>(sink, cycles, buf, cus, "+ loader waves and the barrier per half-chunk");
+    rc |= run<true, 2>(sink, cycles, buf, cus, "+ loader waves and counters in LDS instead of the barrier");
+    rc |= run<true, 0, 4>(sink, cycles, buf, cus, "loaders, no barrier, 4 operand reads per k-step");
+    rc |= run<true, 0, 0>(sink, cycles, buf, cus, "loaders, no barrier, no operand reads");
+    rc |= run<true, 0, 0, 0, false>(sink, cycles, buf, cus, "loaders next to sleeping waves");
+    rc |= run<true, 0, 6, 0, true, 40>(sink, cycles, buf, cus, "loaders with up to 48 loads in flight each, no barrier");
+    rc |= run<true, 0, 6, 3>(sink, cycles, buf, cus, "loader waves at s_setprio 3, no barrier");
+    rc |= run<true, 1, 6, 3>(sink, cycles, buf, cus, "loader waves at s_setprio 3, barrier per half-chunk");
     printf("a 256 x 128 tile: eight self-loading waves of 64 x 64 on 32x32x32 (32 cycles per MFMA = the pipe's rate), 48 KiB stages:\n");
     rc |= run_x<0, false>(sink, cycles, buf, cus, "arithmetic alone (MFMAs, chain, operand reads)");
     rc |= run_x<0, true>(sink, cycles, buf, cus, "+ a barrier per stage");
