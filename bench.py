@@ -368,6 +368,10 @@ def main() -> int:
     v = ctypes.c_double(0.0)
     _lib.check(_lib.lib.bsi_hip_probe_mfma_i8(ctypes.byref(v), stream), "probe_mfma")
     peaks["int8_mfma_TOPS"] = v.value / 1e12
+    # the same loop on pseudo-random bytes shaped like the dot's images: the clock follows the data's switching
+    # activity, so this is the rate real operands can sustain on the matrix pipes alone
+    _lib.check(_lib.lib.bsi_hip_probe_mfma_i8_operands(1, ctypes.byref(v), stream), "probe_mfma_operands")
+    peaks["int8_mfma_TOPS_random_operands"] = v.value / 1e12
     _lib.check(_lib.lib.bsi_hip_probe_valu_popcount(ctypes.byref(v), stream), "probe_valu")
     peaks["valu_and_bcnt_Tbitmac_s"] = v.value * 32 / 2 / 1e12   # one v_and + one v_bcnt per 32 bit-MACs
     buf = torch.ones(1 << 30, dtype=torch.uint8, device="cuda")
@@ -386,6 +390,8 @@ def main() -> int:
     del buf
     result["measured_peaks"] = peaks
     result["roofline"]["frac_of_measured_mfma_peak"] = (int8_ops / (kern_us * 1e-6) / 1e12) / peaks["int8_mfma_TOPS"]
+    result["roofline"]["frac_of_measured_mfma_peak_random_operands"] = \
+        (int8_ops / (kern_us * 1e-6) / 1e12) / peaks["int8_mfma_TOPS_random_operands"]
 
     # dense baselines of the same shape on the same GPU (resident operands, same event timing)
     Xd, Kd = X.cuda(), K.cuda()

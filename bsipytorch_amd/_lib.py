@@ -80,6 +80,7 @@ PROTOTYPES = {
                           ctypes.POINTER(_f), _vp],
     "bsi_hip_probe_valu_popcount": [ctypes.POINTER(_d), _vp],
     "bsi_hip_probe_mfma_i8": [ctypes.POINTER(_d), _vp],
+    "bsi_hip_probe_mfma_i8_operands": [_i, ctypes.POINTER(_d), _vp],
     "bsi_hip_probe_stream_read": [_vp, _sz, ctypes.POINTER(_d), _vp],
     "bsi_hip_probe_l2_to_lds": [_vp, _sz, _i, ctypes.POINTER(_d), _vp],
     "bsi_hip_timeline_read": [ctypes.POINTER(ctypes.c_ulonglong), _i],

@@ -43,8 +43,19 @@ __global__ void probe_valu_kernel(unsigned* __restrict__ sink, unsigned seed, in
     if (s == 0xFFFFFFFFu) sink[0] = s;
 }
 
-__global__ void probe_mfma_kernel(int* __restrict__ sink, int seed, int iters) {
+__global__ void probe_mfma_kernel(int* __restrict__ sink, int seed, int iters, int random_operands) {
     v4i a = {seed + (int)threadIdx.x, seed, 3, 5}, b = {7, seed, 11, (int)threadIdx.x};
+    if (random_operands) {
+        // pseudo-random bytes shaped like the dot's images: 6-bit values << 2 against 7-bit values << 1
+        unsigned s = (threadIdx.x + 1u + blockIdx.x * 977u) * 2654435761u + static_cast<unsigned>(seed);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            s = s * 1664525u + 1013904223u;
+            a[j] = static_cast<int>((s >> 4) & 0xfcfcfcfcu);
+            s = s * 1664525u + 1013904223u;
+            b[j] = static_cast<int>((s >> 4) & 0xfefefefeu);
+        }
+    }
     v4i c0 = {0, 0, 0, 0}, c1 = c0, c2 = c0, c3 = c0;
     for (int i = 0; i < iters; ++i) {
         c0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c0, 0, 0, 0);
@@ -129,14 +140,19 @@ extern "C" int bsi_hip_probe_valu_popcount(double* lane_ops_per_s, void* stream)
 }
 
 extern "C" int bsi_hip_probe_mfma_i8(double* ops_per_s, void* stream) {
+    return bsi_hip_probe_mfma_i8_operands(0, ops_per_s, stream);
+}
+
+extern "C" int bsi_hip_probe_mfma_i8_operands(int random_operands, double* ops_per_s, void* stream) {
     BSI_REQUIRE(ops_per_s, "null pointer");
+    BSI_REQUIRE(random_operands == 0 || random_operands == 1, "random_operands must be 0 or 1");
     hipStream_t st = as_stream(stream);
     int* sink = nullptr;
     BSI_HIP_CHECK(hipMalloc(&sink, 64));
     const int iters = 4096, blocks = 256 * 8, threads = 256;
     float ms = 0.0f;
     int rc = time_launch(st, 5, &ms, [&] {
-        hipLaunchKernelGGL(probe_mfma_kernel, dim3(blocks), dim3(threads), 0, st, sink, 3, iters);
+        hipLaunchKernelGGL(probe_mfma_kernel, dim3(blocks), dim3(threads), 0, st, sink, 3, iters, random_operands);
     });
     (void)hipFree(sink);
     if (rc) return rc;

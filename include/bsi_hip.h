@@ -372,6 +372,11 @@ int bsi_hip_dot_timed(const uint64_t* A, const int8_t* A_ints8, const float* A_c
  * ops per second) and a streaming read (bytes per second).  Each synchronises. */
 int bsi_hip_probe_valu_popcount(double* lane_ops_per_s, void* stream);
 int bsi_hip_probe_mfma_i8(double* ops_per_s, void* stream);
+/* The same MFMA loop on chosen operand data: random_operands = 0, the near-constant registers of
+ * bsi_hip_probe_mfma_i8 (the chip's ceiling); 1, pseudo-random bytes shaped like the dot's int8 images.  The shader
+ * clock follows the switching activity of the data, so the second is what real operands can sustain.  No counterpart
+ * in the reference: a measuring aid. */
+int bsi_hip_probe_mfma_i8_operands(int random_operands, double* ops_per_s, void* stream);
 int bsi_hip_probe_stream_read(const void* buf_device, size_t bytes, double* bytes_per_s, void* stream);
 /* Timeline build only (make -C bsipytorch_amd/csrc TIMELINE=1 -> libbsi_hip_timeline.so; the ordinary library returns
  * BSI_ERR_INVALID): copies out the wall-clock stamps (100 MHz ticks) that the last int8-image chunk-scale dot left,

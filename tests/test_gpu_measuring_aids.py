@@ -82,6 +82,10 @@ def test_peak_probes_report_rates_within_the_machine(ops):
     assert 1e12 < v.value < 256 * 64 * 2.4e9 * 2
     _lib.check(_lib.lib.bsi_hip_probe_mfma_i8(ctypes.byref(v), st), "bsi_hip_probe_mfma_i8")
     assert 1e15 < v.value <= 5.1e15  # int8 ops per second: above a fifth of, and not above, the published 5.0 POP/s
+    ceiling = v.value
+    _lib.check(_lib.lib.bsi_hip_probe_mfma_i8_operands(1, ctypes.byref(v), st), "bsi_hip_probe_mfma_i8_operands")
+    assert 1e15 < v.value <= ceiling * 1.05  # random operands switch more: never faster than near-constant ones
+    assert _lib.lib.bsi_hip_probe_mfma_i8_operands(2, ctypes.byref(v), st) != 0
     buf = torch.empty((256 << 20,), dtype=torch.uint8, device="cuda")
     buf.zero_()
     _lib.check(_lib.lib.bsi_hip_probe_stream_read(buf.data_ptr(), buf.numel(), ctypes.byref(v), st), "bsi_hip_probe_stream_read")
