@@ -1026,6 +1026,24 @@ FUSED_LINEAR_MAX_ROWS = 4
 FUSED_LINEAR_QUERY_LDS_BYTES = 96 * 1024  # the kernel keeps the rows' int8 image and chunk scales in LDS
 
 
+def _check_bias(bias, R: int, device) -> None:
+    """A bias handed to a kernel is read through its device pointer: anything but a contiguous float32 tensor of [R] on
+    the launch device is refused here (a host pointer would fault the GPU)."""
+    if bias is not None:
+        _check(isinstance(bias, torch.Tensor) and bias.is_cuda and bias.device == device and bias.dtype == torch.float32
+               and bias.dim() == 1 and bias.numel() == R and bias.is_contiguous(),
+               "bias must be a contiguous float32 CUDA tensor of [R] on the device of the call")
+
+
+def device_bias(bias, device):
+    """``bias`` if a kernel on ``device`` can add it in its epilogue (see _check_bias), else None: the caller then adds
+    it afterwards."""
+    if (bias is not None and bias.is_cuda and bias.device == device and bias.dtype == torch.float32 and bias.dim() == 1
+            and bias.is_contiguous()):
+        return bias
+    return None
+
+
 def can_fuse_linear_few_rows(x2d: torch.Tensor, keys: "PrebuiltBSIKeysCUDA") -> bool:
     """Whether linear_few_rows_cuda serves this call: a few rows, 7-or-so-bit chunk-scaled queries without
     clipping, fixed 6-plane tiled keys, the matrix-core route not switched off."""
@@ -1055,6 +1073,7 @@ def linear_few_rows_cuda(x2d: torch.Tensor, keyset_cuda_cap, decimal_places: int
     _check(int(decimal_places) == keys.decimals,
            f"Decimal mismatch between queries and keys: q={int(decimal_places)} k={keys.decimals}")
     Q, R = int(x2d.shape[0]), keys.num_keys
+    _check_bias(bias, R, x2d.device)
     out = torch.empty((Q, R), dtype=torch.float32, device=x2d.device)
     check(lib.bsi_hip_linear_few_rows(x2d.data_ptr(), _dtype_code(x2d), Q, int(x2d.shape[1]), int(decimal_places),
                                       _flags()["bits_q"], keys.words.data_ptr(), keys.slice_weights.data_ptr(), keys.Sb,
@@ -1130,6 +1149,7 @@ def linear_cuda(x2d: torch.Tensor, keyset_cuda_cap, decimal_places: int, bias=No
            f"Decimal mismatch between queries and keys: q={int(decimal_places)} k={keys.decimals}")
     f = _flags()
     Q, d, R = int(x2d.shape[0]), int(x2d.shape[1]), keys.num_keys
+    _check_bias(bias, R, x2d.device)
     bits = f["bits_q"]
     need = int(lib.bsi_hip_linear_workspace_bytes(Q, d, bits))
     capturing = _capturing()

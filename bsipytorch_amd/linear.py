@@ -215,15 +215,14 @@ class BSIQuantizedLinear(nn.Module):
                 if last[4] <= 0:
                     group.__dict__["_last_call"] = None
             else:
-                gb = group.bias if (fp32 and group.bias is not None) else None
+                gb = bsi_ops.device_bias(group.bias, batch_inputs.device) if fp32 else None
                 all_scores = bsi_ops.linear_cuda(batch_inputs, keys, self.decimalPlaces, gb, _keys_to_warm(group.next_layer), True)
                 group.__dict__["_last_call"] = [key, batch_inputs, all_scores, gb is not None, len(group.members) - 1]
                 scores, bias_done = all_scores[:, start:stop], gb is not None
                 c["dot_calls"] += 1
                 c["build_calls"] += int(bsi_ops._last_linear_rebuilt[0])
         else:
-            b = self.bias if (fp32 and self.bias is not None and self.bias.dtype == torch.float32
-                              and self.bias.is_cuda and self.bias.is_contiguous()) else None
+            b = bsi_ops.device_bias(self.bias, batch_inputs.device) if fp32 else None
             scores = bsi_ops.linear_cuda(batch_inputs, keys, self.decimalPlaces, b, _keys_to_warm(c.get("_next_bsi_layer")), True)
             bias_done = b is not None
             c["dot_calls"] += 1
@@ -266,14 +265,14 @@ class BSIQuantizedLinear(nn.Module):
                 if last[4] <= 0:
                     group.__dict__["_last_few"] = None
             else:
-                gb = group.bias if (fp32 and group.bias is not None) else None
+                gb = bsi_ops.device_bias(group.bias, batch_inputs.device) if fp32 else None
                 all_scores = bsi_ops.linear_few_rows_cuda(batch_inputs, keys, self.decimalPlaces, gb, True)
                 # holds the input's storage (so that its address is not reused) until every member has been served
                 group.__dict__["_last_few"] = [key, batch_inputs, all_scores, gb is not None, len(group.members) - 1]
                 scores, bias_done = all_scores[:, start:stop], gb is not None
                 c["dot_calls"] += 1
         else:
-            b = self.bias if (fp32 and self.bias is not None and self.bias.dtype == torch.float32) else None
+            b = bsi_ops.device_bias(self.bias, batch_inputs.device) if fp32 else None
             scores, bias_done = bsi_ops.linear_few_rows_cuda(batch_inputs, keys, self.decimalPlaces, b, True), b is not None
             c["dot_calls"] += 1
         q_rows = int(batch_inputs.shape[0])
@@ -335,9 +334,10 @@ class _FusedSiblings:
             if last[3] <= 0:  # every member has had its columns: nothing is held until the next forward
                 self._last = None
             return out, 0, 0.0, 0.0, bias_done
-        bias_done = bool(want_bias and self.bias is not None)
+        gb = bsi_ops.device_bias(self.bias, self.keys.words.device) if want_bias else None
+        bias_done = gb is not None
         out, ns_total, ns_q, ns_s = bsi_ops.batch_dot_product_multiquery_cuda_batch_caps(
-            qcap, self.keys, self.bias if bias_done else None, _keys_to_warm(self.next_layer))
+            qcap, self.keys, gb, _keys_to_warm(self.next_layer))
         self._last = [qcap, out, bias_done, len(self.members) - 1]
         return out, ns_total, ns_q, ns_s, bias_done
 

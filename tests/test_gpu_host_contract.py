@@ -137,3 +137,52 @@ def test_layer_and_fused_qkv_under_inference_mode(ops, monkeypatch, dtype, rows)
                 xi.add_(1.0)                    # in-place work on it must not be mistaken for "unchanged"
                 got2 = model(xi)
                 assert all(torch.equal(a, b) for a, b in zip(got2, want2))
+
+
+@pytest.mark.parametrize("rows", [2, 40])
+@pytest.mark.parametrize("fuse", [False, True])
+def test_layer_with_its_bias_on_the_host(ops, rows, fuse):
+    """A layer quantised while it lives on the CPU keeps its bias there (the reference moves it per call,
+    verify_accuracy_bsi.py:207-211).  No kernel may be handed that host pointer: the few-rows kernel, the one-call path
+    and the fused q/k/v group add such a bias afterwards, with the result of a layer whose bias is on the device; the
+    library-level entry points refuse it."""
+    import torch.nn as nn
+    from bsipytorch_amd.linear import BSIQuantizedLinear, forget_shared_builds, fuse_sibling_layers
+
+    torch.manual_seed(5)
+    D, R = 512, (128 if fuse else 100)  # siblings are stacked only when their key counts are multiples of 64
+
+    class Block(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.q_proj, self.k_proj, self.v_proj = nn.Linear(D, R), nn.Linear(D, R), nn.Linear(D, R)
+
+    def quantised(move_bias):
+        torch.manual_seed(6)
+        blk = Block()
+        for name in ("q_proj", "k_proj", "v_proj"):
+            layer = BSIQuantizedLinear(getattr(blk, name), decimalPlaces=2, compress_threshold=0.5)
+            if move_bias:
+                layer.cuda()  # moves the bias buffer; the keys are on the device either way
+            setattr(blk, name, layer)
+        if fuse:
+            assert fuse_sibling_layers(blk) == 1
+        return blk
+
+    x = torch.randn(rows, D, device="cuda")
+    host, dev = quantised(False), quantised(True)
+    assert not host.q_proj.bias.is_cuda and dev.q_proj.bias.is_cuda
+    for name in ("q_proj", "k_proj", "v_proj"):
+        a, b = getattr(host, name)(x), getattr(dev, name)(x)
+        torch.cuda.synchronize()
+        assert torch.equal(a, b), name
+    forget_shared_builds()
+    keys = dev.q_proj._bsi_keys_cuda
+    with pytest.raises(RuntimeError, match="bias must be"):
+        ops.linear_cuda(x, keys, 2, bias=host.q_proj.bias.detach())
+    if rows <= ops.FUSED_LINEAR_MAX_ROWS:
+        with pytest.raises(RuntimeError, match="bias must be"):
+            ops.linear_few_rows_cuda(x, keys, 2, bias=host.q_proj.bias.detach())
+    with pytest.raises(RuntimeError, match="bias must be"):
+        ops.linear_cuda(x, keys, 2, bias=torch.zeros(R + 1, device="cuda"))
+    forget_shared_builds()
