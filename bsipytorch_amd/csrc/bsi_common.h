@@ -83,9 +83,16 @@ __device__ __forceinline__ float load_as_float<__hip_bfloat16>(const __hip_bfloa
 
 // round half away from zero of x (x = (double)(float)v * 10^dec); the multiply is done by the
 // caller with __dmul_rn so that it is never contracted with the + 0.5
+// Values the conversion cannot hold are given what the reference's own conversion gives them on its hardware (the C++
+// cast is undefined there; cvt.rzi.s64.f64 saturates and turns a NaN into -2^63): magnitudes of 2^63 and more,
+// the infinities included, become +-(2^63 - 1), a NaN becomes -2^63.
+__device__ __forceinline__ long long magnitude_to_ll(double y) {  // y >= 0
+    return y >= 9223372036854775808.0 ? 9223372036854775807LL : static_cast<long long>(y);
+}
 __device__ __forceinline__ long long round_half_away(double x) {
-    if (x >= 0.0) return static_cast<long long>(floor(__dadd_rn(x, 0.5)));
-    return -static_cast<long long>(floor(__dadd_rn(-x, 0.5)));
+    if (x != x) return static_cast<long long>(0x8000000000000000ULL);
+    if (x >= 0.0) return magnitude_to_ll(floor(__dadd_rn(x, 0.5)));
+    return -magnitude_to_ll(floor(__dadd_rn(-x, 0.5)));
 }
 
 __device__ __forceinline__ long long round_scaled(float f, double dec_scale) {
@@ -93,7 +100,7 @@ __device__ __forceinline__ long long round_scaled(float f, double dec_scale) {
 }
 
 __device__ __forceinline__ unsigned long long uabs_ll(long long v) {
-    return static_cast<unsigned long long>(v >= 0 ? v : -v);
+    return v >= 0 ? static_cast<unsigned long long>(v) : 0ULL - static_cast<unsigned long long>(v);  // -2^63 -> 2^63
 }
 
 // bits needed for max_abs minus the magnitude bits available; optional outlier clipping

@@ -34,10 +34,17 @@
 #define BSI_CHUNK_ELEMS 256 /* elements per scale chunk: bsi_cuda_kernels_quant.cuh:170 */
 #define BSI_CHUNK_WORDS 4   /* 64-bit words per chunk: bsi_cuda_kernels_dot.cuh:1306 */
 
-/* bsi_cuda_kernels_quant.cuh:24-29 (bsi_round_half_away_to_ll) */
+/* bsi_cuda_kernels_quant.cuh:24-29 (bsi_round_half_away_to_ll).  The cast there is undefined for values an int64
+ * cannot hold; on the reference's hardware it is cvt.rzi.s64.f64, which saturates and turns a NaN into -2^63.  That
+ * is written out here: magnitudes of 2^63 and more (the infinities included) give +-(2^63 - 1), a NaN (which fails
+ * x >= 0 and takes the second branch, where the negation of -2^63 wraps) gives -2^63. */
+static int64_t magnitude_to_ll(double y) { /* y >= 0 */
+    return y >= 9223372036854775808.0 ? INT64_MAX : (int64_t)y;
+}
 int64_t bsi_oracle_round_half_away(double x) {
-    if (x >= 0.0) return (int64_t)floor(x + 0.5);
-    return -(int64_t)floor(-x + 0.5);
+    if (x != x) return INT64_MIN;
+    if (x >= 0.0) return magnitude_to_ll(floor(x + 0.5));
+    return -magnitude_to_ll(floor(-x + 0.5));
 }
 
 /* bsi_cuda_kernels_quant.cuh:110-121 (quantize_round_to_int64_batch_kernel):
@@ -47,7 +54,7 @@ void bsi_oracle_round_to_int64(const float* x, int64_t n, int decimal_places, in
     for (int64_t i = 0; i < n; ++i) out[i] = bsi_oracle_round_half_away((double)x[i] * dec_scale);
 }
 
-static uint64_t uabs64(int64_t v) { return (uint64_t)(v >= 0 ? v : -v); } /* quant.cuh:31-33 */
+static uint64_t uabs64(int64_t v) { return v >= 0 ? (uint64_t)v : 0 - (uint64_t)v; } /* quant.cuh:31-33; -2^63 -> 2^63 */
 
 /* bsi_cuda_kernels_quant.cuh:82-108 (bsi_compute_shift) */
 int bsi_oracle_compute_shift(uint64_t max_abs, double sum_abs, int count, int fixed_bits, float clip_k) {

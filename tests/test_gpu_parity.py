@@ -133,6 +133,36 @@ def test_build_huge_magnitudes_take_the_wide_path(hip, oracle):
     assert shifts.max() >= 30
 
 
+@pytest.mark.parametrize("Q", [1, 4, 33, 128])
+@pytest.mark.parametrize("dt", [torch.float32, torch.float16, torch.bfloat16])
+def test_activations_an_int64_cannot_hold(ops, oracle, Q, dt):
+    """Infinities, NaNs and magnitudes of 2^63 and more after scaling: the conversion is written out (saturation, NaN ->
+    -2^63, as on the reference's hardware) and every route -- the builder, the few-rows kernel with the build inside,
+    the one-call layer path -- gives the oracle's planes, scales and outputs for them, bit for bit."""
+    rng = np.random.default_rng(Q)
+    R, D = 96, 1024
+    k = (rng.standard_normal((R, D)) * 0.02).astype(np.float32)
+    x = rng.standard_normal((Q, D)).astype(np.float32)
+    x[0, 0], x[0, 1], x[-1, 5], x[0, 2], x[0, 3] = np.inf, -np.inf, np.nan, 1e-45, -0.0
+    if dt == torch.float32:
+        x[0, 300], x[-1, 700], x[0, 600] = 3e38, -1e30, 9.3e16  # 9.3e18 after scaling: just past 2^63
+    xt = torch.from_numpy(x).to(dt)
+    x = xt.float().numpy()
+    qb, kb = oracle.build_queries(x), oracle.build_keys(k)
+    _, want = oracle.dot_fixed(qb["words"], qb["scales"], kb["words"], kb["scales"], oracle.scale_inv(2, 2), want_ints=False)
+    kcap, *_ = ops.build_bsi_keys_cuda(torch.from_numpy(k), 2, 0.5)
+    qcap = ops.build_bsi_queries_cuda_batch_packed(xt.cuda(), 2, 0.5)
+    np.testing.assert_array_equal(host_u64(qcap.words), qb["words"])
+    np.testing.assert_array_equal(qcap.chunk_scales.cpu().numpy(), qb["scales"])
+    out, *_ = ops.batch_dot_product_multiquery_cuda_batch_caps(qcap, kcap)
+    np.testing.assert_array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    if Q <= ops.FUSED_LINEAR_MAX_ROWS:
+        y = ops.linear_few_rows_cuda(xt.cuda(), kcap, 2)
+        np.testing.assert_array_equal(y.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    y = ops.linear_cuda(xt.cuda(), kcap, 2)
+    np.testing.assert_array_equal(y.cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
 @pytest.mark.parametrize("dec", [0, 1, 2, 3])
 @pytest.mark.parametrize("per_wave", [0, 1, 2, 4, 8])
 def test_build_rounding_routes_and_items_per_wave(hip, oracle, dec, per_wave):

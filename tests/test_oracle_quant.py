@@ -30,6 +30,28 @@ def test_round_half_away_grid(oracle):
     assert oracle.round_half_away(-0.0) == 0
 
 
+def test_round_half_away_of_what_an_int64_cannot_hold(oracle):
+    """The reference casts floor(x + 0.5) to long long (bsi_cuda_kernels_quant.cuh:24-29), which C++ leaves undefined
+    past the int64 range; on its hardware the cast is a saturating conversion that turns a NaN into -2^63.  The oracle
+    writes that out: +-(2^63 - 1) for magnitudes of 2^63 and more, infinities included; -2^63 for a NaN (it fails
+    x >= 0, and the negation of -2^63 wraps); everything below 2^63 converts exactly."""
+    big, small = 2 ** 63 - 1, -(2 ** 63)
+    assert oracle.round_half_away(float("inf")) == big
+    assert oracle.round_half_away(float("-inf")) == -big
+    assert oracle.round_half_away(float("nan")) == small
+    assert oracle.round_half_away(2.0 ** 63) == big and oracle.round_half_away(-(2.0 ** 63)) == -big
+    assert oracle.round_half_away(1e300) == big and oracle.round_half_away(-1e300) == -big
+    below = float(np.nextafter(2.0 ** 63, 0.0))  # the largest double under 2^63: an integer, converted exactly
+    assert oracle.round_half_away(below) == int(below) and oracle.round_half_away(-below) == -int(below)
+    # through the whole query quantiser: the chunk of such a value gets the shift of a 64-bit magnitude
+    x = np.zeros((1, 512), dtype=np.float32)
+    x[0, 3], x[0, 7], x[0, 300] = np.inf, 5.0, np.nan
+    ints, shifts, scales = oracle.quantize_fixed(x, 2, 7, True)
+    assert shifts.tolist() == [[57, 58]]           # bit_length(2^63 - 1) - 6, bit_length(2^63) - 6
+    assert ints[0, 3] == 63 and ints[0, 7] == 0    # (2^63 - 1 + 2^56) >> 57 = 64, clamped to 63; 500 >> 57 = 0
+    assert ints[0, 300] == -32                     # -((2^63 + 2^57) >> 58)
+
+
 def test_round_to_int64_random_fp32(oracle):
     rng = np.random.default_rng(1)
     x = np.concatenate([
