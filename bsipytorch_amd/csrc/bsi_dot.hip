@@ -32,6 +32,12 @@
 
 namespace bsi {
 
+// The scale of a key row as the fixed-bit dots use it: the magnitude of its slice-0 weight, 2^shift_r.  (With a
+// single key slice, slice 0 is the sign slice and its weight is negative; the sign of every product is already in
+// the plane signs s_ij the kernels apply.)
+__device__ __forceinline__ float key_factor(float slice0_weight) { return fabsf(slice0_weight); }
+
+
 typedef int v4i __attribute__((ext_vector_type(4)));
 
 // In-place transpose of the 8x8 bit matrices (row = register index, column = bit within byte) held
@@ -335,7 +341,7 @@ __global__ __launch_bounds__(kMfmaBlock) void dot_mfma_kernel(
         const int64_t rb = r0 + wr * 64 + a * 16 + lg * 4;
         float bs[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) bs[e] = (rb + e < R) ? Bw[(rb + e) * Sb] : 0.0f;
+        for (int e = 0; e < 4; ++e) bs[e] = (rb + e < R) ? key_factor(Bw[(rb + e) * Sb]) : 0.0f;
 #pragma unroll
         for (int b = 0; b < 4; ++b) {
             const int64_t q = q0 + wq * 64 + b * 16 + ln;
@@ -650,7 +656,7 @@ __global__ __launch_bounds__(kWsBlock) void dot_mfma_ws_kernel(
             const int64_t rb = r0 + wr * 64 + a * 16 + lg * 4;
             float bs[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) bs[e] = (rb + e < R) ? Bw[(rb + e) * SB] : 0.0f;
+            for (int e = 0; e < 4; ++e) bs[e] = (rb + e < R) ? key_factor(Bw[(rb + e) * SB]) : 0.0f;
 #pragma unroll
             for (int b = 0; b < 2; ++b) {
                 const int64_t q = q0 + wq * 32 + b * 16 + ln;
@@ -1361,7 +1367,7 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
             const int rl = wr * (WM * 16) + a * 16 + lg * 4;  // row of the tile
             const float4 w4 = *reinterpret_cast<const float4*>(epi + rl);
             const float4 b4 = *reinterpret_cast<const float4*>(epi + TM + rl);
-            bs[a][0] = w4.x, bs[a][1] = w4.y, bs[a][2] = w4.z, bs[a][3] = w4.w;
+            bs[a][0] = key_factor(w4.x), bs[a][1] = key_factor(w4.y), bs[a][2] = key_factor(w4.z), bs[a][3] = key_factor(w4.w);
             bi[a][0] = b4.x, bi[a][1] = b4.y, bi[a][2] = b4.z, bi[a][3] = b4.w;
         }
     }
@@ -1597,7 +1603,7 @@ __global__ __launch_bounds__((I8WCfg<WN>::kBlock)) void dot_mfma_i8w_kernel(
             const int rl = wr * 64 + a * 16 + lg * 4;
             const float4 w4 = *reinterpret_cast<const float4*>(epi + rl);
             const float4 b4 = *reinterpret_cast<const float4*>(epi + TM + rl);
-            bs[a][0] = w4.x, bs[a][1] = w4.y, bs[a][2] = w4.z, bs[a][3] = w4.w;
+            bs[a][0] = key_factor(w4.x), bs[a][1] = key_factor(w4.y), bs[a][2] = key_factor(w4.z), bs[a][3] = key_factor(w4.w);
             bi[a][0] = b4.x, bi[a][1] = b4.y, bi[a][2] = b4.z, bi[a][3] = b4.w;
         }
     }
@@ -2404,7 +2410,7 @@ __global__ __launch_bounds__(kValuBlock) void dot_valu_kernel(
     for (int b = 0; b < 4; ++b) {
         const int64_t r = r0 + tr + 16 * b;
         if (r >= R) continue;
-        const float bs = Bw[r * SB];
+        const float bs = key_factor(Bw[r * SB]);
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
             const int64_t q = q0 + tq + 16 * a;
@@ -2413,32 +2419,37 @@ __global__ __launch_bounds__(kValuBlock) void dot_valu_kernel(
     }
 }
 
-// Any Sa, Sb up to 16: one thread per output, planes read straight from global memory.
+// Any Sa, Sb up to 16: one thread per output, planes read straight from global memory.  tiled: the key planes are in
+// the tiled16 layout (word (r, j, 4 c + g) at (((r / 16) chunks + c) Sb + j) 64 + 16 g + r % 16) instead of [R, Sb, W64].
 __global__ void dot_valu_generic_kernel(const unsigned long long* __restrict__ A, const float* __restrict__ qscale,
                                         int qscale_stride, int Sa, const unsigned long long* __restrict__ B,
                                         const float* __restrict__ Bw, int Sb, int W64, int chunks, int64_t R,
                                         int64_t Q, float scale_inv, int64_t R_total, float* __restrict__ out,
-                                        int* __restrict__ chunk_ints) {
+                                        int* __restrict__ chunk_ints, int tiled) {
     const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (idx >= Q * R) return;
     const int64_t q = idx / R;
     const int64_t r = idx - q * R;
     const unsigned long long* Aq = A + static_cast<size_t>(q) * Sa * W64;
     const unsigned long long* Br = B + static_cast<size_t>(r) * Sb * W64;
+    const unsigned long long* Bt = B + static_cast<size_t>(r >> 4) * chunks * Sb * 64 + (r & 15);  // the row's 16-key tile
     float acc = 0.0f;
     for (int c = 0; c < chunks; ++c) {
         int I = 0;
         for (int i = 0; i < Sa; ++i)
             for (int j = 0; j < Sb; ++j) {
                 int cnt = 0;
-                for (int w = c * 4; w < c * 4 + 4 && w < W64; ++w) cnt += __popcll(Aq[i * W64 + w] & Br[j * W64 + w]);
+                for (int w = c * 4; w < c * 4 + 4 && w < W64; ++w) {
+                    const unsigned long long bw = tiled ? Bt[(static_cast<size_t>(c) * Sb + j) * 64 + (w & 3) * 16] : Br[j * W64 + w];
+                    cnt += __popcll(Aq[i * W64 + w] & bw);
+                }
                 const int v = cnt << (i + j);
                 I = ((i == Sa - 1) != (j == Sb - 1)) ? I - v : I + v;
             }
         if (chunk_ints) chunk_ints[(static_cast<size_t>(q) * R + r) * chunks + c] = I;
         acc = fmaf(static_cast<float>(I), qscale[q * qscale_stride + ((qscale_stride == 1) ? 0 : c)], acc);
     }
-    out[static_cast<size_t>(q) * R_total + r] = (acc * Bw[r * Sb]) * scale_inv;
+    out[static_cast<size_t>(q) * R_total + r] = (acc * key_factor(Bw[r * Sb])) * scale_inv;
 }
 
 // Weighted-slice dot for operands whose slice weights are arbitrary floats (the decimal builder's
@@ -2913,13 +2924,11 @@ static int dot_launch(const uint64_t* A, const int8_t* A_ints8, const float* A_c
         BSI_LAUNCH_CHECK("dot_valu_kernel");
         return BSI_OK;
     }
-    if (b_layout != BSI_LAYOUT_CANONICAL)
-        return fail(BSI_ERR_UNSUPPORTED, "generic VALU kernel reads canonical key planes only");
     const int64_t total = Q * R;
     hipLaunchKernelGGL(dot_valu_generic_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, st,
                        reinterpret_cast<const unsigned long long*>(A), A_chunk_scales, A_scale_stride, Sa,
                        reinterpret_cast<const unsigned long long*>(B), Bw, Sb, W64, chunks, R, Q, scale_inv, R_total,
-                       out, chunk_ints);
+                       out, chunk_ints, b_layout == BSI_LAYOUT_TILED16 ? 1 : 0);
     BSI_LAUNCH_CHECK("dot_valu_generic_kernel");
     return BSI_OK;
 }

@@ -204,7 +204,7 @@ size_t bsi_hip_dot_workspace_bytes(int64_t Q, int W64, int core);
  *                  into `workspace` when the MFMA core runs)
  *   A_chunk_scales float [Q, A_scale_stride]; A_scale_stride == chunks for per-chunk scales,
  *                  1 for one scale per row (broadcast over chunks)
- *   B              key words in `b_layout`; Bw float [R, Sb] slice weights (only Bw[r*Sb] is read)
+ *   B              key words in `b_layout`; Bw float [R, Sb] slice weights (only Bw[r*Sb] is read, and its magnitude used: the row scale 2^shift_r)
  *   out            float [Q, R_total] (row stride R_total >= R); every element [q, r<R] is written
  *   chunk_ints     optional int32 [Q, R, chunks]: the integer accumulators I (parity checks)
  * Sa, Sb in [2, 8] for the MFMA core and [1, 16] for the VALU core.

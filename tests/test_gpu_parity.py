@@ -597,7 +597,7 @@ def test_hybrid_query_dot_decodes_inline(ops, oracle, monkeypatch):
 
 
 @pytest.mark.parametrize("Sa,Sb", [(8, 8), (5, 4), (2, 2), (7, 5), (3, 7)])
-@pytest.mark.parametrize("core,tiled", [(1, False), (2, True), (2, "int8-128"), (2, "int8-1284"), (2, "int8-12864"), (2, "int8-64"), (2, "int8-6432")])
+@pytest.mark.parametrize("core,tiled", [(1, False), (1, True), (2, True), (2, "int8-128"), (2, "int8-1284"), (2, "int8-12864"), (2, "int8-64"), (2, "int8-6432")])
 def test_dot_other_bit_widths(hip, oracle, Sa, Sb, core, tiled):
     Q, R, d = 19, 35, 1024
     x, k, qb, kb, want_ints, want_out = _oracle_case(oracle, Q, R, d, seed=Sa * 10 + Sb, ksigma=0.05, bits_q=Sa, bits_k=Sb)
@@ -606,12 +606,35 @@ def test_dot_other_bit_widths(hip, oracle, Sa, Sb, core, tiled):
     np.testing.assert_array_equal(out, want_out)
 
 
+@pytest.mark.parametrize("Sa,Sb", [(7, 1), (1, 6), (1, 1), (9, 1), (2, 1), (1, 12)])
+@pytest.mark.parametrize("core", [0, 1])
+def test_dot_single_slice_operands(hip, oracle, Sa, Sb, core):
+    """One-bit two's-complement operands hold 0 and -1: their only slice is the sign slice, and the keys' slice-0
+    weight, which the dots use as the row scale, is then negative.  The sign of the products is in the plane signs
+    alone: outputs and integer accumulators are the oracle's.  (The matrix-core route takes 2 to 8 bits and says so.)"""
+    Q, R, d = 21, 37, 768
+    x, k, qb, kb, want_ints, want_out = _oracle_case(oracle, Q, R, d, seed=Sa * 20 + Sb, ksigma=0.05, bits_q=Sa, bits_k=Sb)
+    if Sb == 1:
+        assert (kb["slice_weights"] < 0).all() and set(np.unique(kb["ints"])) <= {0, -1}
+    ints, out = _run_dot(hip, qb, kb, Q, R, 12, Sa, Sb, core, tiled=False, with_ints8=False)
+    np.testing.assert_array_equal(ints, want_ints)
+    np.testing.assert_array_equal(out, want_out)
+    assert np.any(want_out != 0)
+    L = hip.lib
+    t = torch.zeros(64, device="cuda")
+    rc = L.bsi_hip_dot(t.data_ptr(), None, t.data_ptr(), 1, Sa, 1, t.data_ptr(), 0, t.data_ptr(), Sb, 1, 1, 1.0, 1,
+                       t.data_ptr(), None, 2, t.data_ptr(), 256, st())
+    if min(Sa, Sb) == 1 or max(Sa, Sb) > 8:
+        assert rc == 3 and b"MFMA core needs" in L.bsi_hip_last_error()
+
+
 def test_dot_wide_planes_valu_only(hip, oracle):
     Q, R, d = 6, 10, 512
     x, k, qb, kb, want_ints, want_out = _oracle_case(oracle, Q, R, d, seed=99, ksigma=0.5, bits_q=12, bits_k=10)
-    ints, out = _run_dot(hip, qb, kb, Q, R, 8, 12, 10, 0, tiled=False, with_ints8=False)  # auto -> VALU
-    np.testing.assert_array_equal(ints, want_ints)
-    np.testing.assert_array_equal(out, want_out)
+    for tiled in (False, True):
+        ints, out = _run_dot(hip, qb, kb, Q, R, 8, 12, 10, 0, tiled=tiled, with_ints8=False)  # auto -> VALU
+        np.testing.assert_array_equal(ints, want_ints)
+        np.testing.assert_array_equal(out, want_out)
     L = hip.lib
     t = torch.zeros(8, device="cuda")
     rc = L.bsi_hip_dot(t.data_ptr(), None, t.data_ptr(), 2, 12, 8, t.data_ptr(), 0, t.data_ptr(), 10, 1, 1, 1.0, 1,
@@ -827,6 +850,27 @@ def test_build_and_dot_replay_from_a_hip_graph(ops):
 
 
 # ------------------------------------------------------------------ through the bsi_ops mirror
+
+
+@pytest.mark.parametrize("bq,bk", [(9, 6), (7, 10), (12, 10), (16, 16), (2, 2), (8, 8), (4, 9)])
+@pytest.mark.parametrize("Q,R,D", [(1, 50, 512), (20, 100, 1024), (140, 130, 768), (3, 40, 700)])
+def test_ops_other_fixed_bit_widths(ops, oracle, monkeypatch, bq, bk, Q, R, D):
+    """BSI_FIXED_BITS_QUERIES / BSI_FIXED_BITS_KEYS other than 7 / 6, wider than the matrix cores take included: the
+    keys are kept tiled all the same, and the popcount kernel for any width reads them there (it used to refuse every
+    layout but the canonical one, so such a dot failed from 33 rows up and for rows without chunk scales)."""
+    monkeypatch.setenv("BSI_FIXED_BITS_QUERIES", str(bq))
+    monkeypatch.setenv("BSI_FIXED_BITS_KEYS", str(bk))
+    ops._reset_flag_cache()
+    rng = np.random.default_rng(bq * 100 + bk + Q)
+    x = rng.standard_normal((Q, D)).astype(np.float32)
+    k = (rng.standard_normal((R, D)) * 0.05).astype(np.float32)
+    qb, kb = oracle.build_queries(x, 2, bq), oracle.build_keys(k, 2, bk)
+    _, want = oracle.dot_fixed(qb["words"], qb["scales"], kb["words"], kb["scales"], oracle.scale_inv(2, 2), want_ints=False)
+    kcap, *_ = ops.build_bsi_keys_cuda(torch.from_numpy(k), 2, 0.5)
+    qcap = ops.build_bsi_queries_cuda_batch_packed(torch.from_numpy(x).cuda(), 2, 0.5)
+    assert qcap.Sa == bq and kcap.Sb == bk
+    out, *_ = ops.batch_dot_product_multiquery_cuda_batch_caps(qcap, kcap)
+    np.testing.assert_array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32))
 
 
 def test_reference_known_answers_gpu(ops, monkeypatch):
