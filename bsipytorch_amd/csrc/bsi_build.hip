@@ -730,7 +730,7 @@ extern "C" int bsi_hip_build_fixed(const void* x, int dtype, int64_t Q, int64_t 
                                    int chunk_scale, float clip_k, uint64_t* words, int32_t* shifts, float* scales,
                                    int8_t* ints8, void* stream) {
     BSI_REQUIRE(Q >= 0 && d >= 0, "negative size");
-    BSI_REQUIRE(fixed_bits >= 2 && fixed_bits <= 32, "fixed_bits must be in [2, 32]");
+    BSI_REQUIRE(fixed_bits >= 2 && fixed_bits <= 63, "fixed_bits must be in [2, 63]");
     BSI_REQUIRE(ints8 == nullptr || fixed_bits <= 8, "int8 output needs fixed_bits <= 8");
     if (Q == 0 || d == 0) return BSI_OK;
     BSI_REQUIRE(x && words && shifts && scales, "null pointer");

@@ -2419,7 +2419,10 @@ __global__ __launch_bounds__(kValuBlock) void dot_valu_kernel(
     }
 }
 
-// Any Sa, Sb up to 16: one thread per output, planes read straight from global memory.  tiled: the key planes are in
+// Any Sa, Sb up to 63 (where the reference clamps its fixed-bit flags, bsi_vector_cuda.cpp:256-262): one thread per
+// output, planes read straight from global memory.  The chunk's integer is summed modulo 2^64 (a term shifted by 64
+// or more is a multiple of 2^64), which is the integer dot of the chunk whenever that fits 64 bits; the per-chunk
+// integers stored for parity checks are its low 32 bits.  tiled: the key planes are in
 // the tiled16 layout (word (r, j, 4 c + g) at (((r / 16) chunks + c) Sb + j) 64 + 16 g + r % 16) instead of [R, Sb, W64].
 __global__ void dot_valu_generic_kernel(const unsigned long long* __restrict__ A, const float* __restrict__ qscale,
                                         int qscale_stride, int Sa, const unsigned long long* __restrict__ B,
@@ -2435,7 +2438,7 @@ __global__ void dot_valu_generic_kernel(const unsigned long long* __restrict__ A
     const unsigned long long* Bt = B + static_cast<size_t>(r >> 4) * chunks * Sb * 64 + (r & 15);  // the row's 16-key tile
     float acc = 0.0f;
     for (int c = 0; c < chunks; ++c) {
-        int I = 0;
+        unsigned long long I = 0ULL;
         for (int i = 0; i < Sa; ++i)
             for (int j = 0; j < Sb; ++j) {
                 int cnt = 0;
@@ -2443,11 +2446,11 @@ __global__ void dot_valu_generic_kernel(const unsigned long long* __restrict__ A
                     const unsigned long long bw = tiled ? Bt[(static_cast<size_t>(c) * Sb + j) * 64 + (w & 3) * 16] : Br[j * W64 + w];
                     cnt += __popcll(Aq[i * W64 + w] & bw);
                 }
-                const int v = cnt << (i + j);
+                const unsigned long long v = (i + j < 64) ? static_cast<unsigned long long>(cnt) << (i + j) : 0ULL;
                 I = ((i == Sa - 1) != (j == Sb - 1)) ? I - v : I + v;
             }
-        if (chunk_ints) chunk_ints[(static_cast<size_t>(q) * R + r) * chunks + c] = I;
-        acc = fmaf(static_cast<float>(I), qscale[q * qscale_stride + ((qscale_stride == 1) ? 0 : c)], acc);
+        if (chunk_ints) chunk_ints[(static_cast<size_t>(q) * R + r) * chunks + c] = static_cast<int>(I);
+        acc = fmaf(static_cast<float>(static_cast<long long>(I)), qscale[q * qscale_stride + ((qscale_stride == 1) ? 0 : c)], acc);
     }
     out[static_cast<size_t>(q) * R_total + r] = (acc * key_factor(Bw[r * Sb])) * scale_inv;
 }
@@ -2846,7 +2849,7 @@ static int dot_launch(const uint64_t* A, const int8_t* A_ints8, const float* A_c
     *bias_fused = false;
     BSI_REQUIRE(Q >= 0 && R >= 0, "negative Q or R");
     BSI_REQUIRE(W64 >= 1, "W64 must be >= 1");
-    BSI_REQUIRE(Sa >= 1 && Sa <= 16 && Sb >= 1 && Sb <= 16, "Sa and Sb must be in [1, 16]");
+    BSI_REQUIRE(Sa >= 1 && Sa <= 63 && Sb >= 1 && Sb <= 63, "Sa and Sb must be in [1, 63]");
     BSI_REQUIRE(R_total >= R, "R_total must be >= R");
     BSI_REQUIRE(b_layout == BSI_LAYOUT_CANONICAL || b_layout == BSI_LAYOUT_TILED16 || b_layout == BSI_LAYOUT_INT8 ||
                     b_layout == BSI_LAYOUT_INT8_TILED,

@@ -873,6 +873,34 @@ def test_ops_other_fixed_bit_widths(ops, oracle, monkeypatch, bq, bk, Q, R, D):
     np.testing.assert_array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32))
 
 
+@pytest.mark.parametrize("bq,bk", [(17, 17), (20, 33), (32, 32), (63, 63)])
+@pytest.mark.parametrize("Q,R,D", [(1, 50, 512), (40, 100, 1024), (3, 40, 700)])
+def test_ops_fixed_bit_widths_up_to_63(ops, oracle, monkeypatch, bq, bk, Q, R, D):
+    """The reference takes fixed-bit flags up to 63 (bsi_vector_cuda.cpp:256-262).  With 17 bits and more nothing of
+    these inputs is shifted away, so every chunk's integer is the integer dot of the values rounded at two decimals
+    (numpy int64) and the output is the fp32 chain over those integers, replayed here in float64 with one rounding
+    per step: bit for bit."""
+    monkeypatch.setenv("BSI_FIXED_BITS_QUERIES", str(bq))
+    monkeypatch.setenv("BSI_FIXED_BITS_KEYS", str(bk))
+    ops._reset_flag_cache()
+    rng = np.random.default_rng(bq + bk + Q)
+    x = rng.standard_normal((Q, D)).astype(np.float32)
+    k = (rng.standard_normal((R, D)) * 0.05).astype(np.float32)
+    kcap, *_ = ops.build_bsi_keys_cuda(torch.from_numpy(k), 2, 0.5)
+    qcap = ops.build_bsi_queries_cuda_batch_packed(torch.from_numpy(x).cuda(), 2, 0.5)
+    assert qcap.Sa == bq and kcap.Sb == bk
+    out, *_ = ops.batch_dot_product_multiquery_cuda_batch_caps(qcap, kcap)
+    xi, ki = oracle.round_to_int64(x, 2), oracle.round_to_int64(k, 2)
+    assert np.abs(xi).max() < 2 ** 16 and np.abs(ki).max() < 2 ** 16
+    acc = np.zeros((Q, R), dtype=np.float32)
+    for c0 in range(0, D, 256):
+        I = xi[:, c0:c0 + 256] @ ki[:, c0:c0 + 256].T
+        assert np.abs(I).max() < 2 ** 24  # exact as float32
+        acc = (I.astype(np.float64) + acc.astype(np.float64)).astype(np.float32)  # fmaf(float(I), 1, acc)
+    want = acc * oracle.scale_inv(2, 2)
+    np.testing.assert_array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
 def test_reference_known_answers_gpu(ops, monkeypatch):
     kat = json.load(open(GOLDEN))
     for case in kat["vector_dot"] + kat["batch_dot"]:
