@@ -721,8 +721,9 @@ def test_dot_int8_image_short_and_odd_chunk_counts(hip, oracle, d, tile):
         hip.check(L.bsi_hip_dot(A.data_ptr(), a8.data_ptr(), scales.data_ptr(), chunks, 7, W, B.data_ptr(), 2, Bw.data_ptr(),
                                 6, R, Q, float(np.float32(1e-4)), R, out.data_ptr(), ints.data_ptr(), 2, None, 0, st()), "dot")
         outb = torch.full((Q, R), float("nan"), dtype=torch.float32, device="cuda")
+        bias_d = dev(bias)  # named, so that it lives until the kernel has run
         hip.check(L.bsi_hip_dot_bias(A.data_ptr(), a8.data_ptr(), scales.data_ptr(), chunks, 7, W, B.data_ptr(), 2,
-                                     Bw.data_ptr(), 6, R, Q, float(np.float32(1e-4)), R, dev(bias).data_ptr(),
+                                     Bw.data_ptr(), 6, R, Q, float(np.float32(1e-4)), R, bias_d.data_ptr(),
                                      outb.data_ptr(), 2, None, 0, st()), "dot_bias")
         torch.cuda.synchronize()
     finally:
@@ -1387,7 +1388,9 @@ def _digits_dev(hip, words: np.ndarray):
     rows, S, W = words.shape
     chunks = (W + 3) // 4
     out = torch.full(((S + 6) // 7, rows, chunks * 256), 77, dtype=torch.int8, device="cuda")
-    hip.check(hip.lib.bsi_hip_planes_to_int8_digits(dev(words).data_ptr(), rows, S, W, out.data_ptr(), st()), "digits")
+    words_d = dev(words)  # named, so that it lives until the kernel has run
+    hip.check(hip.lib.bsi_hip_planes_to_int8_digits(words_d.data_ptr(), rows, S, W, out.data_ptr(), st()), "digits")
+    torch.cuda.synchronize()
     return out
 
 
@@ -1452,12 +1455,14 @@ def test_dot_digits_fixed_images_indices_bias_and_stride(hip, oracle):
     a, b = oracle.build_decimal(x, 2), oracle.build_keys(k, 2, 6)
     want = oracle.dot_weighted(a["words"], a["slice_weights"], b["words"], b["slice_weights"], np.float32(1e-4))
     k8 = torch.empty((1, R, 4 * 256), dtype=torch.int8, device="cuda")
-    hip.check(hip.lib.bsi_hip_planes_to_int8(dev(b["words"]).data_ptr(), R, 6, W, k8.data_ptr(), st()), "image")
+    _src1 = dev(b["words"])  # named, so that it lives until the kernel has run
+    hip.check(hip.lib.bsi_hip_planes_to_int8(_src1.data_ptr(), R, 6, W, k8.data_ptr(), st()), "image")
     a_dig = _digits_dev(hip, a["words"])
     perm = np.random.default_rng(3).permutation(60)[:R]
     bias = torch.randn(R, device="cuda")
     k8t = torch.full((int(hip.lib.bsi_hip_int8_tiled_bytes(R, W)),), 77, dtype=torch.int8, device="cuda")
-    hip.check(hip.lib.bsi_hip_planes_to_int8_tiled(dev(b["words"]).data_ptr(), R, 6, W, k8t.data_ptr(), st()), "image")
+    _src2 = dev(b["words"])  # named, so that it lives until the kernel has run
+    hip.check(hip.lib.bsi_hip_planes_to_int8_tiled(_src2.data_ptr(), R, 6, W, k8t.data_ptr(), st()), "image")
     for route in (1, 2):
         hip.check(hip.lib.bsi_hip_set_option(hip.OPT_DIGITS_ROUTE, route), "opt")
         got = _run_digits(hip, a_dig, a["slice_weights"], a["S"], k8, 2, b["slice_weights"], 6, W, Q, R)
@@ -1475,7 +1480,8 @@ def test_dot_digits_fixed_images_indices_bias_and_stride(hip, oracle):
     kb = oracle.build_decimal(k, 2)
     want = oracle.dot_weighted(oracle.pack(ints, 7), aw, kb["words"], kb["slice_weights"], np.float32(1e-4))
     q8 = torch.empty((1, Q, 4 * 256), dtype=torch.int8, device="cuda")
-    hip.check(hip.lib.bsi_hip_planes_to_int8(dev(oracle.pack(ints, 7)).data_ptr(), Q, 7, W, q8.data_ptr(), st()), "image")
+    _src3 = dev(oracle.pack(ints, 7))  # named, so that it lives until the kernel has run
+    hip.check(hip.lib.bsi_hip_planes_to_int8(_src3.data_ptr(), Q, 7, W, q8.data_ptr(), st()), "image")
     got = _run_digits(hip, q8, aw, 7, _digits_dev(hip, kb["words"]), 1, kb["slice_weights"], kb["S"], W, Q, R)
     assert np.array_equal(got, want)
 
@@ -1711,10 +1717,11 @@ def test_linear_few_rows_other_decimal_places(hip, oracle, dec):
     qb, kb = oracle.build_queries(x, dec, 7), oracle.build_keys(k, dec, 6)
     _, want = oracle.dot_fixed(qb["words"], qb["scales"], kb["words"], kb["scales"], oracle.scale_inv(dec, dec), want_ints=False)
     Bt = torch.empty((4 * 4 * 6 * 64,), dtype=torch.int64, device="cuda")
-    hip.check(L.bsi_hip_tile_key_planes(dev(kb["words"]).data_ptr(), R, 6, 16, Bt.data_ptr(), st()), "tile")
+    planes_d, x_d = dev(kb["words"]), torch.from_numpy(x).cuda()  # named, so that they live until the kernels have run
+    hip.check(L.bsi_hip_tile_key_planes(planes_d.data_ptr(), R, 6, 16, Bt.data_ptr(), st()), "tile")
     Bw = dev(kb["slice_weights"])
     out = torch.empty((Q, R), dtype=torch.float32, device="cuda")
-    hip.check(L.bsi_hip_linear_few_rows(torch.from_numpy(x).cuda().data_ptr(), hip.DTYPE_F32, Q, d, dec, 7, Bt.data_ptr(),
+    hip.check(L.bsi_hip_linear_few_rows(x_d.data_ptr(), hip.DTYPE_F32, Q, d, dec, 7, Bt.data_ptr(),
                                         Bw.data_ptr(), 6, R, float(oracle.scale_inv(dec, dec)), R, None, out.data_ptr(),
                                         st()), "fused")
     torch.cuda.synchronize()
@@ -1734,7 +1741,8 @@ def test_linear_few_rows_long_rows_and_lds_limit(hip, oracle):
     _, want = oracle.dot_fixed(qb["words"], qb["scales"], kb["words"], kb["scales"], oracle.scale_inv(2, 2), want_ints=False)
     W = d // 64
     Bt = torch.empty((2 * (W // 4) * 6 * 64,), dtype=torch.int64, device="cuda")
-    hip.check(L.bsi_hip_tile_key_planes(dev(kb["words"]).data_ptr(), R, 6, W, Bt.data_ptr(), st()), "tile")
+    _src4 = dev(kb["words"])  # named, so that it lives until the kernel has run
+    hip.check(L.bsi_hip_tile_key_planes(_src4.data_ptr(), R, 6, W, Bt.data_ptr(), st()), "tile")
     Bw = dev(kb["slice_weights"])
     xd = torch.from_numpy(x).cuda()
     out = torch.empty((4, R), dtype=torch.float32, device="cuda")
@@ -1756,7 +1764,8 @@ def test_linear_few_rows_half_inputs_and_limits(hip, oracle, dtype):
     qb, kb = oracle.build_queries(x, 2, 7), oracle.build_keys(k, 2, 6)
     _, want = oracle.dot_fixed(qb["words"], qb["scales"], kb["words"], kb["scales"], oracle.scale_inv(2, 2), want_ints=False)
     Bt = torch.empty((3 * 4 * 6 * 64,), dtype=torch.int64, device="cuda")
-    hip.check(L.bsi_hip_tile_key_planes(dev(kb["words"]).data_ptr(), 40, 6, 16, Bt.data_ptr(), st()), "tile")
+    _src5 = dev(kb["words"])  # named, so that it lives until the kernel has run
+    hip.check(L.bsi_hip_tile_key_planes(_src5.data_ptr(), 40, 6, 16, Bt.data_ptr(), st()), "tile")
     Bw = dev(kb["slice_weights"])
     out = torch.empty((2, 40), dtype=torch.float32, device="cuda")
     xd = xh.cuda()
