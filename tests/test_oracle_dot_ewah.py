@@ -212,6 +212,61 @@ def test_ewah_round_trip(oracle, seed):
             assert lens[0] == 1 and lens[1] == 1
 
 
+def _drawn_planes(rng, S, W):
+    """Slices made of stretches of zeros, ones, random literals and one-bit literals of drawn lengths."""
+    words = np.zeros((S, W), dtype=np.uint64)
+    for s in range(S):
+        w = 0
+        while w < W:
+            n = min(int(rng.choice([1, 1, 2, 3, 7, 63, 64, 65, 130])), W - w)
+            kind = rng.integers(0, 4)
+            if kind == 1:
+                words[s, w:w + n] = ONES
+            elif kind == 2:
+                words[s, w:w + n] = rng.integers(1, 2 ** 63, size=n, dtype=np.uint64) * np.uint64(2)
+            elif kind == 3:
+                words[s, w:w + n] = np.uint64(1) << rng.integers(0, 64, size=n, dtype=np.uint64)
+            w += n
+    return words
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_ewah_stream_length_and_fields_in_closed_form(oracle, seed):
+    """What the greedy encoder must produce, stated without walking the slice: a marker for every maximal run of equal
+    clean words plus one if the slice starts with a literal, and every literal once -- so the stream length is a count
+    over the words; the markers' run lengths and literal counts add up to W; the runs name the clean words' kind and the
+    payload is the literal words in order.  (A dropped marker, a run split in two, a literal counted with the wrong
+    marker or a field one bit off fails one of these.)"""
+    rng = np.random.default_rng(100 + seed)
+    S, W = 9, int(rng.choice([1, 5, 64, 65, 200, 513]))
+    words = _drawn_planes(rng, S, W)
+    stream, off, lens = oracle.ewah_encode(words, np.ones(S, dtype=np.int32))
+    for s in range(S):
+        row = words[s]
+        clean = (row == 0) | (row == ONES)
+        prev_same = np.zeros(W, dtype=bool)
+        prev_same[1:] = clean[1:] & clean[:-1] & (row[1:] == row[:-1])
+        run_starts = int((clean & ~prev_same).sum())
+        want_len = int((~clean).sum()) + run_starts + (0 if clean[0] else 1)
+        assert lens[s] == want_len
+        st = stream[off[s]: off[s] + lens[s]]
+        i, covered, payload = 0, 0, []
+        while i < len(st):
+            m = int(st[i])
+            run_bit, run_len, lit = m & 1, (m >> 1) & 0xFFFFFFFF, m >> 33
+            if run_len:
+                assert (row[covered: covered + run_len] == (ONES if run_bit else 0)).all()
+            else:
+                assert run_bit == 0 and covered == 0  # only a slice that starts with a literal has a marker without a run
+            covered += run_len
+            payload.extend(st[i + 1: i + 1 + lit])
+            assert not clean[covered: covered + lit].any()
+            covered += lit
+            i += 1 + lit
+        assert covered == W and i == len(st)
+        np.testing.assert_array_equal(np.array(payload, dtype=np.uint64), row[~clean])
+
+
 def test_relu_queries_sign_plane_is_one_run(oracle):
     # ReLU'd activations: the sign plane is all zero -> a single run marker; dense planes stay verbatim
     rng = np.random.default_rng(9)
