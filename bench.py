@@ -153,7 +153,6 @@ def _decode_shapes(_lib, bsi_ops):
     import torch
 
     rows = []
-    st = torch.cuda.current_stream().cuda_stream
     for name, R5, D5 in (("attn 4096x4096", 4096, 4096), ("fc1 16384x4096", 16384, 4096), ("fc2 4096x16384", 4096, 16384)):
         plane_bytes = R5 * SB * (D5 // 64) * 8
         n_sets = max(2, -(-640 * 1024 * 1024 // plane_bytes))           # at least 640 MB of planes in rotation
@@ -235,7 +234,13 @@ def _opt_prefill():
     keep = ("model", "layers", "seq_len", "num_bsi_layers", "bsi_fwd_ms", "bsi_tokens_per_s", "bsi_graph_fwd_ms",
             "bsi_graph_tokens_per_s", "graph_replays_match_eager", "dot_ms_per_prefill", "dot_share_of_fwd",
             "query_build_kernel_ms_per_prefill", "key_build_s")
-    return {k: r[k] for k in keep if k in r}
+    res = {k: r[k] for k in keep if k in r}
+    # the same model with q_proj, k_proj and v_proj of every layer served by one dot (same bits, one launch for three)
+    f = benchmark_opt_prefill.run("opt-1.3b", seq_len=512, batch=1, iters=5, warmup=2, dense=False, graph=True,
+                                  fuse_qkv=True)
+    res["one_dot_for_q_k_v"] = {k: f[k] for k in ("bsi_fwd_ms", "bsi_tokens_per_s", "bsi_graph_fwd_ms",
+                                                   "bsi_graph_tokens_per_s", "graph_replays_match_eager") if k in f}
+    return res
 
 
 def main() -> int:
@@ -268,7 +273,7 @@ def main() -> int:
     X[:, cols] *= 20.0
     K = torch.randn(R, D) * 0.02
 
-    kcap, key_bytes, _, _, W = bsi_ops.build_bsi_keys_cuda(K, 2, 0.5)
+    kcap, _, _, _, W = bsi_ops.build_bsi_keys_cuda(K, 2, 0.5)
     qcap = bsi_ops.build_bsi_queries_cuda_batch_packed(X.cuda(), 2, 0.5)
     chunks = W // 4
     core = {"auto": _lib.CORE_AUTO, "mfma": _lib.CORE_MFMA, "valu": _lib.CORE_VALU}[args.core]

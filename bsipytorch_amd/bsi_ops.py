@@ -360,7 +360,6 @@ def _build_decimal(x2d: torch.Tensor, decimal_places: int):
     Reads one scalar back from the device to size the planes, as the reference does (``.item()``, :1092-1096)."""
     dev = x2d.device
     Q, d = x2d.shape
-    W = (d + 63) // 64 if d > 0 else 1
     st = _stream()
     ints = torch.empty((Q, d), dtype=torch.int64, device=dev)
     if Q > 0 and d > 0:
