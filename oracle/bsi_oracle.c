@@ -261,17 +261,19 @@ void bsi_oracle_dot_fixed(const uint64_t* A, const float* qscale, int64_t qscale
             for (int c = 0; c < chunks; ++c) {
                 const int w0 = c * BSI_CHUNK_WORDS;
                 const int w1 = (w0 + BSI_CHUNK_WORDS < W) ? w0 + BSI_CHUNK_WORDS : W;
-                int32_t I = 0;
+                /* summed modulo 2^64 (a term shifted by 64 or more is a multiple of 2^64): the chunk's integer dot
+                 * whenever that fits 64 bits, and the reference's int32 for its 7 x 6 bits (|I| <= 2^19) */
+                uint64_t I = 0;
                 for (int i = 0; i < Sa; ++i)
                     for (int j = 0; j < Sb; ++j) {
-                        int32_t cnt = 0;
+                        uint64_t cnt = 0;
                         for (int w = w0; w < w1; ++w)
-                            cnt += __builtin_popcountll(Aq[(size_t)i * W + w] & Br[(size_t)j * W + w]);
-                        const int32_t v = cnt << (i + j);
+                            cnt += (uint64_t)__builtin_popcountll(Aq[(size_t)i * W + w] & Br[(size_t)j * W + w]);
+                        const uint64_t v = (i + j < 64) ? cnt << (i + j) : 0;
                         if ((i == Sa - 1) != (j == Sb - 1)) I -= v; else I += v;
                     }
-                if (chunk_ints) chunk_ints[((size_t)q * R + r) * chunks + c] = I;
-                acc = fmaf((float)I, qscale[q * qscale_stride + c] * bscale[r], acc);
+                if (chunk_ints) chunk_ints[((size_t)q * R + r) * chunks + c] = (int32_t)(uint32_t)I;
+                acc = fmaf((float)(int64_t)I, qscale[q * qscale_stride + c] * bscale[r], acc);
             }
             if (out) out[(size_t)q * R_total + r] = acc * scale_inv;
         }

@@ -40,9 +40,10 @@ def lib():
     global _lib
     if _lib is not None:
         return _lib
-    if not os.path.exists(_SO):
+    override = os.environ.get("BSI_ORACLE_LIBRARY")  # e.g. the sanitized build, `make -C oracle libbsi_oracle_ubsan.so`
+    if override is None and not os.path.exists(_SO):
         build()
-    L = ctypes.CDLL(_SO)
+    L = ctypes.CDLL(override if override is not None else _SO)
     L.bsi_oracle_round_half_away.restype = ctypes.c_int64
     L.bsi_oracle_round_half_away.argtypes = [ctypes.c_double]
     L.bsi_oracle_round_to_int64.restype = None

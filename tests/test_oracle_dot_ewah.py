@@ -96,6 +96,34 @@ def test_dot_fp32_chain_exact_replay(oracle):
     assert sinv == np.float32(1e-4)
 
 
+@pytest.mark.parametrize("bits_q,bits_k", [(33, 20), (16, 16), (40, 23), (2, 63), (63, 63)])
+def test_dot_wide_operands_against_python_integers(oracle, bits_q, bits_k):
+    """Widths up to the 63 bits the reference's flags allow: the chunk integer is the exact dot while it fits 64 bits
+    (Python integers, no popcounts), its low 32 bits are what the int32 output holds, and float(I) enters the chain
+    with one rounding.  With 63 x 63 bits the dot does not fit: then the oracle's integer is the dot modulo 2^64."""
+    rng = np.random.default_rng(bits_q * 64 + bits_k)
+    Q, R, d = 3, 4, 512
+    a = rng.integers(-(1 << (bits_q - 1)), 1 << (bits_q - 1), size=(Q, d), dtype=np.int64)
+    b = rng.integers(-(1 << (bits_k - 1)), 1 << (bits_k - 1), size=(R, d), dtype=np.int64)
+    a[0, :256] = -(1 << (bits_q - 1))  # a chunk of the most negative value on both sides
+    b[0, :256] = -(1 << (bits_k - 1))
+    A, B = oracle.pack(a, bits_q), oracle.pack(b, bits_k)
+    ints, out = oracle.dot_fixed(A, np.ones((Q, 2), np.float32), B, np.ones(R, np.float32), 1.0)
+    for q in range(Q):
+        for r in range(R):
+            acc = 0
+            for c in range(2):
+                exact = sum(int(x) * int(y) for x, y in zip(a[q, c * 256:(c + 1) * 256], b[r, c * 256:(c + 1) * 256]))
+                if bits_q + bits_k + 8 <= 63:
+                    assert abs(exact) < 1 << 63
+                wrapped = (exact + (1 << 63)) % (1 << 64) - (1 << 63)  # the signed 64-bit reading of exact mod 2^64
+                low = wrapped & 0xFFFFFFFF
+                assert int(ints[q, r, c]) == (low - (1 << 32) if low >> 31 else low), (q, r, c)
+                # fmaf(float(I), 1, acc): float(I) rounds once, the exact sum of the two fp32 values once more
+                acc = _rn_f32_int(acc + _rn_f32_int(wrapped))
+            assert out[q, r] == np.float32(acc), (q, r)
+
+
 def test_dot_row_scale_and_partial_chunk(oracle):
     # W64 = 5: no chunk scales (one scale per row), last chunk holds a single word
     rng = np.random.default_rng(5)
