@@ -88,16 +88,17 @@ static int time_launch(hipStream_t st, int reps, float* ms_best, F&& launch) {
     float best = 1e30f;
     hipError_t err = hipSuccess;
     for (int r = 0; r < reps && err == hipSuccess; ++r) {
-        hipEventRecord(e0, st);
+        err = hipEventRecord(e0, st);
+        if (err != hipSuccess) break;
         launch();
-        hipEventRecord(e1, st);
-        err = hipEventSynchronize(e1);
+        err = hipEventRecord(e1, st);
+        if (err == hipSuccess) err = hipEventSynchronize(e1);
         float ms = 0.0f;
         if (err == hipSuccess) err = hipEventElapsedTime(&ms, e0, e1);
         if (ms < best) best = ms;
     }
-    hipEventDestroy(e0);
-    hipEventDestroy(e1);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
     if (err != hipSuccess) return fail(BSI_ERR_HIP, "probe timing failed: %s", hipGetErrorString(err));
     *ms_best = best;
     return BSI_OK;
