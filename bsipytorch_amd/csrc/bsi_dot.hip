@@ -2851,6 +2851,9 @@ static int dot_launch(const uint64_t* A, const int8_t* A_ints8, const float* A_c
     BSI_REQUIRE(W64 >= 1, "W64 must be >= 1");
     BSI_REQUIRE(Sa >= 1 && Sa <= 63 && Sb >= 1 && Sb <= 63, "Sa and Sb must be in [1, 63]");
     BSI_REQUIRE(R_total >= R, "R_total must be >= R");
+    // per-row operands (slice weights, bias, chunk scales) are fetched with 32-bit byte offsets
+    BSI_REQUIRE(R <= (1 << 25) && Q <= (1 << 25), "at most 2^25 key rows and query rows per call (got R = %lld, Q = %lld)",
+                static_cast<long long>(R), static_cast<long long>(Q));
     BSI_REQUIRE(b_layout == BSI_LAYOUT_CANONICAL || b_layout == BSI_LAYOUT_TILED16 || b_layout == BSI_LAYOUT_INT8 ||
                     b_layout == BSI_LAYOUT_INT8_TILED,
                 "unknown key layout %d", b_layout);
@@ -2863,11 +2866,16 @@ static int dot_launch(const uint64_t* A, const int8_t* A_ints8, const float* A_c
     BSI_REQUIRE(A || A_ints8, "neither query planes nor int8 queries given");
     hipStream_t st = as_stream(stream);
 
+    // The matrix-core kernels address a tile's operand rows with 32-bit buffer offsets inside a descriptor of at most
+    // 2 GiB: 128 rows of chunks * 256 bytes must stay below that.
+    constexpr int kMfmaMaxChunks = 32768;
     const bool mfma_ok = (Sa >= 2 && Sa <= 8 && Sb >= 2 && Sb <= 8);
-    if (core == BSI_CORE_AUTO) core = mfma_ok ? BSI_CORE_MFMA : BSI_CORE_VALU;
+    if (core == BSI_CORE_AUTO) core = (mfma_ok && chunks <= kMfmaMaxChunks) ? BSI_CORE_MFMA : BSI_CORE_VALU;
 
     if (core == BSI_CORE_MFMA) {
         if (!mfma_ok) return fail(BSI_ERR_UNSUPPORTED, "MFMA core needs Sa, Sb in [2, 8] (got %d, %d)", Sa, Sb);
+        if (chunks > kMfmaMaxChunks)
+            return fail(BSI_ERR_UNSUPPORTED, "MFMA core takes rows of up to %d chunks of 256 elements (got %d)", kMfmaMaxChunks, chunks);
         const int8_t* A8 = A_ints8;
         BSI_REQUIRE((reinterpret_cast<uintptr_t>(A8) & 15) == 0 && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0,
                     "int8 queries / workspace must be 16-byte aligned");
@@ -2928,6 +2936,7 @@ static int dot_launch(const uint64_t* A, const int8_t* A_ints8, const float* A_c
         return BSI_OK;
     }
     const int64_t total = Q * R;
+    BSI_REQUIRE((total + 255) / 256 <= 0x7fffffffLL, "too many outputs for one launch of the any-width kernel");
     hipLaunchKernelGGL(dot_valu_generic_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, st,
                        reinterpret_cast<const unsigned long long*>(A), A_chunk_scales, A_scale_stride, Sa,
                        reinterpret_cast<const unsigned long long*>(B), Bw, Sb, W64, chunks, R, Q, scale_inv, R_total,

@@ -207,7 +207,9 @@ size_t bsi_hip_dot_workspace_bytes(int64_t Q, int W64, int core);
  *   B              key words in `b_layout`; Bw float [R, Sb] slice weights (only Bw[r*Sb] is read, and its magnitude used: the row scale 2^shift_r)
  *   out            float [Q, R_total] (row stride R_total >= R); every element [q, r<R] is written
  *   chunk_ints     optional int32 [Q, R, chunks]: the integer accumulators I (parity checks)
- * Sa, Sb in [2, 8] for the MFMA core and [1, 63] for the VALU core (canonical or tiled16 key planes).
+ * Sa, Sb in [2, 8] for the MFMA core and [1, 63] for the VALU core (canonical or tiled16 key planes); the MFMA core
+ * takes rows of up to 32768 chunks (2^23 elements: its 32-bit operand offsets), BSI_CORE_AUTO falls back to the VALU
+ * core beyond that.
  */
 int bsi_hip_dot(const uint64_t* A, const int8_t* A_ints8, const float* A_chunk_scales, int A_scale_stride, int Sa,
                 int W64, const uint64_t* B, int b_layout, const float* Bw, int Sb, int64_t R, int64_t Q,
