@@ -182,7 +182,7 @@ static inline unsigned integer_decimal_scale(double dec_scale) {
 }
 
 // Position of element e (0..255) of a chunk inside the chunk's 256 int8 bytes in the MFMA core's
-// order: element 32w + 8m + t sits at byte 32w + 4t + m (see planes_to_int8 in bsi_dot.hip).
+// order: element 32w + 8m + t sits at byte 32w + 4t + m (see planes_to_int8_kernel in bsi_dot_layouts.hip).
 __device__ __forceinline__ int mfma_byte_pos(int e) {
     const int w = e >> 5, r = e & 31;
     const int m = r >> 3, t = r & 7;
