@@ -5,6 +5,7 @@
 
 namespace bsi {
 
+// process-wide options set through bsi_hip_set_option (meanings beside their declarations in bsi_dot_internal.h)
 std::atomic<int> g_i8_tile{0};
 std::atomic<int> g_digits_route{0};
 
