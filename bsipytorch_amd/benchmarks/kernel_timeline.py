@@ -29,11 +29,11 @@ STAMPS = ("mfma wave entered", "first stage in LDS", "chunk loop done", "outputs
 ORDER = (4, 0, 6, 7, 1, 5, 2, 3)  # the order things happen in
 
 
-def timeline(Q: int, R: int, D: int, iters: int = 50) -> dict:
+def timeline(Q: int, R: int, D: int, iters: int = 50, warmup: int = 10) -> dict:
     wgs = 8192
     buf = (ctypes.c_ulonglong * (wgs * 8))()
     _lib.check(_lib.lib.bsi_hip_timeline_read(buf, wgs), "bsi_hip_timeline_read")  # clears what earlier launches left
-    res = micro.run(Q, R, D, 2, 0.5, 10, iters, 123, "mfma", outliers=(D == 2048))
+    res = micro.run(Q, R, D, 2, 0.5, warmup, iters, 123, "mfma", outliers=(D == 2048))
     _lib.check(_lib.lib.bsi_hip_timeline_read(buf, wgs), "bsi_hip_timeline_read")
     t = np.frombuffer(buf, dtype=np.uint64).reshape(wgs, 8).astype(np.int64)
     live = t[t[:, 0] > 0]  # the workgroups of this shape's grid
@@ -64,10 +64,13 @@ def main() -> None:
     p.add_argument("--shapes", nargs="*", default=["512x8192x2048", "512x8192x8192", "512x2048x8192", "512x2048x2048"],
                    help="QxRxD")
     p.add_argument("--iters", type=int, default=50)
+    p.add_argument("--warmup", type=int, default=10,
+                   help="untimed launches before the timed ones; several thousand bring the shader clock to the state "
+                        "it holds under sustained load (about 35 ms of work from an idle GPU)")
     args = p.parse_args()
     for sh in args.shapes:
         Q, R, D = (int(v) for v in sh.lower().split("x"))
-        print(json.dumps(timeline(Q, R, D, args.iters)), flush=True)
+        print(json.dumps(timeline(Q, R, D, args.iters, args.warmup)), flush=True)
 
 
 if __name__ == "__main__":
