@@ -285,8 +285,14 @@ CUDA_BUILDER_VERSION = cuda_builder_version()
 _slice_weight_cache: dict = {}
 
 
+_gpu_present: Optional[bool] = None  # torch.cuda.is_available() costs 2 us a call and cannot change within a process
+
+
 def _capturing() -> bool:
-    return torch.cuda.is_available() and torch.cuda.is_current_stream_capturing()
+    global _gpu_present
+    if _gpu_present is None:
+        _gpu_present = bool(torch.cuda.is_available())
+    return _gpu_present and torch.cuda.is_current_stream_capturing()
 
 
 def _slice_weights(S: int, offset: int, twos: bool, device) -> torch.Tensor:
