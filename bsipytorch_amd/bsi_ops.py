@@ -1124,6 +1124,7 @@ def _linear_workspace(device, need: int, capturing: bool) -> dict:
 
 
 _reserved_linear_shapes: set = set()
+_linear_ws_need: dict = {}
 
 
 def reserve_linear_workspace(x2d: torch.Tensor) -> None:
@@ -1156,7 +1157,9 @@ def linear_cuda(x2d: torch.Tensor, keyset_cuda_cap, decimal_places: int, bias=No
     Q, d, R = int(x2d.shape[0]), int(x2d.shape[1]), keys.num_keys
     _check_bias(bias, R, x2d.device)
     bits = f["bits_q"]
-    need = int(lib.bsi_hip_linear_workspace_bytes(Q, d, bits))
+    need = _linear_ws_need.get((Q, d, bits))
+    if need is None:  # a pure function of the shape: asked once per shape, not once per forward
+        need = _linear_ws_need[(Q, d, bits)] = int(lib.bsi_hip_linear_workspace_bytes(Q, d, bits))
     capturing = _capturing()
     ws = _linear_workspace(x2d.device, need, capturing)
     slot = ws["capture" if capturing else "eager"]

@@ -570,6 +570,51 @@ def link_bsi_layers(model: nn.Module) -> int:
     return len(layers) if on else 0
 
 
+class GraphedForward:
+    """``model(*inputs)`` recorded once into a HIP graph and replayed: the whole forward becomes one submission with no
+    host work per layer (an eager forward of many small BSI layers is bound by that work).  Not in the reference.
+
+    ``example_inputs`` fix the shapes and dtypes; a call copies its inputs into the recorded input tensors, replays the
+    graph and returns the recorded output object (whatever the model returns), whose tensors are overwritten by the
+    next call.  Eager forwards of the same model may run in between.  The model must not change between calls in ways
+    a recording cannot see (weights rebuilt, layers swapped, environment flags): record again then."""
+
+    def __init__(self, model: nn.Module, *example_inputs: torch.Tensor, warmup: int = 2):
+        if not torch.cuda.is_available():
+            raise RuntimeError("GraphedForward needs the GPU")
+        if not example_inputs or not all(isinstance(t, torch.Tensor) and t.is_cuda for t in example_inputs):
+            raise ValueError("GraphedForward takes device tensors as example inputs")
+        self.model = model
+        self.static_inputs = [t.clone() for t in example_inputs]
+        with torch.no_grad():
+            # warm-up on a side stream, as captures need: allocates every workspace and key layout the forward uses
+            forget_shared_builds()
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                for _ in range(max(1, int(warmup))):
+                    model(*self.static_inputs)
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            forget_shared_builds()
+            self.graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(self.graph):
+                self.static_output = model(*self.static_inputs)
+            forget_shared_builds()
+
+    def __call__(self, *inputs: torch.Tensor):
+        if len(inputs) != len(self.static_inputs):
+            raise ValueError(f"recorded with {len(self.static_inputs)} inputs, called with {len(inputs)}")
+        for static, t in zip(self.static_inputs, inputs):
+            if t.shape != static.shape or t.dtype != static.dtype:
+                raise ValueError(f"recorded for inputs of shape {tuple(static.shape)} and dtype {static.dtype}, "
+                                 f"called with {tuple(t.shape)} {t.dtype}")
+            if t.data_ptr() != static.data_ptr():
+                static.copy_(t)
+        self.graph.replay()
+        return self.static_output
+
+
 def save_bsi_model(model: nn.Module, out_dir: str) -> List[Dict[str, Any]]:
     """Write every BSI layer's keyset (and bias) under ``out_dir`` with a ``manifest.json`` holding the fields the
     reference's save_bsi_model records (verify_accuracy_bsi.py:370-386: name, in, out, decimalPlaces,

@@ -186,3 +186,28 @@ def test_layer_with_its_bias_on_the_host(ops, rows, fuse):
     with pytest.raises(RuntimeError, match="bias must be"):
         ops.linear_cuda(x, keys, 2, bias=torch.zeros(R + 1, device="cuda"))
     forget_shared_builds()
+
+
+@pytest.mark.parametrize("rows", [2, 96])
+def test_graphed_forward_replays_match_eager(ops, rows):
+    """linear.GraphedForward: a small model of BSI layers recorded once; every replay, on fresh inputs and with eager
+    forwards of the same model in between, gives the eager bits; a call with another shape is refused."""
+    from bsipytorch_amd import linear
+
+    torch.manual_seed(rows)
+    model = torch.nn.Sequential(torch.nn.Linear(512, 1024), torch.nn.ReLU(), torch.nn.Linear(1024, 256)).cuda()
+    linear.quantize_model_bsi(model, decimalPlaces=2, compress_threshold=0.5, verbose=False)
+    xs = [torch.randn(rows, 512, device="cuda") * (i + 1) for i in range(4)]
+    with torch.no_grad():
+        want = [model(x).clone() for x in xs]
+        graphed = linear.GraphedForward(model, xs[0])
+        for rep in range(2):
+            for x, w in zip(xs, want):
+                got = graphed(x)
+                torch.cuda.synchronize()
+                assert torch.equal(got, w)
+                assert torch.equal(model(xs[(rep + 1) % 4]), want[(rep + 1) % 4])  # eager work between replays
+        with pytest.raises(ValueError):
+            graphed(torch.randn(rows + 1, 512, device="cuda"))
+        with pytest.raises(ValueError):
+            graphed(xs[0], xs[1])
