@@ -282,3 +282,15 @@ def test_reference_launcher_library_exports_the_reference_symbols():
     raw.bsi_launchers_last_error.restype = ctypes.c_char_p
     raw.bsi_launchers_clear_status()
     assert raw.bsi_launchers_last_status() == 0 and raw.bsi_launchers_last_error() == b""
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; asked for more it exits with a message instead of a figure (no GPU needed to say so)."""
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    run = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                         timeout=120)
+    assert run.returncode == 2
+    assert "one GPU" in run.stderr and not run.stdout.strip()
