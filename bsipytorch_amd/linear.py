@@ -584,6 +584,8 @@ class GraphedForward:
             raise RuntimeError("GraphedForward needs the GPU")
         if not example_inputs or not all(isinstance(t, torch.Tensor) and t.is_cuda for t in example_inputs):
             raise ValueError("GraphedForward takes device tensors as example inputs")
+        if bsi_ops._flags()["profile"]:
+            raise RuntimeError("BSI_PROFILE=1 times every dot with events and synchronises: that cannot be recorded into a graph")
         self.model = model
         self.static_inputs = [t.clone() for t in example_inputs]
         with torch.no_grad():
