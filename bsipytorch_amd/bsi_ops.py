@@ -1088,7 +1088,8 @@ def linear_few_rows_cuda(x2d: torch.Tensor, keyset_cuda_cap, decimal_places: int
 
 
 _last_linear_rebuilt = [False]  # whether the last linear_cuda call ran the query build (layer counters read it)
-_linear_ws: dict = {}  # device index -> {"bytes", "eager_buf", "capture_buf", "captured", "eager": [key, input], "capture": [...]}
+# device index -> {"bytes", "capture_buf", "captured", "capture": [key, input], "eager": {stream: (buffer, [key, input])}}
+_linear_ws: dict = {}
 
 
 def can_linear_one_call(x2d: torch.Tensor, keys: "PrebuiltBSIKeysCUDA") -> bool:
@@ -1104,10 +1105,12 @@ def can_linear_one_call(x2d: torch.Tensor, keys: "PrebuiltBSIKeysCUDA") -> bool:
 
 
 def _linear_workspace(device, need: int, capturing: bool) -> dict:
-    """linear_cuda's workspace record of ``device``: one buffer for eager calls and one for launches recorded into a
-    graph, both (re)allocated outside captures when they are missing or smaller than ``need`` bytes.  A recorded
+    """linear_cuda's workspace record of ``device``: one buffer per stream for eager calls (forwards that run on
+    different streams at the same time must not build into each other's operands) and one for launches recorded
+    into a graph, (re)allocated outside captures when they are missing or smaller than ``need`` bytes.  A recorded
     launch holds the capture buffer's address, so once a capture has used it, it is kept alive for good: a larger
-    need adds a new buffer for later captures and retires the old one instead of freeing it."""
+    need adds a new buffer for later captures and retires the old one instead of freeing it.  (Graphs replayed at the
+    same time on different streams still share that one buffer: replay them on one stream.)"""
     ws = _linear_ws.get(device.index)
     if ws is None or ws["bytes"] < need:
         _check(not capturing, "linear_cuda: the workspace must exist before a graph is captured (run the forward once)")
@@ -1115,9 +1118,8 @@ def _linear_workspace(device, need: int, capturing: bool) -> dict:
         if ws is not None and ws["captured"]:
             _retired_workspaces.append(ws["capture_buf"])
         ws = _linear_ws[device.index] = {"bytes": size, "captured": False,
-                                         "eager_buf": torch.empty((size,), dtype=torch.uint8, device=device),
                                          "capture_buf": torch.empty((size,), dtype=torch.uint8, device=device),
-                                         "eager": [None, None], "capture": [None, None]}
+                                         "capture": [None, None], "eager": {}}
     if capturing:
         ws["captured"] = True
     return ws
@@ -1162,11 +1164,18 @@ def linear_cuda(x2d: torch.Tensor, keyset_cuda_cap, decimal_places: int, bias=No
         need = _linear_ws_need[(Q, d, bits)] = int(lib.bsi_hip_linear_workspace_bytes(Q, d, bits))
     capturing = _capturing()
     ws = _linear_workspace(x2d.device, need, capturing)
-    slot = ws["capture" if capturing else "eager"]
+    st = _stream()
+    if capturing:
+        buf, slot = ws["capture_buf"], ws["capture"]
+    else:
+        mine = ws["eager"].get(st)
+        if mine is None:  # first eager call on this stream (allocated under it, so freed in its order too)
+            mine = ws["eager"][st] = (torch.empty((ws["bytes"],), dtype=torch.uint8, device=x2d.device), [None, None])
+        buf, slot = mine
     key = tensor_build_key(x2d, int(decimal_places))
     rebuild = 0 if (key is not None and slot[0] == key) else 1
     slot[0], slot[1] = key, x2d  # holds the input, so that its address is not reused while the build stands for it
-    wsptr = ws["capture_buf" if capturing else "eager_buf"].data_ptr()
+    wsptr = buf.data_ptr()
     out = torch.empty((Q, R), dtype=torch.float32, device=x2d.device)
     core = f["core"]
     kptr, klayout = key_operand(keys, Q, bits, core)
@@ -1175,7 +1184,7 @@ def linear_cuda(x2d: torch.Tensor, keyset_cuda_cap, decimal_places: int, bias=No
     check(lib.bsi_hip_linear(x2d.data_ptr(), _dtype_code(x2d), Q, d, int(decimal_places), bits, rebuild, wsptr, ws["bytes"],
                              kptr, klayout, keys.slice_weights.data_ptr(), keys.Sb, R,
                              _scale_inv(int(decimal_places), keys.decimals), R, _ptr(bias), out.data_ptr(), core, wptr,
-                             wbytes, _stream()), "bsi_hip_linear")
+                             wbytes, st), "bsi_hip_linear")
     _last_linear_rebuilt[0] = bool(rebuild)
     return out
 
@@ -1183,7 +1192,9 @@ def linear_cuda(x2d: torch.Tensor, keyset_cuda_cap, decimal_places: int, bias=No
 def linear_cuda_forget() -> None:
     """Drop what linear_cuda remembers of its last build (and the input tensor it holds)."""
     for ws in _linear_ws.values():
-        ws["eager"], ws["capture"] = [None, None], [None, None]
+        ws["capture"] = [None, None]
+        for _, slot in ws["eager"].values():
+            slot[0], slot[1] = None, None
 
 
 def _dot_result(out, ns, Q, R):

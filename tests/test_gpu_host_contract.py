@@ -211,3 +211,36 @@ def test_graphed_forward_replays_match_eager(ops, rows):
             graphed(torch.randn(rows + 1, 512, device="cuda"))
         with pytest.raises(ValueError):
             graphed(xs[0], xs[1])
+
+
+def test_eager_forwards_on_two_streams_build_into_their_own_workspaces(ops):
+    """Two streams run forwards of two layers at the same time: each stream's query build goes into a workspace of its
+    own (one shared buffer would let one stream's build overwrite the operands the other stream's dot is about to
+    read), and every output has the bits of the same forward run alone."""
+    from bsipytorch_amd import linear
+
+    torch.manual_seed(12)
+    layers = [torch.nn.Linear(1024, 768).cuda(), torch.nn.Linear(1024, 512).cuda()]
+    model = torch.nn.ModuleList(layers)
+    linear.quantize_model_bsi(model, decimalPlaces=2, compress_threshold=0.5, verbose=False)
+    ops._linear_ws.clear()
+    xs = [torch.randn(256, 1024, device="cuda") * (i + 1) for i in range(6)]
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    with torch.no_grad():
+        want = [[model[j](x).clone() for x in xs] for j in range(2)]
+        torch.cuda.synchronize()
+        got = [[None] * len(xs) for _ in range(2)]
+        for rep in range(3):
+            for i, x in enumerate(xs):
+                for j, s in enumerate(streams):
+                    s.wait_stream(torch.cuda.current_stream())
+                    with torch.cuda.stream(s):
+                        got[j][i] = model[j](x)
+            torch.cuda.synchronize()
+            for j in range(2):
+                for i in range(len(xs)):
+                    assert torch.equal(got[j][i], want[j][i]), (rep, j, i)
+    eager = ops._linear_ws[xs[0].device.index]["eager"]
+    handles = {s.cuda_stream for s in streams}
+    assert handles <= set(eager), (handles, set(eager))
+    assert len({eager[h][0].data_ptr() for h in handles}) == 2
