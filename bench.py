@@ -388,7 +388,8 @@ def main() -> int:
                       if used_core == "mfma" else "u32 and/popcount -> int32 per chunk, fp32 fmaf chunk-scale epilogue",
         "data": "synthetic",
         "config": {"workload": "FC1-like fixed76 chunk-scale dot Q512 R8192 D2048, 0.1% outlier columns x20, dec=2",
-                   "core": used_core, "key_layout": {0: "canonical planes", 1: "tiled16 planes", 2: "cached int8 image of the planes"}[klayout],
+                   "core": used_core, "key_layout": {0: "canonical planes", 1: "tiled16 planes", 2: "cached int8 image of the planes",
+                                  3: "cached int8 image of the planes in 64-row tiles"}[klayout],
                    "algorithmic_bytes": alg_bytes, "bit_ops": bit_ops},
         "roofline": roof,
     }

@@ -55,7 +55,7 @@ def run(Q, R, D, decimal_places=2, compress_threshold=0.5, warmup=10, iters=50, 
     t = float(us.value) * 1e-6
     bit_ops = 2.0 * qcap.Sa * kcap.Sb * Q * R * D
     alg_bytes = Q * qcap.Sa * W * 8 + Q * chunks * 4 + R * kcap.Sb * W * 8 + R * 4 + Q * R * 4
-    return {"Q": Q, "R": R, "D": D, "core": core, "layout": {0: "canonical", 1: "tiled16", 2: "int8 image"}[klayout],
+    return {"Q": Q, "R": R, "D": D, "core": core, "layout": {0: "canonical", 1: "tiled16", 2: "int8 image", 3: "int8 image in 64-row tiles"}[klayout],
             "avg_dot_us": t * 1e6, "dot_q_us": t * 1e6 / Q, "dot_s_ns": t * 1e9 / (Q * R),
             "effective_bitop_TOPS": bit_ops / t / 1e12, "int8_TOPS": 2.0 * Q * R * D / t / 1e12,
             "algorithmic_GBps": alg_bytes / t / 1e9, "key_plane_GBps": key_bytes / t / 1e9, "iters": iters}
