@@ -40,6 +40,7 @@ def run(Q, R, D, decimal_places=2, compress_threshold=0.5, warmup=10, iters=50, 
     else:
         scales, stride = qcap.row_scales, 1
     code = {"auto": _lib.CORE_AUTO, "mfma": _lib.CORE_MFMA, "valu": _lib.CORE_VALU}[core]
+    use_ints8 = use_ints8 and qcap.ints8 is not None  # operands wider than 8 bits have no int8 image
     out = torch.empty((Q, R), dtype=torch.float32, device="cuda")
     ws_bytes = 0 if use_ints8 else int(_lib.lib.bsi_hip_dot_workspace_bytes(Q, W, code))
     ws = torch.empty((max(ws_bytes, 16),), dtype=torch.uint8, device="cuda")

@@ -37,7 +37,8 @@ def run(model="opt-6.7b", Qs=(1, 16, 128, 512), core="auto", iters=50, warmup=10
             r["model"] = model
             r["key_plane_frac_of_hbm_peak"] = r["key_plane_GBps"] / HBM_PEAK_GBS
             r["algorithmic_frac_of_hbm_peak"] = r["algorithmic_GBps"] / HBM_PEAK_GBS
-            r["int8_frac_of_mfma_peak"] = r["int8_TOPS"] / MFMA_I8_PEAK_TOPS
+            if "int8_TOPS" in r:  # absent in decimal mode, whose operands are not int8
+                r["int8_frac_of_mfma_peak"] = r["int8_TOPS"] / MFMA_I8_PEAK_TOPS
             rows.append(r)
     return rows
 

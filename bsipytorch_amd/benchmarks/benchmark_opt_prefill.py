@@ -159,7 +159,9 @@ def run(model_name="opt-1.3b", seq_len=512, batch=1, iters=5, warmup=2, decimal_
 
     # pass 1b: the same forward captured once into a HIP graph and replayed (no host work per layer).
     # Replays are checked against the eager logits, with eager work in between, as graph replays must be.
-    if graph:
+    if graph and bsi_ops._flags()["bits_q"] == 0:
+        res["bsi_graph_fwd_ms"] = None  # decimal-mode builds read a scalar back from the device: not recordable
+    elif graph:
         with torch.no_grad():
             eager = model(input_ids).clone()
             graphed = linear.GraphedForward(model, input_ids)

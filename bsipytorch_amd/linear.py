@@ -586,6 +586,9 @@ class GraphedForward:
             raise ValueError("GraphedForward takes device tensors as example inputs")
         if bsi_ops._flags()["profile"]:
             raise RuntimeError("BSI_PROFILE=1 times every dot with events and synchronises: that cannot be recorded into a graph")
+        if bsi_ops._flags()["bits_q"] == 0:
+            raise RuntimeError("decimal-mode query builds (BSI_FIXED_BITS*=0) read their slice count back from the device, "
+                               "as the reference's do: that cannot be recorded into a graph")
         self.model = model
         self.static_inputs = [t.clone() for t in example_inputs]
         with torch.no_grad():

@@ -244,3 +244,22 @@ def test_eager_forwards_on_two_streams_build_into_their_own_workspaces(ops):
     handles = {s.cuda_stream for s in streams}
     assert handles <= set(eager), (handles, set(eager))
     assert len({eager[h][0].data_ptr() for h in handles}) == 2
+
+
+def test_graphed_forward_refuses_what_cannot_be_recorded(ops, monkeypatch):
+    """Decimal-mode builds read a scalar back from the device and BSI_PROFILE=1 synchronises: GraphedForward says so
+    up front instead of failing inside the capture."""
+    from bsipytorch_amd import linear
+
+    model = torch.nn.Sequential(torch.nn.Linear(256, 64)).cuda()
+    linear.quantize_model_bsi(model, decimalPlaces=2, compress_threshold=0.5, verbose=False)
+    x = torch.randn(8, 256, device="cuda")
+    for name, value, text in (("BSI_FIXED_BITS", "0", "decimal-mode"), ("BSI_PROFILE", "1", "BSI_PROFILE")):
+        monkeypatch.setenv(name, value)
+        ops._reset_flag_cache()
+        with pytest.raises(RuntimeError, match=text):
+            linear.GraphedForward(model, x)
+        monkeypatch.delenv(name)
+        ops._reset_flag_cache()
+    with torch.no_grad():
+        assert torch.equal(linear.GraphedForward(model, x)(x), model(x))
