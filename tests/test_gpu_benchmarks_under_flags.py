@@ -1,0 +1,58 @@
+"""The benchmark harnesses under the environment flags a user may set: every combination must run to its report (a
+missing name for a layout, an operand form a flag switches off, a figure that only exists for int8 operands)."""
+import os
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+FLAGS = [
+    {},
+    {"BSI_KEY_IMAGE_TILED": "1"},
+    {"BSI_KEY_INT8_IMAGE": "0"},
+    {"BSI_KEY_LAYOUT": "canonical"},
+    {"BSI_KEY_LAYOUT": "canonical", "BSI_KEY_INT8_IMAGE": "0"},
+    {"BSI_DOT_CORE": "valu"},
+    {"BSI_FIXED_BITS": "0"},
+    {"BSI_FIXED_BITS": "0", "BSI_DECIMAL_MFMA": "0"},
+    {"BSI_FIXED_CHUNK_SCALE": "0"},
+    {"BSI_FIXED_CLIP_K": "3"},
+    {"BSI_FIXED_BITS_QUERIES": "8", "BSI_FIXED_BITS_KEYS": "5"},
+    {"BSI_FIXED_BITS_QUERIES": "12", "BSI_FIXED_BITS_KEYS": "10"},
+    {"BSI_PROFILE": "1"},
+]
+
+
+@pytest.fixture()
+def flags(monkeypatch, request):
+    from bsipytorch_amd import bsi_ops
+
+    for k in list(os.environ):
+        if k.startswith("BSI_"):
+            monkeypatch.delenv(k)
+    for k, v in request.param.items():
+        monkeypatch.setenv(k, v)
+    bsi_ops._reset_flag_cache()
+    yield request.param
+    bsi_ops._reset_flag_cache()
+
+
+@pytest.mark.parametrize("flags", FLAGS, indirect=True, ids=lambda f: ",".join(f"{k[4:]}={v}" for k, v in f.items()) or "default")
+def test_dot_micro_benchmark_reports(flags):
+    from bsipytorch_amd.benchmarks import benchmark_dot_kernel_micro as micro
+
+    for kw in ({}, {"relu": True}, {"outliers": True}, {"use_ints8": False}):
+        r = micro.run(48, 80, 1024, 2, 0.5, 1, 2, 123, "auto", **kw)
+        assert r["avg_dot_us"] > 0 and r["Q"] == 48 and r["R"] == 80 and isinstance(r["layout"], str)
+
+
+@pytest.mark.parametrize("flags", [{}, {"BSI_KEY_IMAGE_TILED": "1"}, {"BSI_FIXED_BITS": "0"}, {"BSI_DOT_CORE": "valu"}],
+                         indirect=True, ids=["default", "tiled-image", "decimal", "valu"])
+def test_layer_sweep_reports(flags, monkeypatch):
+    from bsipytorch_amd.benchmarks import benchmark_layer_sweep as sweep
+
+    monkeypatch.setitem(sweep.MODELS, "tiny", (256, 1024))
+    rows = sweep.run("tiny", Qs=(1, 40), iters=2, warmup=1)
+    assert len(rows) == 6 and all(r["avg_dot_us"] > 0 for r in rows)
+    torch.cuda.synchronize()
