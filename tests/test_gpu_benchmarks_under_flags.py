@@ -56,3 +56,24 @@ def test_layer_sweep_reports(flags, monkeypatch):
     rows = sweep.run("tiny", Qs=(1, 40), iters=2, warmup=1)
     assert len(rows) == 6 and all(r["avg_dot_us"] > 0 for r in rows)
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("flags,options", [({}, {}), ({}, {"fuse_qkv": True}), ({}, {"quantize_lm_head": True, "dense": True}),
+                                           ({"BSI_FIXED_BITS": "0"}, {}), ({"BSI_QUERY_CACHE": "0"}, {}),
+                                           ({"BSI_KEY_IMAGE_TILED": "1"}, {"fuse_qkv": True})],
+                         indirect=["flags"], ids=["default", "fuse", "lm_head+dense", "decimal", "no-cache", "tiled-image+fuse"])
+def test_prefill_benchmark_reports(flags, options, monkeypatch):
+    """benchmark_opt_prefill on a two-layer model of OPT's shape: eager, replayed graph (checked against eager by the
+    benchmark itself) and the per-call profile; decimal mode has no graph leg."""
+    from bsipytorch_amd.benchmarks import benchmark_opt_prefill as prefill
+
+    monkeypatch.setitem(prefill.SHAPES, "tiny", (2, 256, 4, 1024, 512))
+    kw = dict(dense=False)
+    kw.update(options)
+    r = prefill.run("tiny", seq_len=64, batch=1, iters=2, warmup=1, **kw)
+    assert r["num_bsi_layers"] == (13 if options.get("quantize_lm_head") else 12) and r["bsi_fwd_ms"] > 0
+    if flags.get("BSI_FIXED_BITS") == "0":
+        assert r["bsi_graph_fwd_ms"] is None
+    else:
+        assert r["graph_replays_match_eager"] is True and r["bsi_graph_fwd_ms"] > 0
+    assert r["dot_ms_per_prefill"] > 0
