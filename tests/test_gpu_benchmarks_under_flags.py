@@ -77,3 +77,15 @@ def test_prefill_benchmark_reports(flags, options, monkeypatch):
     else:
         assert r["graph_replays_match_eager"] is True and r["bsi_graph_fwd_ms"] > 0
     assert r["dot_ms_per_prefill"] > 0
+
+
+@pytest.mark.parametrize("flags", [{}, {"BSI_FIXED_BITS": "0"}, {"BSI_KEY_INT8_IMAGE": "0"}], indirect=True,
+                         ids=["default", "decimal", "no-image"])
+def test_apples_to_apples_and_dense_benchmarks_report(flags):
+    from bsipytorch_amd.benchmarks import benchmark_apples_to_apples_bsi as apples
+    from bsipytorch_amd.benchmarks import benchmark_dense_matmul_micro as dense
+
+    r = apples.run_modes(["kernel_only", "linear_e2e"], 40, 72, 1024, 2, 0.5, 1, 2, 123, "fp16")
+    assert set(r) == {"kernel_only", "linear_e2e"} and all(v["bsi_ms"] > 0 and v["torch_ms"] > 0 for v in r.values())
+    for dt in ("fp16", "bf16", "fp32"):
+        assert dense.run(40, 72, 1024, dt, 1, 2)
