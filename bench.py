@@ -31,7 +31,7 @@ Q, R, D = 512, 8192, 2048
 # runs of this script scaled by a 256 MiB copy (profiles/dot_mfma_i8_kernel_fc1_Q512_R8192_D2048_hbm_traffic.txt).
 # Hardware counters cannot be read from inside the process, so it is not re-measured by a run of this script.
 MEASURED_TRAFFIC_BYTES = {"mfma": 42439000}
-TRAFFIC_SOURCE = "offline: profiles/dot_mfma_i8_kernel_fc1_Q512_R8192_D2048_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)"
+TRAFFIC_SOURCE = "offline: profiles/dot_mfma_i8_kernel_fc1_Q512_R8192_D2048_hbm_traffic.txt"
 SA, SB = 7, 6
 
 
@@ -68,6 +68,17 @@ def _graph_timed_us(launches, rounds=4, replays=5):
     return best
 
 
+def _compact(o):
+    """Floats to five significant digits: the line stays short enough for whatever keeps only the end of the output."""
+    if isinstance(o, float):
+        return float(f"{o:.5g}")
+    if isinstance(o, dict):
+        return {k: _compact(v) for k, v in o.items()}
+    if isinstance(o, (list, tuple)):
+        return [_compact(v) for v in o]
+    return o
+
+
 def _fc2_like(_lib, bsi_ops, iters, settle_ms):
     """FC2-like dot Q512 x R2048 x D8192, ReLU queries: the int8-image kernel on the verbatim batch, and the same
     batch kept as EWAH streams (decode launch + dot) next to the verbatim planes taken through the same two steps."""
@@ -96,10 +107,10 @@ def _fc2_like(_lib, bsi_ops, iters, settle_ms):
     t = float(us.value) * 1e-6
     int8_ops = 2.0 * Q3 * R3 * D3
     alg_bytes = Q3 * SA * W * 8 + Q3 * chunks * 4 + R3 * SB * W * 8 + R3 * 4 + Q3 * R3 * 4
-    res = {"workload": "FC2-like fixed76 chunk-scale dot Q512 R2048 D8192, ReLU queries", "us_per_call": t * 1e6,
+    res = {"workload": "FC2-like dot Q512 R2048 D8192, ReLU queries", "us_per_call": t * 1e6,
            "effective_bitop_TOPS": 2.0 * SA * SB * Q3 * R3 * D3 / t / 1e12,
            "frac_of_int8_mfma_peak": int8_ops / t / 1e12 / MFMA_I8_PEAK_TOPS,
-           "frac_of_hbm_peak_algorithmic": alg_bytes / t / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": alg_bytes,
+           "frac_of_hbm_peak_algorithmic": alg_bytes / t / 1e9 / HBM_PEAK_GBS,
            "us_per_call_before_settling": first_us}
     # queries as EWAH streams: the dot's load stage turns the streams into the int8 image (one launch), then the same
     # kernel runs; next to it the verbatim planes through planes -> int8 image -> dot (what a caller holding planes pays)
@@ -120,9 +131,7 @@ def _fc2_like(_lib, bsi_ops, iters, settle_ms):
     res["ewah_queries"] = {
         "us_per_call_streams": _graph_timed_us([ewah], rounds=8) ,
         "us_per_call_verbatim_planes": _graph_timed_us([planes], rounds=8),
-        "stored_query_bytes_streams": int(hb.mem_bytes), "stored_query_bytes_verbatim": int(hb.verbatim_bytes),
-        "note": "both include the launch that derives the int8 query image (from streams / from planes); the headline "
-                "figure above reads the image the builder wrote with the planes"}
+        "stored_query_bytes_streams": int(hb.mem_bytes), "stored_query_bytes_verbatim": int(hb.verbatim_bytes)}
     # a few rows (16 tokens against an OPT-6.7B attention projection): the streams are expanded inside the dot kernel
     R6 = D6 = 4096
     g6 = torch.Generator(device="cuda").manual_seed(6)
@@ -186,8 +195,7 @@ def _decode_shapes(_lib, bsi_ops):
 
         resident = _graph_timed_us([launch(keysets[0])], rounds=32)
         rotating = _graph_timed_us([launch(kc) for kc in keysets], rounds=2)
-        rows.append({"layer": name, "Q": 1, "packed_key_plane_bytes": plane_bytes, "keysets_in_rotation": n_sets,
-                     "us_resident": resident, "GBs_on_planes_resident": plane_bytes / resident / 1e3,
+        rows.append({"layer": name, "us_resident": resident, "GBs_on_planes_resident": plane_bytes / resident / 1e3,
                      "us_rotating": rotating, "GBs_on_planes_rotating": plane_bytes / rotating / 1e3,
                      "frac_of_hbm_peak_rotating": plane_bytes / rotating / 1e3 / HBM_PEAK_GBS})
         del keysets
@@ -227,8 +235,8 @@ def _headline_rotating(_lib, bsi_ops):
     resident = _graph_timed_us([launch(keysets[0])], rounds=32)
     rotating = _graph_timed_us([launch(kc) for kc in keysets], rounds=2)
     ops = 2.0 * Qh * Rh * Dh
-    return {"workload": "Q512 R8192 D2048, launches replayed from a HIP graph", "keysets_in_rotation": n_sets,
-            "key_image_bytes": image_bytes, "us_resident": resident, "us_rotating": rotating,
+    return {"workload": "Q512 R8192 D2048 replayed from a HIP graph", "keysets_in_rotation": n_sets,
+            "us_resident": resident, "us_rotating": rotating,
             "frac_of_int8_mfma_peak_rotating": ops / (rotating * 1e-6) / 1e12 / MFMA_I8_PEAK_TOPS}
 
 
@@ -238,7 +246,7 @@ def _opt_prefill():
     from bsipytorch_amd.benchmarks import benchmark_opt_prefill
 
     r = benchmark_opt_prefill.run("opt-1.3b", seq_len=512, batch=1, iters=5, warmup=2, dense=False, graph=True)
-    keep = ("model", "layers", "seq_len", "num_bsi_layers", "bsi_fwd_ms", "bsi_tokens_per_s", "bsi_graph_fwd_ms",
+    keep = ("model", "seq_len", "num_bsi_layers", "bsi_fwd_ms", "bsi_tokens_per_s", "bsi_graph_fwd_ms",
             "bsi_graph_tokens_per_s", "graph_replays_match_eager", "dot_ms_per_prefill", "dot_share_of_fwd",
             "query_build_kernel_ms_per_prefill", "key_build_s")
     res = {k: r[k] for k in keep if k in r}
@@ -330,9 +338,8 @@ def main() -> int:
         settle_steps = max(1, int(args.settle_ms / from_idle_ms))
         for _ in range(settle_steps):  # no synchronisation in between: an idle gap would let the clock state decay
             step()
-        settle = {"ms": args.settle_ms, "untimed_steps": settle_steps, "us_per_call_from_idle": from_idle_ms * 1e3,
-                  "note": "untimed steps run back to back before the warm-up steps until the shader clock holds its "
-                          "sustained state; us_per_call_from_idle is the same warm-up + timed steps on an idle GPU"}
+        # untimed steps run back to back before the warm-up steps; us_per_call_from_idle: the same W + K steps on an idle GPU
+        settle = {"ms": args.settle_ms, "untimed_steps": settle_steps, "us_per_call_from_idle": from_idle_ms * 1e3}
     ms_per_step = timed_steps()
 
     # kernel duration with HIP events on the launch stream (same K launches, back to back)
@@ -364,8 +371,6 @@ def main() -> int:
     roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(used_core)
     roof["traffic_source"] = TRAFFIC_SOURCE if roof["traffic"] is not None else None
     roof["kernel_us"] = kern_us
-    roof["algorithmic_bytes"] = alg_bytes
-    roof["hbm_GBs_algorithmic"] = hbm_gbs
     # one v_and_b32 + one v_bcnt_u32_b32 per 32 bit-MACs; 256 CU x 4 SIMD x 16 lanes x 2.4 GHz lane-ops/s
     valu_peak = 256 * 4 * 16 * 2.4e9 * 32 / 2 / 1e12
     valu = {"achieved_Tbitmac_s": bit_ops / 2 / (kern_us * 1e-6) / 1e12, "peak_Tbitmac_s": valu_peak}
@@ -384,13 +389,12 @@ def main() -> int:
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "int8" if used_core == "mfma" else "u32",
-        "dtype_note": "int8 x int8 -> int32 MFMA per 256-element chunk, fp32 fmaf chunk-scale epilogue"
-                      if used_core == "mfma" else "u32 and/popcount -> int32 per chunk, fp32 fmaf chunk-scale epilogue",
+        "dtype_note": "int8 MFMA -> int32 per chunk, fp32 chain" if used_core == "mfma" else "u32 and/popcount -> int32 per chunk, fp32 chain",
         "data": "synthetic",
         "config": {"workload": "FC1-like fixed76 chunk-scale dot Q512 R8192 D2048, 0.1% outlier columns x20, dec=2",
                    "core": used_core, "key_layout": {0: "canonical planes", 1: "tiled16 planes", 2: "cached int8 image of the planes",
                                   3: "cached int8 image of the planes in 64-row tiles"}[klayout],
-                   "algorithmic_bytes": alg_bytes, "bit_ops": bit_ops},
+                   "algorithmic_bytes": alg_bytes, "bit_ops": int(bit_ops)},
         "roofline": roof,
     }
     if settle is not None:
@@ -400,7 +404,7 @@ def main() -> int:
 
     # peaks measured on this GPU by the library's probes (a pure v_mfma_i32_16x16x64_i8 loop, a pure
     # v_and/v_bcnt loop, a streaming read of 1 GiB), next to the published figures the roofline uses
-    peaks = {"published": {"int8_mfma_TOPS": MFMA_I8_PEAK_TOPS, "hbm_GBs": HBM_PEAK_GBS}}
+    peaks = {}
     v = ctypes.c_double(0.0)
     _lib.check(_lib.lib.bsi_hip_probe_mfma_i8(ctypes.byref(v), stream), "probe_mfma")
     peaks["int8_mfma_TOPS"] = v.value / 1e12
@@ -421,7 +425,6 @@ def main() -> int:
     peaks["l2_to_lds_GBs_four_loader_waves_row_pieces"] = v.value / 1e9
     # what the headline kernel's chunk loop has to move along that path: (TM + TN) x D bytes per workgroup
     loop_bytes = ((R + 127) // 128) * ((Q + 127) // 128) * (128 + 128) * D
-    peaks["headline_loop_bytes_l2_to_lds"] = loop_bytes
     peaks["headline_loop_floor_us_at_the_loader_rate"] = loop_bytes / v.value * 1e6
     del buf
     result["measured_peaks"] = peaks
@@ -485,8 +488,7 @@ def main() -> int:
         torch.cuda.synchronize()
         same = bool(np.array_equal(out.cpu().numpy(), ref))
         result["cpu_baseline"] = {"value": bit_ops / (t_cpu / reps) / 1e12, "unit": "TOPS", "cores": bsi_oracle.num_threads(),
-                                  "kind": "port", "sample": f"{reps} full passes of the same Q512 R8192 D2048 dot "
-                                  f"(oracle popcount form, OpenMP over keys); {t_cpu / reps * 1e3:.1f} ms per pass",
+                                  "kind": "port", "sample": f"{reps} full passes of the same dot (oracle popcount form, OpenMP over keys)",
                                   "ms_per_call": t_cpu / reps * 1e3, "gpu_output_bit_identical": same}
     if not args.no_extras and used_core == "mfma":
         extras = {}
@@ -500,7 +502,7 @@ def main() -> int:
                 extras[key] = {"error": f"{type(exc).__name__}: {exc}"}
             torch.cuda.empty_cache()
         result["other_configs"] = extras
-    print(json.dumps(result))
+    print(json.dumps(_compact(result)))
     return 0
 
 
