@@ -78,6 +78,9 @@ static int dot_launch(const uint64_t* A, const int8_t* A_ints8, const float* A_c
     // per-row operands (slice weights, bias, chunk scales) are fetched with 32-bit byte offsets
     BSI_REQUIRE(R <= (1 << 25) && Q <= (1 << 25), "at most 2^25 key rows and query rows per call (got R = %lld, Q = %lld)",
                 static_cast<long long>(R), static_cast<long long>(Q));
+    // query tiles (32 rows in the smallest kernel tile) ride on the launch grid's second dimension, which holds 65535
+    BSI_REQUIRE((Q + 31) / 32 <= 65535, "at most 65535 x 32 query rows per call (got Q = %lld); split the batch",
+                static_cast<long long>(Q));
     BSI_REQUIRE(b_layout == BSI_LAYOUT_CANONICAL || b_layout == BSI_LAYOUT_TILED16 || b_layout == BSI_LAYOUT_INT8 ||
                     b_layout == BSI_LAYOUT_INT8_TILED,
                 "unknown key layout %d", b_layout);
@@ -301,7 +304,10 @@ extern "C" int bsi_hip_dot_timed(const uint64_t* A, const int8_t* A_ints8, const
     hipStream_t st = as_stream(stream);
     hipEvent_t e0, e1;
     BSI_HIP_CHECK(hipEventCreate(&e0));
-    BSI_HIP_CHECK(hipEventCreate(&e1));
+    if (hipError_t ec = hipEventCreate(&e1); ec != hipSuccess) {
+        (void)hipEventDestroy(e0);
+        return fail(BSI_ERR_HIP, "hipEventCreate failed: %s", hipGetErrorString(ec));
+    }
     int rc = BSI_OK;
     hipError_t se = hipEventRecord(e0, st);
     for (int i = 0; i < iters && rc == BSI_OK; ++i)

@@ -127,8 +127,11 @@ __device__ __forceinline__ void i8_loader_wave(unsigned char* __restrict__ lds, 
     static_assert(KG % L == 0 && QG % L == 0 && NI == KG / L + QG / L, "loads per loader wave");
     unsigned char* const scale_lds = lds + 4 * C::kStage;  // [chunk & 3][loader][64] floats
     // The prologue below is kept short on purpose: it runs on one wave per SIMD while the whole workgroup waits for
-    // the first stage.  No row is clamped: a load that starts past its operand's end reads nothing (buffer bounds),
-    // and whatever such a row or query leaves in LDS only reaches outputs past R or Q, which are never stored.
+    // the first stage.  No row is clamped: the offset of a lane's ROW (group and row inside it) travels in the
+    // per-lane offset of the buffer load, which the hardware compares with the descriptor's size, so a row past its
+    // operand's end reads nothing; whatever such a row or query leaves in LDS only reaches outputs past R or Q, which
+    // are never stored.  The wave-uniform offset of the load carries the position INSIDE the row only (the
+    // half-chunk), so nothing depends on whether that offset takes part in the range check.
     // tiled keys: blocks of 64 rows x 128 bytes per half-chunk, 2 chunks of them per 64-row tile; rows past R
     // are zero padding inside the last block
     const uint32_t rowbytes32 = static_cast<uint32_t>(chunks) << 8;
@@ -143,9 +146,9 @@ __device__ __forceinline__ void i8_loader_wave(unsigned char* __restrict__ lds, 
     // A load moves group g of the stage: 8 rows x 128 bytes; lane = (row lr of the group, 16-byte column lc), and the
     // logical column that lands in LDS column lc of row 8 g + lr is lc ^ (((8 g + lr) >> 1) & 7) = lc ^ (4 (g & 1) +
     // (lr >> 1)).  Per lane: the offset inside the group, for either parity of g and for either layout; per load
-    // (scalar): the offset of its group.
+    // the offset of its group.
     const uint32_t lr = static_cast<uint32_t>(lane) >> 3, lc = static_cast<uint32_t>(lane) & 7;
-    uint32_t voff[NI], goff[NI];
+    uint32_t voff[NI];
     bool is_key[NI];  // known at compile time once the loops are unrolled
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
@@ -153,9 +156,9 @@ __device__ __forceinline__ void i8_loader_wave(unsigned char* __restrict__ lds, 
         const int gg = is_key[i] ? lw + L * i : lw + L * (i - KG / L);  // group of its operand
         const uint32_t col = (lc ^ (static_cast<uint32_t>(gg & 1) * 4 + (lr >> 1))) * 16;
         const bool tiled = is_key[i] && key_tiled;
-        voff[i] = (tiled ? lr * 128 : lr * rowbytes32) + col;
-        goff[i] = tiled ? static_cast<uint32_t>(gg >> 3) * kblock + static_cast<uint32_t>(gg & 7) * 1024
-                        : static_cast<uint32_t>(gg) * 8 * rowbytes32;
+        voff[i] = (tiled ? lr * 128 : lr * rowbytes32) + col +
+                  (tiled ? static_cast<uint32_t>(gg >> 3) * kblock + static_cast<uint32_t>(gg & 7) * 1024
+                         : static_cast<uint32_t>(gg) * 8 * rowbytes32);
     }
     const uint32_t kstep_bytes = key_tiled ? 8192u : 128u;  // from one half-chunk of a key row to the next
     // scales: loader wave lw fetches the 64 queries of group lw % (TN / 64) (waves fetching the same group
@@ -188,7 +191,7 @@ __device__ __forceinline__ void i8_loader_wave(unsigned char* __restrict__ lds, 
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
             const int g = i < KG / L ? lw + L * i : KG + lw + L * (i - KG / L);  // group of the stage
-            load16_to_lds(is_key[i] ? rk : rq, voff[i], goff[i] + (is_key[i] ? so_k : so_q),
+            load16_to_lds(is_key[i] ? rk : rq, voff[i], is_key[i] ? so_k : so_q,
                           lds + (h & 3) * C::kStage + g * 1024);
         }
         if (!kSum && (h & 1)) {  // with the second half of chunk c = h / 2: its scales

@@ -56,12 +56,18 @@ struct Workspace {
 std::mutex g_ws_mutex;
 Workspace g_ws[64];
 
-int workspace_for(size_t need, void** ptr, size_t* bytes) {
+// Growing the buffer synchronises the device and frees memory, which a stream that is being captured into a graph
+// must not see: while `stream` is capturing, a need beyond the present buffer is refused (run the call once eagerly
+// first, and the buffer is there).
+int workspace_for(size_t need, hipStream_t stream, void** ptr, size_t* bytes) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return BSI_ERR_HIP;
     std::lock_guard<std::mutex> lock(g_ws_mutex);
     Workspace& w = g_ws[dev];
     if (w.bytes < need) {
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &capturing) != hipSuccess) return BSI_ERR_HIP;
+        if (capturing != hipStreamCaptureStatusNone) return BSI_ERR_UNSUPPORTED;
         // the old buffer may still be read by launches in flight: free it only once the device is idle
         if (w.ptr != nullptr) {
             if (hipDeviceSynchronize() != hipSuccess) return BSI_ERR_HIP;
@@ -137,9 +143,12 @@ void launch_popcount_weighted_keys_literal_fused_multiq(const unsigned long long
     void* ws = nullptr;
     size_t ws_bytes = 0;
     if (need > 0) {
-        const int rc = workspace_for(need, &ws, &ws_bytes);
+        const int rc = workspace_for(need, stream, &ws, &ws_bytes);
         if (rc != BSI_OK) {
-            note_msg(kName, rc, "could not allocate the int8 query workspace");
+            note_msg(kName, rc, rc == BSI_ERR_UNSUPPORTED
+                                    ? "the int8 query workspace would have to grow while the stream is being captured; run "
+                                      "this call once outside the capture first"
+                                    : "could not allocate the int8 query workspace");
             return;
         }
     }

@@ -50,6 +50,10 @@ def test_argument_validation_returns_error_codes():
     W_long = 4 * 32769
     rc = L.bsi_hip_dot(1, None, 1, 1, 7, W_long, 1, 0, 1, 6, 4, 4, 1.0, 4, 1, None, _lib.CORE_MFMA, None, 0, None)
     assert rc == 3 and b"chunks" in L.bsi_hip_last_error()
+    # more query rows than the launch grid's second dimension holds tiles of 32 for: refused as an argument error
+    too_many = 65535 * 32 + 1
+    rc = L.bsi_hip_dot(1, None, 1, 8, 7, 32, 1, 0, 1, 6, 4, too_many, 1.0, 4, 1, None, 0, None, 0, None)
+    assert rc == 1 and b"query rows per call" in L.bsi_hip_last_error()
     # empty problems are fine and launch nothing
     assert L.bsi_hip_dot(None, None, None, 8, 7, 32, None, 0, None, 6, 0, 0, 1.0, 0, None, None, 0, None, 0, None) == 0
     assert L.bsi_hip_build_fixed(None, 0, 0, 128, 2, 7, 1, 0.0, None, None, None, None, None) == 0
