@@ -20,6 +20,7 @@ OPT_I8_TILE = 1
 OPT_DIGITS_ROUTE = 2
 OPT_BUILD_ITEMS = 3
 OPT_OUTPUT_STORES = 4
+OPT_I8_SPLIT = 5
 
 _vp = ctypes.c_void_p
 _i = ctypes.c_int
@@ -53,6 +54,9 @@ PROTOTYPES = {
     "bsi_hip_planes_to_int8": [_vp, _i64, _i, _i, _vp, _vp],
     "bsi_hip_set_option": [_i, _i],
     "bsi_hip_dot_workspace_bytes": [_i64, _i, _i],
+    "bsi_hip_dot_split_scratch_bytes": [],
+    "bsi_hip_dot_attach_split_scratch": [_vp, _sz],
+    "bsi_hip_dot_split_plan": [_i64, _i64, _i, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)],
     "bsi_hip_dot": [_vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _i, _i64, _i64, _f, _i64, _vp, _vp, _i, _vp, _sz, _vp],
     "bsi_hip_dot_static_scratch": [_vp, _vp, _i, _i, _i, _vp, _i, _vp, _i, _i64, _i64, _f, _i64, _vp, _vp, _vp],
     "bsi_hip_add_bias": [_vp, _vp, _i64, _i64, _i64, _vp],
@@ -91,6 +95,7 @@ _RESTYPES = {
     "bsi_hip_version": ctypes.c_char_p,
     "bsi_hip_last_error": ctypes.c_char_p,
     "bsi_hip_dot_workspace_bytes": _sz,
+    "bsi_hip_dot_split_scratch_bytes": _sz,
     "bsi_hip_dot_ewah_batch_workspace_bytes": _sz,
     "bsi_hip_linear_workspace_bytes": _sz,
     "bsi_hip_dot_digits_workspace_bytes": _sz,

@@ -46,6 +46,9 @@ def run(Q, R, D, decimal_places=2, compress_threshold=0.5, warmup=10, iters=50, 
     ws = torch.empty((max(ws_bytes, 16),), dtype=torch.uint8, device="cuda")
     st = torch.cuda.current_stream().cuda_stream
     kptr, klayout = bsi_ops.key_operand(kcap, Q, qcap.Sa, code)
+    bsi_ops.attach_split_scratch()  # as every dot through bsi_ops does: the D-split route, where the launcher picks it
+    tile, segments = ctypes.c_int(0), ctypes.c_int(0)
+    _lib.check(_lib.lib.bsi_hip_dot_split_plan(R, Q, W, ctypes.byref(tile), ctypes.byref(segments)), "bsi_hip_dot_split_plan")
     args = (qcap.words.data_ptr(), qcap.ints8.data_ptr() if use_ints8 else None, scales.data_ptr(), stride, qcap.Sa, W,
             kptr, klayout, kcap.slice_weights.data_ptr(), kcap.Sb, R, Q, 1.0 / 10.0 ** (2 * decimal_places),
             R, out.data_ptr(), code, ws.data_ptr(), ws_bytes)
@@ -57,6 +60,7 @@ def run(Q, R, D, decimal_places=2, compress_threshold=0.5, warmup=10, iters=50, 
     bit_ops = 2.0 * qcap.Sa * kcap.Sb * Q * R * D
     alg_bytes = Q * qcap.Sa * W * 8 + Q * chunks * 4 + R * kcap.Sb * W * 8 + R * 4 + Q * R * 4
     return {"Q": Q, "R": R, "D": D, "core": core, "layout": {0: "canonical", 1: "tiled16", 2: "int8 image", 3: "int8 image in 64-row tiles"}[klayout],
+            "i8_tile": tile.value if klayout >= 2 else None, "d_split_segments": segments.value if klayout >= 2 else None,
             "avg_dot_us": t * 1e6, "dot_q_us": t * 1e6 / Q, "dot_s_ns": t * 1e9 / (Q * R),
             "effective_bitop_TOPS": bit_ops / t / 1e12, "int8_TOPS": 2.0 * Q * R * D / t / 1e12,
             "algorithmic_GBps": alg_bytes / t / 1e9, "key_plane_GBps": key_bytes / t / 1e9, "iters": iters}
@@ -120,12 +124,16 @@ def main() -> None:
     p.add_argument("--report_stats", action="store_true")
     p.add_argument("--i8_tile", type=int, default=0, choices=[0, 128, 1284, 12864, 64, 6432],
                    help="force a tile of the int8-image kernel (1284: 128 x 128 on four MFMA waves of 64 x 64); 0 = automatic")
+    p.add_argument("--split", type=int, default=0,
+                   help="D-split of the int8-image kernel: 0 = by the launcher's cost model, 1 = never, n >= 2 = n segments "
+                        "per output tile (on --i8_tile 128 or 12864)")
     p.add_argument("--image_fill", default="built", choices=["built", "zero", "random", "magnitude"],
                    help="timing only: overwrite the int8 images (the clock follows the power the data draws)")
     a = p.parse_args()
     if not torch.cuda.is_available():
         raise RuntimeError("a GPU is required for this microbench")
     _lib.check(_lib.lib.bsi_hip_set_option(_lib.OPT_I8_TILE, a.i8_tile), "bsi_hip_set_option")
+    _lib.check(_lib.lib.bsi_hip_set_option(_lib.OPT_I8_SPLIT, a.split), "bsi_hip_set_option")
     r = run(a.Q, a.R, a.D, a.decimal_places, a.compress_threshold, a.warmup, a.iters, a.seed, a.core, a.key_sigma,
             a.outliers, a.relu, not a.planes_only, a.report_stats, a.image_fill)
     print(f"[Microbench] Q={a.Q} R={a.R} D={a.D} iters={a.iters} core={r['core']} layout={r['layout']}")

@@ -22,6 +22,7 @@ from __future__ import annotations
 import json
 import os
 import sys
+import threading
 from typing import List, Optional
 
 import torch
@@ -99,6 +100,7 @@ def _flags() -> dict:
         ewah_inline=(_env_int("BSI_EWAH_INLINE", 1) or 0) != 0,
         decimal_mfma=(_env_int("BSI_DECIMAL_MFMA", 1) or 0) != 0,
         image_tiled=(_env_int("BSI_KEY_IMAGE_TILED", 0) or 0) != 0,
+        dot_split=(_env_int("BSI_DOT_SPLIT", 1) or 0) != 0,
     )
     return _flag_cache
 
@@ -656,6 +658,8 @@ def _dot_ewah_batch(qb: "PrebuiltBSIQueryBatchHybridCUDA", keys: "PrebuiltBSIKey
     kptr, klayout = key_operand(keys, Q, Sa, _lib.CORE_MFMA)
     ws_bytes = int(lib.bsi_hip_dot_ewah_batch_workspace_bytes(Q, W))
     ws = _get_workspace(ws_bytes, dev)
+    if Q >= _SPLIT_MIN_Q and chunk_ints is None:
+        attach_split_scratch(dev)
     prof = f["profile"]
     if prof:
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -900,6 +904,54 @@ def _get_workspace(nbytes: int, dev) -> Optional[torch.Tensor]:
     return rec["buf"]
 
 
+# D-split scratch of the int8-image dot (bsi_hip_dot_attach_split_scratch): device index -> {"capture": buffer,
+# "eager": {stream: buffer}}.  One region per stream for eager launches (launches that share a region must not overlap
+# on the GPU) and one for launches recorded into a graph; regions are never freed, since a recorded launch holds its
+# region's address.  The library keeps the attachment per calling thread; _split_tls mirrors it to skip repeats.
+_split_scratch: dict = {}
+_split_tls = threading.local()
+_SPLIT_MIN_Q = 33  # fewer query rows go to the few-rows kernels, which never split
+
+
+def _new_split_region(dev) -> torch.Tensor:
+    # zero-filled: the region's counters must start at zero, and every launch leaves them so
+    return torch.zeros((int(lib.bsi_hip_dot_split_scratch_bytes()),), dtype=torch.uint8, device=dev)
+
+
+def attach_split_scratch(dev=None) -> bool:
+    """Attach this thread's D-split scratch region for the current stream of ``dev`` (default: the current device)
+    before a dot is launched; returns whether one is attached.  BSI_DOT_SPLIT=0 never attaches one.  While a graph is
+    being captured only a region that already exists is attached (a capture cannot allocate): the first eager call on
+    a device creates the capture region too."""
+    if not _flags()["dot_split"]:
+        if getattr(_split_tls, "ptr", 0):
+            check(lib.bsi_hip_dot_attach_split_scratch(None, 0), "bsi_hip_dot_attach_split_scratch")
+            _split_tls.ptr = 0
+        return False
+    dev = _device() if dev is None else dev
+    rec = _split_scratch.get(dev.index)
+    capturing = _capturing()
+    if rec is None:
+        if capturing:
+            buf = None
+        else:
+            rec = _split_scratch[dev.index] = {"capture": _new_split_region(dev), "eager": {}}
+    if rec is not None:
+        if capturing:
+            buf = rec["capture"]
+        else:
+            st = _stream()
+            buf = rec["eager"].get(st)
+            if buf is None:
+                buf = rec["eager"][st] = _new_split_region(dev)
+    ptr = 0 if buf is None else buf.data_ptr()
+    if getattr(_split_tls, "ptr", 0) != ptr or getattr(_split_tls, "dev", -1) != dev.index:
+        check(lib.bsi_hip_dot_attach_split_scratch(ptr or None, 0 if buf is None else buf.numel()),
+              "bsi_hip_dot_attach_split_scratch")
+        _split_tls.ptr, _split_tls.dev = ptr, dev.index
+    return buf is not None
+
+
 def _scale_inv(dec_q: int, dec_k: int) -> float:
     # bsi_cuda.cpp:709-711: (float)(1.0 / 10^(dq + dk)); the C ABI takes it as float
     total = dec_q + dec_k
@@ -944,6 +996,8 @@ def _dot(words, ints8, scales, scale_stride, Sa, W, keys: PrebuiltBSIKeysCUDA, Q
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
     kptr, klayout = key_operand(keys, Q, Sa, core)
+    if Q >= _SPLIT_MIN_Q and chunk_ints is None:
+        attach_split_scratch(dev)
     if warm_keys is not None and chunk_ints is None:
         # the kernel also touches what the next layer's dot will read, so that it is cache-resident by then
         wptr, wbytes = _warm_region(warm_keys, Q, Sa, core)
@@ -1179,6 +1233,8 @@ def linear_cuda(x2d: torch.Tensor, keyset_cuda_cap, decimal_places: int, bias=No
     out = torch.empty((Q, R), dtype=torch.float32, device=x2d.device)
     core = f["core"]
     kptr, klayout = key_operand(keys, Q, bits, core)
+    if Q >= _SPLIT_MIN_Q:
+        attach_split_scratch(x2d.device)
     wptr, wbytes = _warm_region(_capsule(warm_keys, PrebuiltBSIKeysCUDA, "Invalid CUDA keys capsule") if warm_keys is not None
                                 else None, Q, bits, core)
     check(lib.bsi_hip_linear(x2d.data_ptr(), _dtype_code(x2d), Q, d, int(decimal_places), bits, rebuild, wsptr, ws["bytes"],

@@ -50,6 +50,10 @@ extern "C" int bsi_hip_set_option(int option, int value) {
             BSI_REQUIRE(value >= 0 && value <= 2, "output stores must be 0 (by entry point), 1 (plain) or 2 (nontemporal)");
             g_output_stores = value;
             return BSI_OK;
+        case BSI_OPT_I8_SPLIT:
+            BSI_REQUIRE(value >= 0 && value <= 64, "split must be 0 (by cost), 1 (never) or a number of segments up to 64");
+            g_i8_split = value;
+            return BSI_OK;
         case BSI_OPT_BUILD_ITEMS:
             BSI_REQUIRE(value == 0 || value == 1 || value == 2 || value == 4 || value == 8, "items must be 0, 1, 2, 4 or 8");
             g_build_items = value;
@@ -62,6 +66,36 @@ extern "C" int bsi_hip_set_option(int option, int value) {
 extern "C" size_t bsi_hip_dot_workspace_bytes(int64_t Q, int W64, int core) {
     if (core == BSI_CORE_VALU || Q <= 0 || W64 <= 0) return 0;
     return static_cast<size_t>(Q) * static_cast<size_t>((W64 + 3) / 4) * 256;
+}
+
+extern "C" size_t bsi_hip_dot_split_scratch_bytes(void) {
+    // one round of 256 workgroups, each with the partial sums of a 128 x 128 tile
+    return kSplitCounterBytes + static_cast<size_t>(256) * 128 * 128 * sizeof(float);
+}
+
+extern "C" int bsi_hip_dot_attach_split_scratch(void* scratch_device, size_t bytes) {
+    if (scratch_device == nullptr || bytes == 0) {
+        t_split_scratch = nullptr;
+        t_split_bytes = 0;
+        t_split_device = -1;
+        return BSI_OK;
+    }
+    BSI_REQUIRE((reinterpret_cast<uintptr_t>(scratch_device) & 255) == 0, "the split scratch must be 256-byte aligned");
+    BSI_REQUIRE(bytes > kSplitCounterBytes, "a split scratch holds %zu bytes of counters and then the partial sums (got %zu bytes)",
+                kSplitCounterBytes, bytes);
+    int dev = -1;
+    BSI_HIP_CHECK(hipGetDevice(&dev));
+    t_split_scratch = static_cast<unsigned char*>(scratch_device);
+    t_split_bytes = bytes;
+    t_split_device = dev;
+    return BSI_OK;
+}
+
+extern "C" int bsi_hip_dot_split_plan(int64_t R, int64_t Q, int W64, int* tile, int* segments) {
+    BSI_REQUIRE(tile && segments && R >= 1 && Q >= 1 && W64 >= 1, "bad arguments");
+    const int split_tile = choose_i8_split(R, Q, (W64 + 3) / 4, segments);
+    *tile = split_tile != 0 ? split_tile : choose_i8_tile(R, Q);
+    return BSI_OK;
 }
 
 // Validation, kernel selection and launch.  `bias` (optional) is added to every output; *bias_fused tells

@@ -87,7 +87,13 @@ struct I8Cfg {
     static constexpr int kScaleBytes = 4 * kLoaders * 256;  // chunk scales: ring of 4 chunks x loader regions x 64 floats
     static constexpr int kEpilogueBytes = 2 * TM * 4;  // the tile's key factors, then its biases (chain modes)
     static constexpr int kLds = 4 * kStage + kScaleBytes + kEpilogueBytes;
+    // D-split launches: one flag word per MFMA wave (a prefix of its chain came near the exactness limit), then the
+    // workgroup's decision (kSplitLeave / kSplitCombine / kSplitRedo)
+    static constexpr int kSplitFlagBytes = 64;
+    static constexpr int kLdsSplit = kLds + kSplitFlagBytes;
+    static_assert(kConsumers < 15, "flag words of the MFMA waves, then the decision word");
 };
+constexpr int kSplitLeave = 0, kSplitCombine = 1, kSplitRedo = 2;
 
 // Timeline build (make TIMELINE=1, -DBSI_TIMELINE): one MFMA wave and one loader wave of every workgroup of
 // dot_mfma_i8_kernel stamp the 100 MHz wall clock at the points below, 8 slots per workgroup (the first
@@ -101,7 +107,7 @@ enum TimelineStamp {
 __device__ unsigned long long g_timeline[kTimelineWorkgroups * 8];
 #define BSI_STAMP(slot)                                                                    \
     {                                                                                      \
-        const unsigned wg_ = blockIdx.y * gridDim.x + blockIdx.x;                          \
+        const unsigned wg_ = (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x; \
         if (lane == 0 && wg_ < kTimelineWorkgroups) g_timeline[wg_ * 8 + (slot)] = wall_clock64(); \
     }
 #else
@@ -115,8 +121,8 @@ template <typename C, bool kSum>
 __device__ __forceinline__ void i8_loader_wave(unsigned char* __restrict__ lds, int lw, int lane,
                                                const int8_t* __restrict__ A8, const float* __restrict__ qscale,
                                                int qscale_stride, const int8_t* __restrict__ K8,
-                                               const float* __restrict__ Bw, int Sb, int chunks, int halves, int64_t R,
-                                               int64_t Q, int64_t r0, int64_t q0, size_t rowbytes,
+                                               const float* __restrict__ Bw, int Sb, int chunks, int first_chunk,
+                                               int halves, int64_t R, int64_t Q, int64_t r0, int64_t q0, size_t rowbytes,
                                                const float* __restrict__ bias, int ndig, long long dig_stride,
                                                int key_tiled, const unsigned char* __restrict__ warm,
                                                long long warm_lines) {
@@ -166,8 +172,9 @@ __device__ __forceinline__ void i8_loader_wave(unsigned char* __restrict__ lds, 
     const bsi_rsrc rs = make_rsrc(qscale + q0 * qscale_stride, static_cast<size_t>(Q - q0) * qscale_stride * 4);
     const uint32_t soff = static_cast<uint32_t>((lw % (TN >= 64 ? TN / 64 : 1)) * 64 + lane) * static_cast<uint32_t>(qscale_stride) * 4;
     const int sstep = (qscale_stride == 1) ? 0 : 4;
-    // issue() is called for h = 0, 1, 2, ... in order; in the sum mode (next_c, next_dg) follow the chunk and
-    // the digit (counted from the top one) of the half-chunk to come
+    // issue() is called for h = 0, 1, 2, ... in order, h counted from the first half of chunk first_chunk (the
+    // workgroup's share of the row in a D-split launch, else 0); in the sum mode (next_c, next_dg) follow the chunk
+    // and the digit (counted from the top one) of the half-chunk to come
     int next_c = 0, next_dg = 0;
     uint32_t so_k = 0, so_q = 0;
     auto issue = [&](int h) {  // stage of half-chunk h (clamped to the last) into its ring slot
@@ -185,8 +192,8 @@ __device__ __forceinline__ void i8_loader_wave(unsigned char* __restrict__ lds, 
                 }
             }
         } else {
-            so_q = static_cast<uint32_t>(hc) * 128;
-            so_k = static_cast<uint32_t>(hc) * kstep_bytes;
+            so_q = static_cast<uint32_t>(hc + 2 * first_chunk) * 128;
+            so_k = static_cast<uint32_t>(hc + 2 * first_chunk) * kstep_bytes;
         }
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
@@ -198,7 +205,7 @@ __device__ __forceinline__ void i8_loader_wave(unsigned char* __restrict__ lds, 
             const int c = hc >> 1;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(
                 rs, BSI_LDS_PTR(scale_lds + ((c & 3) * C::kLoaders + lw) * 256), 4, static_cast<int>(soff),
-                c * sstep, 0, 0);
+                (c + first_chunk) * sstep, 0, 0);
         }
     };
     if (lw == 0) BSI_STAMP(kStampFirstIssue);
@@ -249,8 +256,8 @@ __device__ __forceinline__ void i8_loader_wave(unsigned char* __restrict__ lds, 
     if (warm_lines > 0) {
         // one lane per 128-byte line, 64 lines per load; this loader wave's share of the region.  The values
         // are summed only so that the loads stay; the store below never happens.
-        const long long waves = static_cast<long long>(gridDim.x) * gridDim.y * C::kLoaders;
-        const long long mine = (static_cast<long long>(blockIdx.y) * gridDim.x + blockIdx.x) * C::kLoaders + lw;
+        const long long waves = static_cast<long long>(gridDim.x) * gridDim.y * gridDim.z * C::kLoaders;
+        const long long mine = ((static_cast<long long>(blockIdx.z) * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * C::kLoaders + lw;
         const long long per = (warm_lines + waves - 1) / waves;
         const long long first = mine * per;
         const long long last = (first + per < warm_lines) ? first + per : warm_lines;
@@ -270,14 +277,19 @@ __device__ __forceinline__ void i8_loader_wave(unsigned char* __restrict__ lds, 
 // kMode: kI8Chain (fp32 chunk-scale chain), kI8Ints (the same, and the per-chunk integers are stored) or kI8Sum
 // (plain int32 sum over all chunks: no scales, no epilogue).
 constexpr int kI8Chain = 0, kI8Ints = 1, kI8Sum = 2;
-template <int WM, int WN, int KS, int kMode>
+#ifndef BSI_SPLIT_TRACK
+#define BSI_SPLIT_TRACK kSplit
+#endif
+template <int WM, int WN, int KS, int kMode, bool kTrack>
 __device__ __forceinline__ void i8_kstep(const v4i (&ka)[WM], const v4i (&qb)[WN], v4i (&ka_n)[WM], v4i (&qb_n)[WN],
                                          const unsigned char* __restrict__ krow_n,
                                          const unsigned char* __restrict__ qrow_n, v4i (&acc)[WM][WN],
                                          const v4i (&prev)[WM][WN], float (&accf)[WM][WN][4],
                                          const float (&qs_prev)[WN], int* __restrict__ ints_prev,
                                          const int64_t (&int_off)[WM][WN], const int (&int_rows)[WM], int down_shift,
-                                         int chunks) {
+                                         int chunks, float& peak) {
+    // kTrack (D-split launches): `peak` follows the largest magnitude the lane's chain values take, two of them per
+    // three-input maximum
     static_assert(WM + WN <= 2 * WM * WN, "two operand reads behind each MFMA of a k-step");
 #pragma unroll
     for (int a = 0; a < WM; ++a)
@@ -290,6 +302,7 @@ __device__ __forceinline__ void i8_kstep(const v4i (&ka)[WM], const v4i (&qb)[WN
             if (kMode != kI8Sum) {
                 const int idx = KS * (WM * WN) + t, tt = idx >> 2, e = idx & 3, ea = tt / WN, eb = tt % WN;
                 accf[ea][eb][e] = fmaf(static_cast<float>(prev[ea][eb][e]), qs_prev[eb], accf[ea][eb][e]);
+                if (kTrack && (e & 1)) peak = fmaxf(fmaxf(peak, fabsf(accf[ea][eb][e - 1])), fabsf(accf[ea][eb][e]));
                 if (kInts && ints_prev != nullptr && int_off[ea][eb] >= 0 && e < int_rows[ea])
                     ints_prev[int_off[ea][eb] + static_cast<int64_t>(e) * chunks] = prev[ea][eb][e] >> down_shift;
             }
@@ -348,14 +361,25 @@ __device__ __forceinline__ bool i8_store_lines(const float (&v)[WM][WN][4], floa
     return true;
 }
 
-template <int TM, int TN, int kMode>
+template <int TM, int TN, int kMode, bool kSplit>
 __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
     const int8_t* __restrict__ A8, const float* __restrict__ qscale, int qscale_stride,
     const int8_t* __restrict__ K8,  // int8 key image [R, chunks * 256]
     const float* __restrict__ Bw, int Sb, int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv,
     int64_t R_total, float* __restrict__ out, int* __restrict__ chunk_ints, const float* __restrict__ bias,
     int ndig, long long dig_stride, const long long* __restrict__ key_indices, int key_tiled,
-    const unsigned char* __restrict__ warm, long long warm_lines, int out_stream) {
+    const unsigned char* __restrict__ warm, long long warm_lines, int out_stream, float* __restrict__ split_partials,
+    unsigned* __restrict__ split_counters, float split_limit, int split_shape) {
+    // kSplit (chain mode only): a D-split launch.  gridDim.z workgroups share an output tile, each running the chain
+    // over its own run of chunks from zero.  All operands of the chain are integers (times one power of two), so
+    // as long as no value the chain takes exceeds 2^24 of its unit nothing is ever rounded, the value after every
+    // chunk is the exact sum so far, and sums of the segments' results in any order equal the one sequential chain over
+    // all chunks bit for bit.  Each workgroup follows the largest magnitude its chain values take; with every
+    // segment's peak at most split_limit = 2^24 units / gridDim.z, every prefix of the sequential chain is at most
+    // 2^24 units as well, which proves the equality.  A workgroup stores its partial sums to split_partials, then
+    // counts itself in at split_counters[tile] (bit 16 and up: segments whose peak went over the limit); the last
+    // one to arrive adds the others' sums to its own and writes the outputs -- or, if any segment went over the
+    // limit, runs the whole tile again over all chunks in order.  It leaves the counter at zero.
     // out_stream: the float outputs of whole tiles go out with nontemporal stores (they leave the caches as they are
     // written) instead of plain ones (they stay for the kernel that reads them next).
     // warm / warm_lines: an optional region of 128-byte lines (the keys the NEXT dot will read) that the loader
@@ -377,17 +401,53 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int64_t r0 = static_cast<int64_t>(blockIdx.x) * TM;
-    const int64_t q0 = static_cast<int64_t>(blockIdx.y) * TN;
+    // Which tile (and, in a D-split launch, which segment) this workgroup computes.  A D-split launch is a 1-D grid
+    // decoded so that -- workgroups being dealt to the eight XCDs in turn -- an XCD gets one segment of a few key
+    // tiles for all query tiles: its L2 then fetches that run of chunks of those key rows and of all query rows
+    // once, as in an unsplit launch of a short row, instead of every segment of whole rows.
+    int bx = static_cast<int>(blockIdx.x), by = static_cast<int>(blockIdx.y), seg = 0, nseg = 1, tiles_x = static_cast<int>(gridDim.x);
+    if (kSplit) {
+        tiles_x = split_shape & 1023;
+        const int tiles_y = (split_shape >> 10) & 1023;
+        nseg = split_shape >> 20;
+        const int id = static_cast<int>(blockIdx.x);
+        if (nseg == 2 || nseg == 4 || nseg == 8) {
+            const int per = 8 / nseg, slot = id & 7, rest = id >> 3;   // key tiles of one segment per round of 8 workgroups
+            const int xh_count = (tiles_x + per - 1) / per;
+            seg = slot / per;
+            bx = (rest % xh_count) * per + slot % per;
+            by = rest / xh_count;
+        } else {
+            bx = id % tiles_x;
+            by = (id / tiles_x) % tiles_y;
+            seg = id / (tiles_x * tiles_y);
+        }
+        if (bx >= tiles_x || by >= tiles_y || seg >= nseg) return;  // padding of the last round
+    }
+    const int64_t r0 = static_cast<int64_t>(bx) * TM;
+    const int64_t q0 = static_cast<int64_t>(by) * TN;
     const size_t rowbytes = static_cast<size_t>(chunks) * 256;
+    static_assert(!kSplit || kMode == kI8Chain, "only the plain chain splits D");
     const int vchunks = kSum ? chunks * ndig : chunks;  // chunks of the loop: every digit image runs over all chunks
-    const int halves = vchunks * 2;
+    // the workgroup's run of chunks: all of them, or segment seg of nseg
+    const int first_chunk = kSplit ? (chunks * seg) / nseg : 0;
+    const int my_chunks = kSplit ? (chunks * (seg + 1)) / nseg - first_chunk : vchunks;
     unsigned char* const scale_lds = lds + 4 * C::kStage;  // [chunk & 3][loader][64] floats
+    // kSplit: [MFMA wave] flags, [15] = decision
+    volatile __attribute__((address_space(3))) int* const split_flags =
+        reinterpret_cast<volatile __attribute__((address_space(3))) int*>(BSI_LDS_PTR(lds + C::kLds));
 
     if (wave >= C::kConsumers) {
         if (wave == C::kConsumers) BSI_STAMP(kStampLoaderEntry);
-        i8_loader_wave<C, kSum>(lds, wave - C::kConsumers, lane, A8, qscale, qscale_stride, K8, Bw, Sb, chunks, halves, R,
-                                     Q, r0, q0, rowbytes, bias, ndig, dig_stride, key_tiled, warm, warm_lines);
+        i8_loader_wave<C, kSum>(lds, wave - C::kConsumers, lane, A8, qscale, qscale_stride, K8, Bw, Sb, chunks, first_chunk,
+                                my_chunks * 2, R, Q, r0, q0, rowbytes, bias, ndig, dig_stride, key_tiled, warm, warm_lines);
+        if (kSplit) {
+            lds_barrier();  // the MFMA waves have stored their partial sums
+            lds_barrier();  // the decision is in LDS
+            if (__builtin_amdgcn_readfirstlane(split_flags[15]) == kSplitRedo)
+                i8_loader_wave<C, kSum>(lds, wave - C::kConsumers, lane, A8, qscale, qscale_stride, K8, Bw, Sb, chunks, 0,
+                                        chunks * 2, R, Q, r0, q0, rowbytes, bias, ndig, dig_stride, key_tiled, nullptr, 0);
+        }
         if (wave == C::kConsumers) BSI_STAMP(kStampLoaderDone);
         return;
     }
@@ -444,10 +504,10 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
     // which its last operands were read (the even ones); the same barrier tells that the next stage has landed.
     v4i ka[2][WM], qb[2][WN];  // operand sets of even / odd k-steps
 #define BSI_I8_KSTEP(KS, nslot, acc, prev, qs, ip)                                                                  \
-    i8_kstep<WM, WN, KS, kMode>(ka[(KS) & 1], qb[(KS) & 1], ka[((KS) + 1) & 1], qb[((KS) + 1) & 1],                 \
+    i8_kstep<WM, WN, KS, kMode, BSI_SPLIT_TRACK>(ka[(KS) & 1], qb[(KS) & 1], ka[((KS) + 1) & 1], qb[((KS) + 1) & 1],         \
                                 lds + (nslot) * C::kStage + krow_off + pcol[((KS) + 1) & 1],                        \
                                 lds + (nslot) * C::kStage + qrow_off + pcol[((KS) + 1) & 1], acc, prev, accf, qs,   \
-                                ip, int_off, int_rows, down_shift, chunks);
+                                ip, int_off, int_rows, down_shift, chunks, peak);
     // a chunk whose halves sit in ring slots s0, s0 + 1; nslot: slot of the next chunk's first half
 #define BSI_I8_CHUNK(s0, nslot, acc, prev, qs, ip)                                                                  \
     BSI_I8_KSTEP(0, s0, acc, prev, qs, ip);                                                                         \
@@ -457,6 +517,23 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
     lds_barrier();                                                                                                  \
     BSI_I8_KSTEP(3, nslot, acc, prev, qs, ip);
 
+    float peak = 0.0f;      // kSplit: the largest magnitude the lane's chain values have taken
+    int run_chunks = my_chunks;
+    bool last_in_acc0 = false;
+#pragma nounroll
+    for (int pass = 0;; ++pass) {  // one pass; a D-split launch's last workgroup of a tile may need a second over all chunks
+    if (kSplit && pass > 0) {
+#pragma unroll
+        for (int a = 0; a < WM; ++a)
+#pragma unroll
+            for (int b = 0; b < WN; ++b) {
+                acc0[a][b] = acc1[a][b] = (v4i){0, 0, 0, 0};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) accf[a][b][e] = 0.0f;
+            }
+#pragma unroll
+        for (int b = 0; b < WN; ++b) qsa[b] = qsb[b] = 0.0f;
+    }
     lds_barrier();  // stage 0 is there
     if (wave == 0) BSI_STAMP(kStampFirstStage);
 #pragma unroll
@@ -477,7 +554,7 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
         --to_next_digit;                                                              \
     }
     int c = 0;
-    for (; c + 1 < vchunks; c += 2) {
+    for (; c + 1 < run_chunks; c += 2) {
         int* const ip = (!kSum && c > 0) ? chunk_ints + (c - 1) : nullptr;
         // even chunk c -> acc0, ring slots 0 and 1; epilogue of chunk c-1 (acc1, scales qsb)
         BSI_I8_HORNER();
@@ -492,8 +569,8 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
             BSI_I8_SCALES(qsb, c + 1);
         }
     }
-    bool last_in_acc0 = false;
-    if (c < vchunks) {  // odd number of chunks: one more even chunk; its halves sit in slots 0 and 1
+    last_in_acc0 = false;
+    if (c < run_chunks) {  // odd number of chunks: one more even chunk; its halves sit in slots 0 and 1
         int* const ip = (!kSum && c > 0) ? chunk_ints + (c - 1) : nullptr;
         BSI_I8_HORNER();
         BSI_I8_CHUNK(0, 2, acc0, acc1, qsb, ip);
@@ -504,6 +581,86 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
     // one); nothing uses those operands
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     if (wave == 0) BSI_STAMP(kStampLoopDone);
+    if (!kSplit) break;
+    if (kSplit) {
+        // the chain step of the run's last chunk
+#pragma unroll
+        for (int a = 0; a < WM; ++a)
+#pragma unroll
+            for (int b = 0; b < WN; ++b)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int v = last_in_acc0 ? acc0[a][b][e] : acc1[a][b][e];
+                    accf[a][b][e] = fmaf(static_cast<float>(v), last_in_acc0 ? qsa[b] : qsb[b], accf[a][b][e]);
+                    peak = fmaxf(peak, fabsf(accf[a][b][e]));
+                }
+        if (pass > 0) break;  // the whole row in order: these are the sequential chain's values
+        typedef float v4f __attribute__((ext_vector_type(4)));
+        // (formed here, from values the compiler cannot see through, so that no address of the partial sums is
+        // computed ahead of the chunk loop and held in registers the loop has none to spare of)
+        int lane_late = lane, tile_late = by * tiles_x + bx;
+        asm volatile("" : "+v"(lane_late), "+s"(tile_late));
+        const size_t tile = static_cast<size_t>(tile_late);
+        constexpr size_t kWaveVecs = static_cast<size_t>(WM) * WN * 64;  // 16-byte pieces of an MFMA wave's outputs
+        v4f* const parts = reinterpret_cast<v4f*>(split_partials) + tile * nseg * (C::kConsumers * kWaveVecs);
+        {
+            v4f* mine = parts + (static_cast<size_t>(seg) * C::kConsumers + wave) * kWaveVecs + lane_late;
+#pragma unroll
+            for (int a = 0; a < WM; ++a)
+#pragma unroll
+                for (int b = 0; b < WN; ++b)
+                    __builtin_nontemporal_store((v4f){accf[a][b][0], accf[a][b][1], accf[a][b][2], accf[a][b][3]},
+                                                mine + (a * WN + b) * 64);
+        }
+        const int wave_over = (__builtin_amdgcn_ballot_w64(!(peak <= split_limit)) != 0) ? 1 : 0;  // any lane of the wave
+        if (lane == 0) split_flags[wave] = wave_over;
+        // This wave's partial sums have reached the L2 (stores are counted down once the L2 has them).  One lane of
+        // the workgroup then makes the whole workgroup's stores visible to the device (a release fence writes back
+        // the L2's dirty lines, whichever wave wrote them) before it counts the workgroup in: one write-back per
+        // workgroup.  Fences from every wave, and fences that also invalidate, cost the launch ten times the split's gain.
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        lds_barrier();
+        if (wave == 0 && lane == 0) {
+            unsigned any = 0;
+            for (int w = 0; w < C::kConsumers; ++w) any |= static_cast<unsigned>(split_flags[w]);
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+            const unsigned old = __hip_atomic_fetch_add(split_counters + tile, 1u + (any ? 0x10000u : 0u), __ATOMIC_RELAXED,
+                                                        __HIP_MEMORY_SCOPE_AGENT);
+            int decision = kSplitLeave;
+            if ((old & 0xFFFFu) == static_cast<unsigned>(nseg - 1)) {  // the tile's last workgroup
+                // what the other workgroups stored before they counted themselves in, not what this CU's caches
+                // may hold of an earlier launch: the invalidation is the CU's, so it serves the waves that load
+                // behind the barrier below
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+                decision = ((old >> 16) != 0 || any != 0) ? kSplitRedo : kSplitCombine;
+                __hip_atomic_store(split_counters + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
+                // running totals behind the tile counters: tiles combined, tiles computed again
+                __hip_atomic_fetch_add(split_counters + kSplitMaxTiles + (decision == kSplitRedo ? 1 : 0), 1u,
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            split_flags[15] = decision;
+        }
+        lds_barrier();
+        const int decision = __builtin_amdgcn_readfirstlane(split_flags[15]);
+        if (decision == kSplitLeave) return;
+        if (decision == kSplitCombine) {
+            for (int sg = 0; sg < nseg; ++sg) {
+                if (sg == seg) continue;
+                const v4f* theirs = parts + (static_cast<size_t>(sg) * C::kConsumers + wave) * kWaveVecs + lane_late;
+#pragma unroll
+                for (int a = 0; a < WM; ++a)
+#pragma unroll
+                    for (int b = 0; b < WN; ++b) {
+                        const v4f v = __builtin_nontemporal_load(theirs + (a * WN + b) * 64);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) accf[a][b][e] += v[e];  // exact: see the head of the kernel
+                    }
+            }
+            break;
+        }
+        run_chunks = chunks;  // kSplitRedo: the loader waves fill the ring from chunk 0 again
+    }
+    }  // passes
 #undef BSI_I8_HORNER
 #undef BSI_I8_CHUNK
 #undef BSI_I8_KSTEP
@@ -603,7 +760,8 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
         }
         return;
     }
-    // epilogue of the last chunk
+    // epilogue of the last chunk (a D-split launch has done it above)
+    if (!kSplit)
 #pragma unroll
     for (int a = 0; a < WM; ++a)
 #pragma unroll
@@ -760,7 +918,7 @@ __global__ __launch_bounds__((I8WCfg<WN>::kBlock)) void dot_mfma_i8w_kernel(
     unsigned char* const scale_lds = lds + 4 * C::kStage;
 
     if (wave >= W::kConsumers) {
-        i8_loader_wave<C, false>(lds, wave - W::kConsumers, lane, A8, qscale, qscale_stride, K8, Bw, Sb, chunks, halves, R, Q,
+        i8_loader_wave<C, false>(lds, wave - W::kConsumers, lane, A8, qscale, qscale_stride, K8, Bw, Sb, chunks, 0, halves, R, Q,
                                  r0, q0, rowbytes, bias, 1, 0, key_tiled, warm, warm_lines);
         return;
     }
@@ -943,11 +1101,42 @@ static void launch_mfma_i8_tm(const int8_t* A8, const float* qscale, int stride,
     using C = I8Cfg<TM, TN>;
     const dim3 grid(static_cast<unsigned>((R + TM - 1) / TM), static_cast<unsigned>((Q + TN - 1) / TN));
     static LdsOptIn once0;
-    lds_opt_in(once0, reinterpret_cast<const void*>(&dot_mfma_i8_kernel<TM, TN, kMode>), C::kLds);
-    hipLaunchKernelGGL((dot_mfma_i8_kernel<TM, TN, kMode>), grid, dim3(C::kBlock), C::kLds, st, A8, qscale, stride, K8,
+    lds_opt_in(once0, reinterpret_cast<const void*>(&dot_mfma_i8_kernel<TM, TN, kMode, false>), C::kLds);
+    hipLaunchKernelGGL((dot_mfma_i8_kernel<TM, TN, kMode, false>), grid, dim3(C::kBlock), C::kLds, st, A8, qscale, stride, K8,
                        Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias, ndig, dig_stride,
                        key_indices, key_tiled, static_cast<const unsigned char*>(g_warm_ptr),
-                       static_cast<long long>(g_warm_bytes / 128), stream_output());
+                       static_cast<long long>(g_warm_bytes / 128), stream_output(), static_cast<float*>(nullptr),
+                       static_cast<unsigned*>(nullptr), 0.0f, 0);
+}
+
+// The D-split launch of the chain mode: `segments` workgroups per output tile, each over its own run of chunks (see
+// the head of dot_mfma_i8_kernel).  scratch: the calling thread's attached split scratch (counters, then partial sums).
+template <int TM, int TN>
+static void launch_mfma_i8_split(int segments, unsigned char* scratch, const int8_t* A8, const float* qscale, int stride,
+                                 const int8_t* K8, const float* Bw, int Sb, int chunks, int64_t R, int64_t Q, int down_shift,
+                                 float scale_inv, int64_t R_total, float* out, const float* bias, hipStream_t st,
+                                 int key_tiled) {
+    using C = I8Cfg<TM, TN>;
+    const int tiles_x = static_cast<int>((R + TM - 1) / TM), tiles_y = static_cast<int>((Q + TN - 1) / TN);
+    unsigned workgroups = static_cast<unsigned>(tiles_x * tiles_y * segments);
+    if (segments == 2 || segments == 4 || segments == 8) {  // rounds of 8: see the decoding at the head of the kernel
+        const int per = 8 / segments;
+        workgroups = static_cast<unsigned>(8 * ((tiles_x + per - 1) / per) * tiles_y);
+    }
+    const dim3 grid(workgroups);
+    const int split_shape = tiles_x | (tiles_y << 10) | (segments << 20);
+    // every segment's chain values stay at or below 2^(24 + down_shift) / segments (rounded down to a power of two)
+    int log2_segments = 0;
+    while ((1 << log2_segments) < segments) ++log2_segments;
+    const float limit = __builtin_ldexpf(1.0f, 24 + down_shift - log2_segments);
+    static LdsOptIn once0;
+    lds_opt_in(once0, reinterpret_cast<const void*>(&dot_mfma_i8_kernel<TM, TN, kI8Chain, true>), C::kLdsSplit);
+    hipLaunchKernelGGL((dot_mfma_i8_kernel<TM, TN, kI8Chain, true>), grid, dim3(C::kBlock), C::kLdsSplit, st, A8, qscale,
+                       stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, static_cast<int*>(nullptr), bias,
+                       1, 0LL, static_cast<const long long*>(nullptr), key_tiled,
+                       static_cast<const unsigned char*>(g_warm_ptr), static_cast<long long>(g_warm_bytes / 128),
+                       stream_output(), reinterpret_cast<float*>(scratch + kSplitCounterBytes),
+                       reinterpret_cast<unsigned*>(scratch), limit, split_shape);
 }
 
 // Sum mode (ndig >= 1 digit images of the queries; int32 sums into chunk_ints when given, else the float epilogue)
@@ -1013,10 +1202,90 @@ int choose_i8_tile(int64_t R, int64_t Q, int64_t* cost_out) {
     return tiles[best];
 }
 
+// D-split choice for a chain-mode call whose grid leaves most CUs idle: the 128 x 128 or 128 x 64 tile with `segments`
+// workgroups per tile over runs of chunks, if the calling thread has attached a scratch region that holds the
+// partial sums and the modelled time beats the best unsplit tile.  The model, in microseconds, from measurements on
+// the MI355X: a workgroup's half-chunk costs 0.0045 us per unit of choose_i8_tile's scale; the partial sums' way
+// through memory (stores, one write-back fence per workgroup, the counter, the last workgroup's loads) costs about
+// 2 + 0.9 x segments + 0.5 per MiB of partial sums.  That overhead is why shapes like Q512 x R2048 x D8192 stay
+// unsplit (16.3 us on 64 x 64 tiles against 22.6 - 26.5 split), and why grids of a few tiles over long rows split
+// (Q128 x R512 x D16384: 20.0 -> 13.6 us; Q64 x R256 x D32768: 37.0 -> 17.3; Q256 x R1024 x D16384: 24.9 -> 18.3).
+// Returns the tile (128 or 12864) and sets *segments, or 0 for no split.  g_i8_split: 0 = by this model, 1 = never,
+// n >= 2 = n segments on the forced tile (g_i8_tile 128 or 12864; 128 x 128 otherwise) whenever the scratch allows it.
+thread_local unsigned char* t_split_scratch = nullptr;
+thread_local size_t t_split_bytes = 0;
+thread_local int t_split_device = -1;
+std::atomic<int> g_i8_split{0};
+constexpr double kCostUnitUs = 0.0045;
+constexpr int kSplitMinChunks = 2;  // chunks per segment at least
+constexpr int kSplitMaxSegments = 64;
+
+static size_t split_scratch_need(int64_t tiles, int segments, int TM, int TN) {
+    return kSplitCounterBytes + static_cast<size_t>(tiles) * segments * TM * TN * sizeof(float);
+}
+
+int choose_i8_split(int64_t R, int64_t Q, int chunks, int* segments) {
+    *segments = 1;
+    const int mode = g_i8_split.load(std::memory_order_relaxed);
+    if (mode == 1 || t_split_scratch == nullptr) return 0;
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev != t_split_device) return 0;
+    const int64_t kr = (R + 127) / 128;
+    const int64_t tiles_of[2] = {kr * ((Q + 127) / 128), kr * ((Q + 63) / 64)};
+    const int tile_id[2] = {128, 12864}, tn_of[2] = {128, 64}, unit[2] = {100, 63};
+    if (mode >= 2) {
+        const int forced = g_i8_tile.load(std::memory_order_relaxed);
+        const int i = forced == 12864 ? 1 : 0;
+        const int seg = mode < chunks ? mode : chunks;
+        if (seg < 2 || tiles_of[i] > kSplitMaxTiles || split_scratch_need(tiles_of[i], seg, 128, tn_of[i]) > t_split_bytes) return 0;
+        *segments = seg;
+        return tile_id[i];
+    }
+    if (tiles_of[0] >= 128) return 0;  // half the GPU busy on the large tile: nothing to gain
+    int64_t unsplit = 0;
+    (void)choose_i8_tile(R, Q, &unsplit);
+    double best_us = kCostUnitUs * static_cast<double>(unsplit) * chunks * 2;
+    int best = 0;
+    for (int i = 0; i < 2; ++i) {
+        const int64_t n = tiles_of[i];
+        if (n > 128) continue;
+        int max_seg = static_cast<int>(256 / n);
+        if (max_seg > kSplitMaxSegments) max_seg = kSplitMaxSegments;
+        if (max_seg > chunks / kSplitMinChunks) max_seg = chunks / kSplitMinChunks;
+        for (int seg = 2; seg <= max_seg; ++seg) {
+            const size_t need = split_scratch_need(n, seg, 128, tn_of[i]);
+            if (need > t_split_bytes) break;
+            const int64_t run = (chunks + seg - 1) / seg;  // chunks of the longest segment
+            const double us = kCostUnitUs * unit[i] * static_cast<double>(run) * 2 + 2.0 + 0.9 * seg +
+                              0.5 * static_cast<double>(need - kSplitCounterBytes) / (1 << 20);
+            if (us < best_us) {
+                best_us = us;
+                best = tile_id[i];
+                *segments = seg;
+            }
+        }
+    }
+    return best;
+}
+
 void launch_mfma_i8(const int8_t* A8, const float* qscale, int stride, const int8_t* K8, const float* Bw, int Sb,
                            int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv, int64_t R_total,
                            float* out, int32_t* chunk_ints, const float* bias, hipStream_t st, int key_tiled,
                            int ndig, long long dig_stride, const long long* key_indices) {
+    if (ndig == 0 && chunk_ints == nullptr) {
+        int segments = 1;
+        const int split_tile = choose_i8_split(R, Q, chunks, &segments);
+        if (split_tile == 128) {
+            launch_mfma_i8_split<128, 128>(segments, t_split_scratch, A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift,
+                                           scale_inv, R_total, out, bias, st, key_tiled);
+            return;
+        }
+        if (split_tile == 12864) {
+            launch_mfma_i8_split<128, 64>(segments, t_split_scratch, A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift,
+                                          scale_inv, R_total, out, bias, st, key_tiled);
+            return;
+        }
+    }
     const int tile = choose_i8_tile(R, Q);
     if (tile == 1284 && ndig == 0) {
         launch_mfma_i8w<4>(A8, qscale, stride, K8, Bw, Sb, chunks, R, Q, down_shift, scale_inv, R_total, out, chunk_ints, bias,

@@ -28,6 +28,17 @@ extern thread_local size_t g_warm_bytes;
 // Set by the entry points of a linear layer around their launch: the next kernel of the model reads that output.
 extern thread_local int t_layer_output;
 int choose_i8_tile(int64_t R, int64_t Q, int64_t* cost_out = nullptr);
+// D-split of the chain-mode int8-image dot (bsi_hip_dot_attach_split_scratch): the calling thread's scratch region
+// (counters of kSplitCounterBytes, then the segments' partial sums) and the device it lies on; the option
+// BSI_OPT_I8_SPLIT; the choice itself (tile 128 / 12864 and *segments, or 0).
+constexpr size_t kSplitCounterBytes = BSI_SPLIT_COUNTER_BYTES;
+constexpr int64_t kSplitMaxTiles = BSI_SPLIT_MAX_TILES;  // then two running totals (BSI_SPLIT_STAT_*)
+static_assert((kSplitMaxTiles + 2) * sizeof(unsigned) <= kSplitCounterBytes, "counters and totals fit their area");
+extern thread_local unsigned char* t_split_scratch;
+extern thread_local size_t t_split_bytes;
+extern thread_local int t_split_device;
+extern std::atomic<int> g_i8_split;
+int choose_i8_split(int64_t R, int64_t Q, int chunks, int* segments);
 void launch_mfma_i8(const int8_t* A8, const float* qscale, int stride, const int8_t* K8, const float* Bw, int Sb,
                     int chunks, int64_t R, int64_t Q, int down_shift, float scale_inv, int64_t R_total, float* out,
                     int32_t* chunk_ints, const float* bias, hipStream_t st,

@@ -188,6 +188,9 @@ int bsi_hip_planes_to_int8_tiled(const uint64_t* words_device, int64_t rows, int
                                    in the caches for the next kernel), 2 = nontemporal stores (it leaves them as it is
                                    written); 0 (default) = plain from the linear-layer entry points (bsi_hip_dot_bias,
                                    bsi_hip_dot_bias_warm, bsi_hip_linear), nontemporal from the other dot entry points */
+#define BSI_OPT_I8_SPLIT 5 /* D-split of the int8-image dot (see bsi_hip_dot_attach_split_scratch): 1 = never, n >= 2 = n
+                              segments (on the tile BSI_OPT_I8_TILE forces, 128 or 12864; 128 otherwise) whenever the
+                              attached scratch holds them; 0 (default) = chosen per call by a cost model */
 int bsi_hip_set_option(int option, int value);
 
 /* Bytes of device workspace bsi_hip_dot needs for this shape and core (0 when none). */
@@ -215,6 +218,38 @@ int bsi_hip_dot(const uint64_t* A, const int8_t* A_ints8, const float* A_chunk_s
                 int W64, const uint64_t* B, int b_layout, const float* Bw, int Sb, int64_t R, int64_t Q,
                 float scale_inv, int64_t R_total, float* out, int32_t* chunk_ints, int core, void* workspace,
                 size_t workspace_bytes, void* stream);
+
+/*
+ * D-split of the int8-image dot.  A call of a few hundred query rows against a few thousand keys has fewer output
+ * tiles of 128 x 128 than the GPU has CUs; smaller tiles fill the GPU but move twice the operand bytes per
+ * multiply-add into the CUs.  With a scratch region attached, such a call runs the large tile with several
+ * workgroups per output tile, each over its own run of chunks, and the tile's last workgroup adds the partial sums.
+ * The result is the one sequential chunk chain of bsi_cuda_kernels_dot.cuh:1516-1540 bit for bit, not within a
+ * tolerance: every operand of the chain is an integer times one power of two, so a chain whose values all stay below
+ * 2^24 units never rounds and equals the exact sum in any order of addition; every workgroup measures the largest
+ * magnitude its chain values take, and a tile whose segments do not all stay below 2^24 / segments units is computed
+ * again by its last workgroup over all chunks in order.  No counterpart in the reference, whose grid is one workgroup
+ * per 32 x 32 output tile (bsi_cuda_kernels_dot.cuh:2780-2993).
+ *
+ * bsi_hip_dot_attach_split_scratch names the region the CALLING THREAD's later dots (every entry point that reaches
+ * the int8-image kernel: bsi_hip_dot, _bias, _bias_warm, _timed, bsi_hip_linear, bsi_hip_dot_ewah_batch) may use on
+ * the current device; NULL / 0 detaches.  The region is `bytes` of device memory, 256-byte aligned, whose first
+ * BSI_SPLIT_COUNTER_BYTES are ZERO when it is attached for the first time (hipMemset once after hipMalloc); every
+ * launch that completes leaves them zero.  bsi_hip_dot_split_scratch_bytes() is the size that serves every shape the
+ * choice can make.  Launches that use one region must not overlap on the GPU (one region per stream).
+ */
+#define BSI_SPLIT_COUNTER_BYTES 4096
+/* Layout of those bytes, as uint32 words: one counter per output tile (a split launch has at most BSI_SPLIT_MAX_TILES
+ * tiles), then two running totals that the kernels only ever add to: output tiles whose partial sums were added, and
+ * output tiles that were computed again in chunk order (a caller may read or clear the totals between launches). */
+#define BSI_SPLIT_MAX_TILES 1008
+#define BSI_SPLIT_STAT_COMBINED 1008
+#define BSI_SPLIT_STAT_RECOMPUTED 1009
+size_t bsi_hip_dot_split_scratch_bytes(void);
+int bsi_hip_dot_attach_split_scratch(void* scratch_device, size_t bytes);
+/* What a chain-mode int8-image dot of this shape would do on the calling thread right now: *tile = 128 or 12864 and
+ * *segments >= 2 for a D-split launch, *tile = the unsplit tile and *segments = 1 otherwise.  Host only. */
+int bsi_hip_dot_split_plan(int64_t R, int64_t Q, int W64, int* tile, int* segments);
 
 /* bsi_hip_dot on the matrix cores for callers that cannot allocate device memory or hold a workspace of their own
  * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
