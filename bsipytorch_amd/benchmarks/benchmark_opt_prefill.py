@@ -118,6 +118,69 @@ def time_forward(model, input_ids, iters: int, warmup: int):
     return times[len(times) // 2], times[0]
 
 
+@torch.no_grad()
+def kernel_time_of_dots_and_builds(model, input_ids, replays: int = 5):
+    """(dot ms, query-build ms) per forward as GPU time without any synchronisation in between: every BSI layer's dot
+    -- on the activations the layer sees in this forward, with its bias and its warm-up of the next keyset as the
+    forward launches it -- recorded into one HIP graph and replayed, and the query builds likewise (layers fed the
+    same tensor share one build, as in the forward).  Per-call device events (BSI_PROFILE=1) synchronise after every
+    call and so charge each dot its launch latency as well; these figures do not."""
+    from bsipytorch_amd import bsi_ops, linear
+
+    layers = [m for m in model.modules() if isinstance(m, linear.BSIQuantizedLinear)]
+    seen = {}
+
+    def note_input(mod, args):
+        seen[id(mod)] = args[0]  # kept alive, so that no later tensor takes its address
+
+    hooks = [m.register_forward_pre_hook(note_input) for m in layers]
+    model(input_ids)
+    for h in hooks:
+        h.remove()
+    builds, dots, groups_done, prev = [], [], set(), None
+    for m in layers:
+        x = seen[id(m)]
+        x2d = x.reshape(-1, x.shape[-1]).detach().contiguous()
+        fused = m.__dict__.get("_fused")
+        if fused is not None:
+            group = fused[0]
+            if id(group) in groups_done:
+                continue
+            groups_done.add(id(group))
+            keys, bias, nxt = group.keys, group.bias, group.next_layer
+        else:
+            keys, bias, nxt = m._bsi_keys_cuda, m.bias, m.__dict__.get("_next_bsi_layer")
+        thr = float(m.query_compress_threshold)
+        if x is not prev:
+            builds.append(lambda x2d=x2d, dec=m.decimalPlaces, thr=thr: bsi_ops.build_bsi_queries_cuda_batch_packed(x2d, dec, thr))
+        prev = x
+        qcap = bsi_ops.build_bsi_queries_cuda_batch_packed(x2d, m.decimalPlaces, thr)
+        b = bsi_ops.device_bias(bias, x2d.device) if (bias is not None and x.dtype == torch.float32) else None
+        dots.append(lambda q=qcap, k=keys, b=b, w=linear._keys_to_warm(nxt):
+                    bsi_ops.batch_dot_product_multiquery_cuda_batch_caps(q, k, b, w))
+
+    def replayed_ms(launches):
+        for f in launches:  # once eagerly: workspaces and scratch regions exist before the capture
+            f()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            kept = [f() for f in launches]  # the outputs stay allocated while the graph lives
+        times = []
+        for _ in range(replays + 1):
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            g.replay()
+            e.record()
+            torch.cuda.synchronize()
+            times.append(s.elapsed_time(e))
+        del kept
+        times = sorted(times[1:])
+        return times[len(times) // 2]
+
+    return replayed_ms(dots), replayed_ms(builds), len(dots), len(builds)
+
+
 def run(model_name="opt-1.3b", seq_len=512, batch=1, iters=5, warmup=2, decimal_places=2, compress_threshold=0.5,
         seed=123, dense=True, graph=True, fuse_qkv=False, quantize_lm_head=False):
     from bsipytorch_amd import bsi_ops, linear
@@ -181,7 +244,16 @@ def run(model_name="opt-1.3b", seq_len=512, batch=1, iters=5, warmup=2, decimal_
             res["bsi_graph_tokens_per_s"] = tokens / (times[len(times) // 2] * 1e-3)
             res["graph_replays_match_eager"] = same
 
-    # pass 2: per-call device events on the dot and the builder -> shares
+    # pass 2a: GPU time of the dots and of the query builds by themselves, unsynchronised -> the shares of the forward
+    if graph and bsi_ops._flags()["bits_q"] != 0 and res.get("bsi_graph_fwd_ms"):
+        dot_gpu_ms, build_gpu_ms, n_dots, n_builds = kernel_time_of_dots_and_builds(model, input_ids)
+        res["dot_gpu_ms_per_prefill"] = dot_gpu_ms
+        res["query_build_gpu_ms_per_prefill"] = build_gpu_ms
+        res["dot_launches_per_prefill"], res["query_builds_per_prefill"] = n_dots, n_builds
+        res["dot_share_of_graph_fwd"] = dot_gpu_ms / res["bsi_graph_fwd_ms"]
+        res["query_build_share_of_graph_fwd"] = build_gpu_ms / res["bsi_graph_fwd_ms"]
+
+    # pass 2: per-call device events on the dot and the builder (each call synchronised, so launch latency is in)
     os.environ["BSI_PROFILE"] = "1"
     bsi_ops._reset_flag_cache()
     time_forward(model, input_ids, 1, 1)

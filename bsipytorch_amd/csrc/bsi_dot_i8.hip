@@ -401,28 +401,18 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    // Which tile (and, in a D-split launch, which segment) this workgroup computes.  A D-split launch is a 1-D grid
-    // decoded so that -- workgroups being dealt to the eight XCDs in turn -- an XCD gets one segment of a few key
-    // tiles for all query tiles: its L2 then fetches that run of chunks of those key rows and of all query rows
-    // once, as in an unsplit launch of a short row, instead of every segment of whole rows.
+    // Which tile (and, in a D-split launch, which segment) this workgroup computes.  A D-split launch is a 1-D grid:
+    // key tile fastest, then query tile, then segment, so that workgroups which share a key tile and a run of chunks
+    // are neighbours (a grid that gave every XCD one segment of a few key tiles was measured and is slower).
     int bx = static_cast<int>(blockIdx.x), by = static_cast<int>(blockIdx.y), seg = 0, nseg = 1, tiles_x = static_cast<int>(gridDim.x);
     if (kSplit) {
         tiles_x = split_shape & 1023;
         const int tiles_y = (split_shape >> 10) & 1023;
         nseg = split_shape >> 20;
         const int id = static_cast<int>(blockIdx.x);
-        if (nseg == 2 || nseg == 4 || nseg == 8) {
-            const int per = 8 / nseg, slot = id & 7, rest = id >> 3;   // key tiles of one segment per round of 8 workgroups
-            const int xh_count = (tiles_x + per - 1) / per;
-            seg = slot / per;
-            bx = (rest % xh_count) * per + slot % per;
-            by = rest / xh_count;
-        } else {
-            bx = id % tiles_x;
-            by = (id / tiles_x) % tiles_y;
-            seg = id / (tiles_x * tiles_y);
-        }
-        if (bx >= tiles_x || by >= tiles_y || seg >= nseg) return;  // padding of the last round
+        bx = id % tiles_x;
+        by = (id / tiles_x) % tiles_y;
+        seg = id / (tiles_x * tiles_y);
     }
     const int64_t r0 = static_cast<int64_t>(bx) * TM;
     const int64_t q0 = static_cast<int64_t>(by) * TN;
@@ -1118,12 +1108,7 @@ static void launch_mfma_i8_split(int segments, unsigned char* scratch, const int
                                  int key_tiled) {
     using C = I8Cfg<TM, TN>;
     const int tiles_x = static_cast<int>((R + TM - 1) / TM), tiles_y = static_cast<int>((Q + TN - 1) / TN);
-    unsigned workgroups = static_cast<unsigned>(tiles_x * tiles_y * segments);
-    if (segments == 2 || segments == 4 || segments == 8) {  // rounds of 8: see the decoding at the head of the kernel
-        const int per = 8 / segments;
-        workgroups = static_cast<unsigned>(8 * ((tiles_x + per - 1) / per) * tiles_y);
-    }
-    const dim3 grid(workgroups);
+    const dim3 grid(static_cast<unsigned>(tiles_x * tiles_y * segments));
     const int split_shape = tiles_x | (tiles_y << 10) | (segments << 20);
     // every segment's chain values stay at or below 2^(24 + down_shift) / segments (rounded down to a power of two)
     int log2_segments = 0;

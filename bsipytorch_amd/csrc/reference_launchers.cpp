@@ -17,6 +17,7 @@
 #include <cstdio>
 #include <mutex>
 #include <string>
+#include <vector>
 
 #include "../../include/bsi_hip.h"
 
@@ -84,9 +85,96 @@ int workspace_for(size_t need, hipStream_t stream, void** ptr, size_t* bytes) {
     return BSI_OK;
 }
 
+// ---- keysets registered for the fast dot
+//
+// The reference hands the dot launcher canonical key planes (bsi_cuda.cpp:724-746), which the library can only run on
+// its plane-reading kernel.  A ROCm build of the reference registers a keyset once, after building it
+// (build_bsi_keys_cuda, bsi_cuda.cpp:863-910): the int8 image of the same integers is derived into memory this module
+// owns, and every later dot on those planes contracts the image instead -- the library's compute-bound kernel, the
+// planes and the results unchanged.  The query side is remembered the same way: launch_quantize_shift_pack_chunk_batch
+// also derives the int8 image of the planes it has just packed (one more launch in the build, none in the dot), and the
+// dot finds it by the planes' address.
+struct RegisteredKeys {
+    const void* planes;
+    int R, Sb, W, device;
+    int8_t* image;
+};
+std::mutex g_keys_mutex;
+std::vector<RegisteredKeys> g_keys;
+
+struct QueryImage {  // per device: the int8 image of the query planes packed last
+    const void* planes = nullptr;
+    int64_t Q = 0;
+    int Sa = 0, W = 0;
+    int8_t* image = nullptr;
+    size_t bytes = 0;
+};
+QueryImage g_query_image[64];
+
+// Every other launcher that writes plane words: whatever image is remembered may describe planes that are being
+// replaced at the same address.
+void forget_query_image() {
+    int dev = 0;
+    if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64) g_query_image[dev].planes = nullptr;
+}
+
+const int8_t* registered_key_image(const void* planes, int R, int Sb, int W) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+    std::lock_guard<std::mutex> lock(g_keys_mutex);
+    for (const RegisteredKeys& k : g_keys)
+        if (k.planes == planes && k.R == R && k.Sb == Sb && k.W == W && k.device == dev) return k.image;
+    return nullptr;
+}
+
 }  // namespace
 
 extern "C" {
+
+int bsi_launchers_forget_keys(const unsigned long long* B);
+
+int bsi_launchers_register_keys(const unsigned long long* B, int R, int Sb, int W, hipStream_t stream) {
+    static const char* kName = "bsi_launchers_register_keys";
+    if (B == nullptr || R <= 0 || W <= 0 || Sb < 2 || Sb > 8) {
+        note_msg(kName, BSI_ERR_INVALID, "needs key planes [R, Sb, W] with 2 <= Sb <= 8");
+        return BSI_ERR_INVALID;
+    }
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return BSI_ERR_HIP;
+    (void)bsi_launchers_forget_keys(B);  // planes built anew at an address registered before
+    int8_t* image = nullptr;
+    const size_t bytes = static_cast<size_t>(R) * static_cast<size_t>((W + 3) / 4) * 256;
+    if (hipMalloc(reinterpret_cast<void**>(&image), bytes) != hipSuccess) {
+        note_msg(kName, BSI_ERR_HIP, "could not allocate the int8 key image");
+        return BSI_ERR_HIP;
+    }
+    const int rc = bsi_hip_planes_to_int8(reinterpret_cast<const uint64_t*>(B), R, Sb, W, image, stream);
+    if (rc != BSI_OK) {
+        (void)hipFree(image);
+        note(kName, rc);
+        return rc;
+    }
+    std::lock_guard<std::mutex> lock(g_keys_mutex);
+    g_keys.push_back(RegisteredKeys{B, R, Sb, W, dev, image});
+    return BSI_OK;
+}
+
+// Forgets the keyset registered for these planes (when the reference's keyset capsule is destroyed).  The image is
+// freed, which waits for work in flight on the device, so: not while a stream is being captured.
+int bsi_launchers_forget_keys(const unsigned long long* B) {
+    int8_t* image = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(g_keys_mutex);
+        for (size_t i = 0; i < g_keys.size(); ++i)
+            if (g_keys[i].planes == B) {
+                image = g_keys[i].image;
+                g_keys.erase(g_keys.begin() + static_cast<long>(i));
+                break;
+            }
+    }
+    if (image == nullptr) return BSI_OK;
+    return hipFree(image) == hipSuccess ? BSI_OK : BSI_ERR_HIP;
+}
 
 int bsi_launchers_last_status(void) { return t_status; }
 const char* bsi_launchers_last_error(void) { return t_error.c_str(); }
@@ -98,6 +186,7 @@ void bsi_launchers_clear_status(void) {
 // ---- bsi_cuda.cpp:29-57
 
 void launch_ewah_decompress(const unsigned long long* in, int in_len, int W, unsigned long long* out, hipStream_t stream) {
+    forget_query_image();
     note("launch_ewah_decompress", bsi_hip_ewah_decompress(reinterpret_cast<const uint64_t*>(in), in_len, W,
                                                            reinterpret_cast<uint64_t*>(out), stream));
 }
@@ -133,6 +222,29 @@ void launch_popcount_weighted_keys_literal_fused_multiq(const unsigned long long
         return;
     }
     const int core = (Sa >= 2 && Sa <= 8 && Sb >= 2 && Sb <= 8) ? BSI_CORE_MFMA : BSI_CORE_VALU;
+    if (core == BSI_CORE_MFMA && Q > 32) {  // up to 32 rows the library streams the planes, which is the faster read there
+        if (const int8_t* image = registered_key_image(B, R, Sb, W)) {
+            int dev = 0;
+            const int8_t* a8 = nullptr;
+            if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64) {
+                const QueryImage& qi = g_query_image[dev];
+                if (qi.planes == A && qi.Q == Q && qi.Sa == Sa && qi.W == W) a8 = qi.image;
+            }
+            if (a8 != nullptr) {
+                note(kName, bsi_hip_dot(reinterpret_cast<const uint64_t*>(A), a8, A_chunk_scales, A_scale_stride, Sa, W,
+                                        reinterpret_cast<const uint64_t*>(image), BSI_LAYOUT_INT8, Bw, Sb, R, Q, scale_inv,
+                                        R_total, out_global, nullptr, core, nullptr, 0, stream));
+                return;
+            }
+            const size_t qneed = bsi_hip_dot_workspace_bytes(Q, W, core);
+            if (qneed <= BSI_STATIC_SCRATCH_BYTES) {
+                note(kName, bsi_hip_dot_static_scratch(reinterpret_cast<const uint64_t*>(A), A_chunk_scales, A_scale_stride,
+                                                       Sa, W, reinterpret_cast<const uint64_t*>(image), BSI_LAYOUT_INT8, Bw,
+                                                       Sb, R, Q, scale_inv, R_total, out_global, nullptr, stream));
+                return;
+            }
+        }
+    }
     const size_t need = bsi_hip_dot_workspace_bytes(Q, W, core);
     if (need <= BSI_STATIC_SCRATCH_BYTES && core == BSI_CORE_MFMA) {
         note(kName, bsi_hip_dot_static_scratch(reinterpret_cast<const uint64_t*>(A), A_chunk_scales, A_scale_stride, Sa, W,
@@ -161,6 +273,7 @@ void launch_popcount_weighted_keys_literal_fused_multiq(const unsigned long long
 
 void launch_pack_bits_all_ballot(const long long* values, long long n, int slices, int words_per_slice,
                                  unsigned long long value_mask, unsigned long long* out, hipStream_t stream) {
+    forget_query_image();
     if (!mask_is_low_bits(value_mask, slices)) {
         note_msg("launch_pack_bits_all_ballot", BSI_ERR_UNSUPPORTED, "value_mask must be the low `slices` bits");
         return;
@@ -171,6 +284,7 @@ void launch_pack_bits_all_ballot(const long long* values, long long n, int slice
 
 void launch_pack_bits_all_ballot_batch(const long long* values, int Q, long long n, int slices, int words_per_slice,
                                        unsigned long long value_mask, unsigned long long* out, hipStream_t stream) {
+    forget_query_image();
     if (!mask_is_low_bits(value_mask, slices)) {
         note_msg("launch_pack_bits_all_ballot_batch", BSI_ERR_UNSUPPORTED, "value_mask must be the low `slices` bits");
         return;
@@ -225,6 +339,7 @@ void launch_compute_chunk_shift_scale_from_input(const void* input, int input_dt
 void launch_quantize_shift_pack_row_batch(const void* input, int input_dtype, int64_t Q, int64_t d, int slices,
                                           int words_per_slice, unsigned long long value_mask, double dec_scale, int fixed_bits,
                                           const int* shifts, unsigned long long* out, hipStream_t stream) {
+    forget_query_image();
     if (!mask_is_low_bits(value_mask, slices)) {
         note_msg("launch_quantize_shift_pack_row_batch", BSI_ERR_UNSUPPORTED, "value_mask must be the low `slices` bits");
         return;
@@ -237,13 +352,45 @@ void launch_quantize_shift_pack_row_batch(const void* input, int input_dtype, in
 void launch_quantize_shift_pack_chunk_batch(const void* input, int input_dtype, int64_t Q, int64_t d, int chunks, int slices,
                                             int words_per_slice, unsigned long long value_mask, double dec_scale,
                                             int fixed_bits, const int* shifts, unsigned long long* out, hipStream_t stream) {
+    forget_query_image();
     if (!mask_is_low_bits(value_mask, slices)) {
         note_msg("launch_quantize_shift_pack_chunk_batch", BSI_ERR_UNSUPPORTED, "value_mask must be the low `slices` bits");
         return;
     }
-    note("launch_quantize_shift_pack_chunk_batch",
-         bsi_hip_quantize_shift_pack_chunk_batch(input, input_dtype, Q, d, chunks, slices, words_per_slice, dec_scale, fixed_bits,
-                                                 shifts, reinterpret_cast<uint64_t*>(out), stream));
+    const int rc = bsi_hip_quantize_shift_pack_chunk_batch(input, input_dtype, Q, d, chunks, slices, words_per_slice, dec_scale,
+                                                           fixed_bits, shifts, reinterpret_cast<uint64_t*>(out), stream);
+    note("launch_quantize_shift_pack_chunk_batch", rc);
+    // The int8 image of these planes, for a dot against a registered keyset: kept per device, for the planes packed
+    // last.  Its buffer grows outside stream captures only; without it the dot derives the image itself.
+    int dev = 0;
+    if (rc != BSI_OK || slices < 2 || slices > 8 || hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return;
+    QueryImage& qi = g_query_image[dev];
+    qi.planes = nullptr;
+    bool any_keys;
+    {
+        std::lock_guard<std::mutex> lock(g_keys_mutex);
+        any_keys = !g_keys.empty();
+    }
+    if (!any_keys || Q <= 32) return;
+    const size_t bytes = static_cast<size_t>(Q) * static_cast<size_t>((words_per_slice + 3) / 4) * 256;
+    if (qi.bytes < bytes) {
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) return;
+        if (qi.image != nullptr) {
+            if (hipDeviceSynchronize() != hipSuccess) return;
+            (void)hipFree(qi.image);
+            qi.image = nullptr;
+            qi.bytes = 0;
+        }
+        const size_t size = (bytes + (size_t{1} << 20) - 1) & ~((size_t{1} << 20) - 1);
+        if (hipMalloc(reinterpret_cast<void**>(&qi.image), size) != hipSuccess) return;
+        qi.bytes = size;
+    }
+    if (bsi_hip_planes_to_int8(reinterpret_cast<const uint64_t*>(out), Q, slices, words_per_slice, qi.image, stream) != BSI_OK) return;
+    qi.planes = out;
+    qi.Q = Q;
+    qi.Sa = slices;
+    qi.W = words_per_slice;
 }
 
 void launch_slice_popcount_sum(const unsigned long long* words, int S, int W, unsigned long long* out_counts, hipStream_t stream) {

@@ -164,3 +164,62 @@ def test_reference_codec_sequence_through_the_launchers(launchers, oracle):
         torch.cuda.synchronize()
         np.testing.assert_array_equal(back.cpu().numpy().view(np.uint64), words[s])
     _ok(L)
+
+
+def test_registered_keys_take_the_int8_image_route(launchers, oracle):
+    """A keyset registered with bsi_launchers_register_keys: the reference's dot launcher, handed the same canonical
+    planes as before, contracts the int8 image derived at registration with the image of the query planes that the
+    chunk packer left -- same bits as the oracle, before and after the keyset is forgotten; planes rebuilt at the
+    same address by another launcher are not served from the remembered image."""
+    L = launchers
+    L.bsi_launchers_register_keys.argtypes, L.bsi_launchers_register_keys.restype = [vp, i32, i32, i32, vp], i32
+    L.bsi_launchers_forget_keys.argtypes, L.bsi_launchers_forget_keys.restype = [vp], i32
+    L.bsi_launchers_clear_status()
+    Q, R, d = 200, 300, 2048
+    W, chunks = d // 64, d // 256
+    rng = np.random.default_rng(77)
+    st = _st()
+    k = (rng.standard_normal((R, d)) * 0.02).astype(np.float32)
+    kb = oracle.build_keys(k)
+    B = torch.from_numpy(kb["words"].view(np.int64)).cuda()
+    Bw = torch.from_numpy(kb["slice_weights"]).cuda()
+    assert L.bsi_launchers_register_keys(B.data_ptr(), R, 6, W, st) == 0
+    Aw = torch.tensor([1, 2, 4, 8, 16, 32, -64], dtype=torch.float32, device="cuda").repeat(Q, 1).contiguous()
+    A = torch.empty((Q, 7, W), dtype=torch.int64, device="cuda")
+    qshift = torch.empty((Q, chunks), dtype=torch.int32, device="cuda")
+    qscale = torch.empty((Q, chunks), dtype=torch.float32, device="cuda")
+    scale_inv = float(np.float32(1.0 / 10.0 ** 4))
+
+    def build_and_dot(x):
+        xd = torch.from_numpy(x).cuda()
+        L.launch_compute_chunk_shift_scale_from_input(xd.data_ptr(), 0, Q, d, chunks, 100.0, 7, 0.0, qshift.data_ptr(),
+                                                      qscale.data_ptr(), st)
+        L.launch_quantize_shift_pack_chunk_batch(xd.data_ptr(), 0, Q, d, chunks, 7, W, 0x7F, 100.0, 7, qshift.data_ptr(),
+                                                 A.data_ptr(), st)
+        return dot()
+
+    def dot():
+        out = torch.zeros((Q, R), dtype=torch.float32, device="cuda")
+        L.launch_popcount_weighted_keys_literal_fused_multiq(A.data_ptr(), Aw.data_ptr(), qscale.data_ptr(), chunks, 7, W,
+                                                             B.data_ptr(), Bw.data_ptr(), 6, R, Q, 8, 4, None, None,
+                                                             scale_inv, R, out.data_ptr(), st)
+        torch.cuda.synchronize()
+        _ok(L)
+        return out.cpu().numpy()
+
+    def want(x):
+        qb = oracle.build_queries(x)
+        return oracle.dot_fixed(qb["words"], qb["scales"], kb["words"], kb["scales"], oracle.scale_inv(2, 2), want_ints=False)[1], qb
+
+    xs = [rng.standard_normal((Q, d)).astype(np.float32) for _ in range(2)]
+    for x in xs:  # two batches through the same buffers: the remembered image follows the packer
+        np.testing.assert_array_equal(build_and_dot(x), want(x)[0])
+    # the same planes address refilled by another launcher (packed from integers): the image of the earlier planes is not used
+    w2, qb2 = want(xs[0])
+    ints = torch.from_numpy(np.ascontiguousarray(qb2["ints"])).cuda()
+    L.launch_pack_bits_all_ballot_batch(ints.data_ptr(), Q, d, 7, W, 0x7F, A.data_ptr(), st)
+    qscale.copy_(torch.from_numpy(qb2["scales"]).cuda())
+    np.testing.assert_array_equal(dot(), w2)
+    assert L.bsi_launchers_forget_keys(B.data_ptr()) == 0
+    np.testing.assert_array_equal(build_and_dot(xs[1]), want(xs[1])[0])
+    assert L.bsi_launchers_forget_keys(B.data_ptr()) == 0   # forgetting twice is not an error
