@@ -53,6 +53,7 @@ PROTOTYPES = {
     "bsi_hip_tile_key_planes": [_vp, _i64, _i, _i, _vp, _vp],
     "bsi_hip_planes_to_int8": [_vp, _i64, _i, _i, _vp, _vp],
     "bsi_hip_set_option": [_i, _i],
+    "bsi_hip_stream_capture_id": [_vp, ctypes.POINTER(ctypes.c_ulonglong)],
     "bsi_hip_dot_workspace_bytes": [_i64, _i, _i],
     "bsi_hip_dot_split_scratch_bytes": [],
     "bsi_hip_dot_attach_split_scratch": [_vp, _sz],

@@ -19,6 +19,7 @@ code paths (``BSI_TC_DOT``, ``BSI_TC_TMA``, ``BSI_TC_CPASYNC``, ``BSI_TC_R_SWEEP
 """
 from __future__ import annotations
 
+import ctypes
 import json
 import os
 import sys
@@ -255,6 +256,15 @@ def tensor_build_key(t: torch.Tensor, *extra):
         return None
     f = _flags()
     return (t.data_ptr(), tuple(t.shape), t.dtype, t._version, f["bits_q"], f["chunk_scale"], f["clip_k"]) + extra
+
+
+def capture_id() -> int:
+    """Identifier of the graph capture the current stream is recording into, 0 when it is not capturing."""
+    if not _capturing():
+        return 0
+    cid = ctypes.c_ulonglong(0)
+    check(lib.bsi_hip_stream_capture_id(_stream(), ctypes.byref(cid)), "bsi_hip_stream_capture_id")
+    return int(cid.value)
 
 
 def _capsule(obj, cls, what: str):
@@ -1227,6 +1237,10 @@ def linear_cuda(x2d: torch.Tensor, keyset_cuda_cap, decimal_places: int, bias=No
             mine = ws["eager"][st] = (torch.empty((ws["bytes"],), dtype=torch.uint8, device=x2d.device), [None, None])
         buf, slot = mine
     key = tensor_build_key(x2d, int(decimal_places))
+    if capturing and key is not None:
+        # a build recorded by one capture is not part of another capture's graph: the capture's identifier is part
+        # of what a recorded launch may reuse (a second capture starting on the same static input builds anew)
+        key = key + (capture_id(),)
     rebuild = 0 if (key is not None and slot[0] == key) else 1
     slot[0], slot[1] = key, x2d  # holds the input, so that its address is not reused while the build stands for it
     wsptr = buf.data_ptr()

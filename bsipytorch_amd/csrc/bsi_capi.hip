@@ -108,6 +108,15 @@ static int time_launch(hipStream_t st, int reps, float* ms_best, F&& launch) {
 
 using namespace bsi;
 
+extern "C" int bsi_hip_stream_capture_id(void* stream, unsigned long long* id) {
+    BSI_REQUIRE(id != nullptr, "null pointer");
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    unsigned long long cid = 0;
+    BSI_HIP_CHECK(hipStreamGetCaptureInfo(bsi::as_stream(stream), &status, &cid));
+    *id = status == hipStreamCaptureStatusActive ? cid : 0;
+    return BSI_OK;
+}
+
 extern "C" const char* bsi_hip_version(void) { return "bsi_hip gfx950 0.1 (" __DATE__ ")"; }
 
 extern "C" const char* bsi_hip_last_error(void) { return last_error_ref().c_str(); }

@@ -33,7 +33,8 @@ def forget_shared_builds() -> None:
 
 def _cached_query_build(batch_inputs: torch.Tensor, decimal_places: int, threshold: float, packed: bool):
     use_cache = bsi_ops.fast_getenv("BSI_QUERY_CACHE", "1") != "0"
-    key = bsi_ops.tensor_build_key(batch_inputs, int(decimal_places), bool(packed)) if use_cache else None
+    # (the capture's identifier is part of the key: a build that one graph capture recorded is not part of another's)
+    key = bsi_ops.tensor_build_key(batch_inputs, int(decimal_places), bool(packed), bsi_ops.capture_id()) if use_cache else None
     use_cache = use_cache and key is not None  # a tensor without a version counter (inference mode) is built anew
     if use_cache and _last_query_build.get("key") == key and _last_query_build.get("src") is not None:
         return _last_query_build["cap"], True
@@ -207,7 +208,7 @@ class BSIQuantizedLinear(nn.Module):
         fp32 = original_dtype == torch.float32
         if fused is not None:
             group, start, stop = fused
-            key = bsi_ops.tensor_build_key(batch_inputs)
+            key = bsi_ops.tensor_build_key(batch_inputs, bsi_ops.capture_id())
             last = group.__dict__.get("_last_call")
             if last is not None and key is not None and last[0] == key:
                 scores, bias_done = last[2][:, start:stop], last[3]
@@ -257,7 +258,7 @@ class BSIQuantizedLinear(nn.Module):
         bsi_ops.reserve_linear_workspace(batch_inputs)  # a later capture of this forward may take the one-call path
         if fused is not None:
             group, start, stop = fused
-            key = bsi_ops.tensor_build_key(batch_inputs)
+            key = bsi_ops.tensor_build_key(batch_inputs, bsi_ops.capture_id())
             last = group.__dict__.get("_last_few")
             if last is not None and key is not None and last[0] == key:
                 scores, bias_done = last[2][:, start:stop], last[3]

@@ -53,6 +53,12 @@ const char* bsi_hip_last_error(void);
 /* Name of the device architecture (e.g. "gfx950"), CU count and LDS bytes per workgroup. */
 int bsi_hip_device_info(char* arch, int arch_len, int* cu_count, int* lds_bytes);
 
+/* The identifier of the graph capture `stream` is recording into (hipStreamGetCaptureInfo), 0 when it is not
+ * capturing.  Host-side callers that reuse work across launches (a query build shared by layers fed the same tensor)
+ * key that reuse by it: what one capture recorded is not part of another capture's graph.  No counterpart in the
+ * reference, which never records its launches. */
+int bsi_hip_stream_capture_id(void* stream, unsigned long long* id);
+
 /* ---------------------------------------------------------------- builder */
 
 /* out[i] = round_half_away((double)(float)x[i] * dec_scale).
@@ -258,7 +264,10 @@ int bsi_hip_dot_split_plan(int64_t R, int64_t Q, int W64, int* tile, int* segmen
  * hipMalloc / hipFree and no other allocating call.  Q * ceil(W64 / 4) * 256 must not exceed BSI_STATIC_SCRATCH_BYTES
  * (BSI_ERR_INVALID otherwise; bsi_hip_dot with a workspace has no such limit).  Every call on a GPU writes the same
  * array: calls that overlap on one GPU (two streams, two threads) race, calls on one stream do not.  Nothing in the
- * array has to start at zero: each call overwrites the part it reads.  Arguments and results as bsi_hip_dot. */
+ * array has to start at zero: each call overwrites the part it reads.  The FIRST call on a device (it looks the
+ * array's address up) and the first call of each kernel it selects (the kernel's one-time LDS opt-in and code
+ * load) do host-side set-up that a stream capture must not see: make one call of the same shape class (same key
+ * layout, Q above or up to 32) outside the capture before recording it.  Arguments and results as bsi_hip_dot. */
 #define BSI_STATIC_SCRATCH_BYTES (8u << 20)
 int bsi_hip_dot_static_scratch(const uint64_t* A, const float* A_chunk_scales, int A_scale_stride, int Sa, int W64,
                                const uint64_t* B, int b_layout, const float* Bw, int Sb, int64_t R, int64_t Q,

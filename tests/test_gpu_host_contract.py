@@ -263,3 +263,35 @@ def test_graphed_forward_refuses_what_cannot_be_recorded(ops, monkeypatch):
         ops._reset_flag_cache()
     with torch.no_grad():
         assert torch.equal(linear.GraphedForward(model, x)(x), model(x))
+
+
+@pytest.mark.parametrize("fuse", [False, True])
+def test_a_second_capture_on_the_same_static_input_builds_anew(ops, fuse):
+    """Two graphs recorded by hand, one after the other, with no forget_shared_builds() in between, the second starting
+    on the tensor the first ended on (same address, shape and version): the second graph carries its own query build,
+    so its replays follow what is copied into the static input."""
+    from bsipytorch_amd import linear
+
+    torch.manual_seed(17)
+    model = torch.nn.ModuleDict({n: torch.nn.Linear(512, 128).cuda() for n in ("q_proj", "k_proj", "v_proj")})
+    linear.quantize_model_bsi(model, decimalPlaces=2, compress_threshold=0.5, verbose=False, fuse_qkv=fuse)
+    x0, x1 = torch.randn(96, 512, device="cuda"), torch.randn(96, 512, device="cuda")
+    with torch.no_grad():
+        want0 = [model[n](x0).clone() for n in ("q_proj", "k_proj", "v_proj")]
+        want1 = [model[n](x1).clone() for n in ("q_proj", "k_proj", "v_proj")]
+        static_x = x0.clone()
+        fwd = lambda: [model[n](static_x) for n in ("q_proj", "k_proj", "v_proj")]  # noqa: E731
+        g1, out1 = _capture(fwd, fwd)
+        g2, out2 = _capture(fwd, lambda: None)   # nothing in between: same storage, same version counter
+        static_x.copy_(x1)
+        g2.replay()
+        torch.cuda.synchronize()
+        for got, want in zip(out2, want1):
+            assert torch.equal(got, want)
+        static_x.copy_(x0)
+        g1.replay()
+        g2.replay()
+        torch.cuda.synchronize()
+        for a, b, want in zip(out1, out2, want0):
+            assert torch.equal(a, want) and torch.equal(b, want)
+    linear.forget_shared_builds()

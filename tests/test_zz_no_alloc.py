@@ -107,3 +107,44 @@ def test_static_scratch_dot_rejects_what_does_not_fit():
     rc = L.bsi_hip_dot_static_scratch(None, t.data_ptr(), 1, 7, 4, t.data_ptr(), 2, t.data_ptr(), 6, 16, 16, 1.0, 16,
                                       t.data_ptr(), None, _st())
     assert rc == 1
+
+
+def test_static_scratch_dot_replays_from_a_captured_graph(oracle):
+    """After one eager call of the shape class (which looks the array's address up and opts the kernels in to their
+    LDS), the entry point is recorded into a HIP graph and replayed several times with new query planes copied in and
+    eager work between the replays: every replay equals the eager result and the oracle."""
+    from bsipytorch_amd import _lib as hip
+
+    L = hip.lib
+    Q, R, d = 130, 200, 2048
+    W, chunks = d // 64, d // 256
+    cases = [_case(oracle, Q, R, d, seed=s) for s in (1, 2, 3)]
+    kb = cases[0][1]
+    B = _key_operand(L, hip, kb, R, W, 2)
+    Bw = _dev(kb["slice_weights"])
+    A, scales = _dev(cases[0][0]["words"]).clone(), _dev(cases[0][0]["scales"]).clone()
+    out = torch.full((Q, R), float("nan"), dtype=torch.float32, device="cuda")
+    scale_inv = float(np.float32(1e-4))
+
+    def call(stream):
+        hip.check(L.bsi_hip_dot_static_scratch(A.data_ptr(), scales.data_ptr(), chunks, 7, W, B.data_ptr(), 2, Bw.data_ptr(), 6,
+                                               R, Q, scale_inv, R, out.data_ptr(), None, stream), "bsi_hip_dot_static_scratch")
+
+    call(_st())                       # the warm-up call, outside the capture
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        call(torch.cuda.current_stream().cuda_stream)
+    for rep in range(2):
+        for qb, kb_i, _, _ in cases:
+            # every case against the first case's keys
+            _, want = oracle.dot_fixed(qb["words"], qb["scales"], kb["words"], kb["scales"], oracle.scale_inv(2, 2), want_ints=False)
+            A.copy_(_dev(qb["words"]))
+            scales.copy_(_dev(qb["scales"]))
+            out.fill_(float("nan"))
+            g.replay()
+            torch.cuda.synchronize()
+            np.testing.assert_array_equal(out.cpu().numpy(), want)
+            other = torch.randn(256, 256, device="cuda") @ torch.randn(256, 256, device="cuda")  # eager work in between
+            torch.cuda.synchronize()
+            del other
