@@ -347,14 +347,20 @@ int bsi_hip_dot_ewah_query(const uint64_t* comp_words, const int64_t* comp_off, 
  * comp_words + comp_off[q * Sa + s] with comp_len[q * Sa + s] words, is slice s of query q, encoded as
  * bsi_hip_ewah_emit writes it and decoded with the semantics of ewah_decompress_kernel
  * (bsi_cuda_kernels_ewah.cuh:5-33).  The result is that of bsi_hip_dot_bias on the decoded planes, bit for bit.
- * The decode is the call's load stage, never a pass that writes verbatim planes:
- *   - at most 32 rows on tiled16 6-plane keys (the bandwidth-bound regime): inside the dot kernel -- every workgroup
- *     expands its 16 queries' streams into LDS planes, then streams the key planes once;
- *   - otherwise: one launch turns the streams straight into the int8 query image in `workspace`
- *     (bsi_hip_dot_ewah_batch_workspace_bytes), a second one contracts it.  (Every key-tile workgroup of the
- *     compute-bound kernel reads the whole query tile; decoding there would repeat the work once per key tile.)
- * Slices whose stream is the encoder's all-zero form are skipped, not expanded.  B / b_layout / Bw / out /
- * chunk_ints / bias as for bsi_hip_dot and bsi_hip_dot_bias; Sa, Sb in [2, 8]. */
+ * Verbatim planes are never written; where the decode runs depends on the number of rows:
+ *   - at most 32 rows on tiled16 6-plane keys (the bandwidth-bound regime): inside the dot kernel's load stage --
+ *     every workgroup expands its 16 queries' streams into LDS planes, then streams the key planes once;
+ *   - otherwise: a separate launch, ahead of the dot, decodes the streams into the int8 query image in `workspace`
+ *     (bsi_hip_dot_ewah_batch_workspace_bytes: 1 byte per element, more than the 7/8 byte of verbatim planes), and
+ *     the int8-image kernel contracts it.  (Every key-tile workgroup of the compute-bound kernel reads the whole
+ *     query tile; decoding there would repeat the work once per key tile.)
+ * Slices whose stream is the encoder's all-zero form are skipped, not expanded.
+ * What it costs: streams are a STORAGE format here, not a faster route.  With chunk scales only the sign plane of
+ * ReLU'd activations and the top planes of outlier chunks compress (Q512 x D8192 after ReLU: 3.28 MB stored against
+ * 3.74 MB verbatim), and the decode launch adds to the dot: Q512 x R2048 x D8192 25 us from streams against 16.3 us
+ * on the int8 image the fused builder writes (bsi_hip_build_fixed) and 23.7 us from verbatim planes without that
+ * image; 16 rows x R4096 x D4096 9.7 us against 5.7 us.  A caller that has the activations should build the image.
+ * B / b_layout / Bw / out / chunk_ints / bias as for bsi_hip_dot and bsi_hip_dot_bias; Sa, Sb in [2, 8]. */
 size_t bsi_hip_dot_ewah_batch_workspace_bytes(int64_t Q, int W64);
 int bsi_hip_dot_ewah_batch(const uint64_t* comp_words, const int64_t* comp_off, const int32_t* comp_len, int Sa, int W64,
                            const float* A_chunk_scales, int A_scale_stride, const uint64_t* B, int b_layout,
