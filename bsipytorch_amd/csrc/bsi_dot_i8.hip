@@ -622,6 +622,7 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
                 // may hold of an earlier launch: the invalidation is the CU's, so it serves the waves that load
                 // behind the barrier below
                 __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the invalidation has been carried out, not just issued
                 decision = ((old >> 16) != 0 || any != 0) ? kSplitRedo : kSplitCombine;
                 __hip_atomic_store(split_counters + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
                 // running totals behind the tile counters: tiles combined, tiles computed again

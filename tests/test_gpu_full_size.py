@@ -184,6 +184,48 @@ def test_opt13b_shaped_two_layer_decoder_layer_by_layer(ops, oracle, fuse_qkv):
         np.testing.assert_array_equal(y.reshape(-1, y.shape[-1]).cpu().numpy(), want, err_msg=n)
 
 
+def test_opt13b_shaped_full_stack(ops, oracle):
+    """The whole C4 configuration as the benchmark builds it (24 decoder layers, hidden 2048, 32 heads, FFN 8192,
+    vocab 50272, 144 BSI layers, one prefill of 512 tokens): the layers sampled from the first, a middle and the last
+    block equal the oracle's dot of their own input plus their bias bit for bit, the logits are finite, and the
+    forward replayed from a HIP graph gives the eager logits."""
+    from bsipytorch_amd import linear
+    from bsipytorch_amd.benchmarks import benchmark_opt_prefill as bench_model
+
+    model = bench_model.build_model("opt-1.3b", 123, "cuda")
+    with torch.no_grad():
+        for n, p in model.named_parameters():
+            if n.endswith("bias") and "layer_norm" not in n:
+                p.normal_(0.0, 0.02, generator=torch.Generator(device="cuda").manual_seed(len(n)))
+    linear.quantize_model_bsi(model, decimalPlaces=2, compress_threshold=0.5, verbose=False)
+    layers = {n: m for n, m in model.named_modules() if isinstance(m, linear.BSIQuantizedLinear)}
+    assert len(layers) == 144
+    sampled = ["layers.0.self_attn.q_proj", "layers.0.fc2", "layers.11.self_attn.out_proj", "layers.11.fc1",
+               "layers.23.self_attn.v_proj", "layers.23.fc2"]
+    seen = {}
+    hooks = [layers[n].register_forward_hook(
+        lambda mod, args, out, n=n: seen.__setitem__(n, (args[0].detach().clone(), out.detach().clone()))) for n in sampled]
+    ids = torch.randint(0, 50272, (1, 512), generator=torch.Generator().manual_seed(123)).cuda()
+    with torch.no_grad():
+        logits = model(ids).clone()
+    for h in hooks:
+        h.remove()
+    assert logits.shape == (1, 512, 50272) and torch.isfinite(logits).all()
+    for n in sampled:
+        x, y = seen[n]
+        m = layers[n]
+        kb = oracle.build_keys(m.weight_fp32.numpy())
+        want = _oracle_out(oracle, x.reshape(-1, x.shape[-1]).float().cpu().numpy(), kb) + m.bias_fp32.numpy()[None, :]
+        np.testing.assert_array_equal(y.reshape(-1, y.shape[-1]).cpu().numpy(), want, err_msg=n)
+    with torch.no_grad():
+        graphed = linear.GraphedForward(model, ids)
+        for _ in range(2):
+            assert torch.equal(graphed(ids), logits)
+            assert torch.equal(model(ids), logits)   # eager work between the replays
+    del graphed, model
+    torch.cuda.empty_cache()
+
+
 _C5_SHAPES = {"attn": (4096, 4096), "fc1": (16384, 4096), "fc2": (4096, 16384)}
 _c5_cache = {}
 
