@@ -53,7 +53,7 @@ class _Operands:
     """Device operands of one dot on the int8 images, built from the oracle's planes by the library's own layout
     kernels (checked against the oracle elsewhere)."""
 
-    def __init__(self, hip, qb, kb, Q, R, d, Sa=7, Sb=6):
+    def __init__(self, hip, qb, kb, Q, R, d, Sa=7, Sb=6, image_tiled=False):
         L = hip.lib
         self.Q, self.R, self.W, self.Sa, self.Sb = Q, R, (d + 63) // 64, Sa, Sb
         self.chunks = (self.W + 3) // 4
@@ -64,15 +64,20 @@ class _Operands:
         self.Bw = _dev(kb["slice_weights"])
         self.A8 = torch.zeros((Q, self.chunks * 256), dtype=torch.int8, device="cuda")
         hip.check(L.bsi_hip_planes_to_int8(self.A.data_ptr(), Q, Sa, self.W, self.A8.data_ptr(), _st()), "query image")
-        self.K8 = torch.full((R, self.chunks * 256), 77, dtype=torch.int8, device="cuda")
-        hip.check(L.bsi_hip_planes_to_int8(self.B.data_ptr(), R, Sb, self.W, self.K8.data_ptr(), _st()), "key image")
+        self.layout = 3 if image_tiled else 2
+        if image_tiled:   # the image in tiles of 64 rows x half-chunks
+            self.K8 = torch.full((int(L.bsi_hip_int8_tiled_bytes(R, self.W)),), 77, dtype=torch.int8, device="cuda")
+            hip.check(L.bsi_hip_planes_to_int8_tiled(self.B.data_ptr(), R, Sb, self.W, self.K8.data_ptr(), _st()), "key image")
+        else:
+            self.K8 = torch.full((R, self.chunks * 256), 77, dtype=torch.int8, device="cuda")
+            hip.check(L.bsi_hip_planes_to_int8(self.B.data_ptr(), R, Sb, self.W, self.K8.data_ptr(), _st()), "key image")
 
     def dot(self, hip, bias=None, R_total=None):
         L = hip.lib
         R_total = self.R if R_total is None else R_total
         out = torch.full((self.Q, R_total), float("nan"), dtype=torch.float32, device="cuda")
         args = (self.A.data_ptr(), self.A8.data_ptr(), self.scales.data_ptr(), self.stride, self.Sa, self.W,
-                self.K8.data_ptr(), 2, self.Bw.data_ptr(), self.Sb, self.R, self.Q, float(np.float32(1e-4)), R_total)
+                self.K8.data_ptr(), self.layout, self.Bw.data_ptr(), self.Sb, self.R, self.Q, float(np.float32(1e-4)), R_total)
         if bias is None:
             hip.check(L.bsi_hip_dot(*args, out.data_ptr(), None, hip.CORE_MFMA, None, 0, _st()), "dot")
         else:
@@ -127,6 +132,29 @@ def test_split_equals_the_unsplit_launch_and_the_oracle(split, oracle, Q, R, d, 
     got_b = ops.dot(hip, bias=bias, R_total=R + 5)
     np.testing.assert_array_equal(got_b[:, :R], want + bias.cpu().numpy()[None, :])
     assert np.isnan(got_b[:, R:]).all()
+
+
+@pytest.mark.parametrize("Sa,Sb", [(7, 6), (8, 8), (4, 3), (2, 5)])
+@pytest.mark.parametrize("image_tiled", [False, True])
+def test_split_on_other_bit_widths_and_the_tiled_key_image(split, oracle, Sa, Sb, image_tiled):
+    """The exactness limit follows the operands' widths (the accumulators carry 2^(16 - Sa - Sb) times the integers),
+    and a segment's run of chunks is addressed in the tiled key image as in the row-major one."""
+    hip, scratch = split
+    L = hip.lib
+    Q, R, d = 150, 260, 2560
+    rng = np.random.default_rng(Sa * 10 + Sb)
+    x = rng.standard_normal((Q, d)).astype(np.float32)
+    x[:, 7] *= 30.0
+    k = (rng.standard_normal((R, d)) * 0.02).astype(np.float32)
+    qb, kb = oracle.build_queries(x, 2, Sa), oracle.build_keys(k, 2, Sb)
+    _, want = oracle.dot_fixed(qb["words"], qb["scales"], kb["words"], kb["scales"], oracle.scale_inv(2, 2))
+    ops = _Operands(hip, qb, kb, Q, R, d, Sa, Sb, image_tiled)
+    for tile, segments in ((128, 5), (12864, 2), (12864, 10)):
+        hip.check(L.bsi_hip_set_option(hip.OPT_I8_TILE, tile), "set_option")
+        hip.check(L.bsi_hip_set_option(hip.OPT_I8_SPLIT, segments), "set_option")
+        before = _stats(scratch)[0]
+        np.testing.assert_array_equal(ops.dot(hip), want)
+        assert _stats(scratch)[0] - before == _tiles(Q, R, tile) and _stats(scratch)[1] == 0
 
 
 def _rounding_case(oracle, Q, R, chunks, seed, big_queries):
