@@ -403,7 +403,7 @@ __global__ __launch_bounds__((I8Cfg<TM, TN>::kBlock)) void dot_mfma_i8_kernel(
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     // Which tile (and, in a D-split launch, which segment) this workgroup computes.  A D-split launch is a 1-D grid:
     // key tile fastest, then query tile, then segment, so that workgroups which share a key tile and a run of chunks
-    // are neighbours (a grid that gave every XCD one segment of a few key tiles was measured and is slower).
+    // are neighbours (a grid that gave every XCD one segment of a few key tiles was measured and is no faster).
     int bx = static_cast<int>(blockIdx.x), by = static_cast<int>(blockIdx.y), seg = 0, nseg = 1, tiles_x = static_cast<int>(gridDim.x);
     if (kSplit) {
         tiles_x = split_shape & 1023;
