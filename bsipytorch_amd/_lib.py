@@ -89,6 +89,7 @@ PROTOTYPES = {
     "bsi_hip_probe_stream_read": [_vp, _sz, ctypes.POINTER(_d), _vp],
     "bsi_hip_probe_l2_to_lds": [_vp, _sz, _i, ctypes.POINTER(_d), _vp],
     "bsi_hip_timeline_read": [ctypes.POINTER(ctypes.c_ulonglong), _i],
+    "bsi_hip_timeline_read_cycles": [ctypes.POINTER(ctypes.c_ulonglong), _i],
     "bsi_hip_version": [],
     "bsi_hip_last_error": [],
 }

@@ -34,8 +34,11 @@ def timeline(Q: int, R: int, D: int, iters: int = 50, warmup: int = 10) -> dict:
     buf = (ctypes.c_ulonglong * (wgs * 8))()
     _lib.check(_lib.lib.bsi_hip_timeline_read(buf, wgs), "bsi_hip_timeline_read")  # clears what earlier launches left
     res = micro.run(Q, R, D, 2, 0.5, warmup, iters, 123, "mfma", outliers=(D == 2048))
+    cbuf = (ctypes.c_ulonglong * (wgs * 8))()
+    _lib.check(_lib.lib.bsi_hip_timeline_read_cycles(cbuf, wgs), "bsi_hip_timeline_read_cycles")  # before the read that clears
     _lib.check(_lib.lib.bsi_hip_timeline_read(buf, wgs), "bsi_hip_timeline_read")
     t = np.frombuffer(buf, dtype=np.uint64).reshape(wgs, 8).astype(np.int64)
+    cyc = np.frombuffer(cbuf, dtype=np.uint64).reshape(wgs, 8).astype(np.int64)[t[:, 0] > 0]
     live = t[t[:, 0] > 0]  # the workgroups of this shape's grid
     base = min(live[:, 0].min(), live[:, 4].min())
     us = (live - base) / 100.0
@@ -54,6 +57,12 @@ def timeline(Q: int, R: int, D: int, iters: int = 50, warmup: int = 10) -> dict:
         "chunk_loop_per_half_chunk": round(loop / halves, 3),
         "output_stores": round(float(np.median(us[:, 3] - us[:, 2])), 2),
     }
+    # the shader clock's own counter over the chunk loop: cycles per half-chunk (512 is what the MFMAs of a 128 x 128
+    # tile need, and what 32 KiB take at 64 bytes per clock), and the clock the GPU held there
+    loop_cycles = (cyc[:, 2] - cyc[:, 1]).astype(np.float64)
+    loop_ticks = (live[:, 2] - live[:, 1]).astype(np.float64)
+    out["per_workgroup_median_us"]["chunk_loop_cycles_per_half_chunk"] = round(float(np.median(loop_cycles)) / halves, 1)
+    out["per_workgroup_median_us"]["shader_clock_GHz_in_the_loop"] = round(float(np.median(loop_cycles / (loop_ticks / 100.0))) / 1e3, 3)
     out["in_kernel_us"] = round(float(us[:, 3].max()), 2)
     out["between_launches_us"] = round(out["us_per_launch_by_events"] - out["in_kernel_us"], 2)
     return out

@@ -105,10 +105,14 @@ enum TimelineStamp {
 };
 #ifdef BSI_TIMELINE
 __device__ unsigned long long g_timeline[kTimelineWorkgroups * 8];
+__device__ unsigned long long g_timeline_cycles[kTimelineWorkgroups * 8];  // the shader-clock counter at the same points
 #define BSI_STAMP(slot)                                                                    \
     {                                                                                      \
         const unsigned wg_ = (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x; \
-        if (lane == 0 && wg_ < kTimelineWorkgroups) g_timeline[wg_ * 8 + (slot)] = wall_clock64(); \
+        if (lane == 0 && wg_ < kTimelineWorkgroups) {                                      \
+            g_timeline[wg_ * 8 + (slot)] = wall_clock64();                                 \
+            g_timeline_cycles[wg_ * 8 + (slot)] = clock64();                               \
+        }                                                                                  \
     }
 #else
 #define BSI_STAMP(slot)
@@ -1416,6 +1420,18 @@ extern "C" int bsi_hip_timeline_read(unsigned long long* stamps_host, int workgr
     void* dev = nullptr;  // cleared, so that the next read shows which workgroups have run since
     BSI_HIP_CHECK(hipGetSymbolAddress(&dev, HIP_SYMBOL(g_timeline)));
     BSI_HIP_CHECK(hipMemset(dev, 0, sizeof(unsigned long long) * 8 * kTimelineWorkgroups));
+    return BSI_OK;
+#else
+    return fail(BSI_ERR_INVALID, "this library was built without the timeline stamps (make TIMELINE=1 builds one with)");
+#endif
+}
+
+extern "C" int bsi_hip_timeline_read_cycles(unsigned long long* cycles_host, int workgroups) {
+    BSI_REQUIRE(cycles_host && workgroups >= 1 && workgroups <= kTimelineWorkgroups, "workgroups must be 1 .. %d",
+                kTimelineWorkgroups);
+#ifdef BSI_TIMELINE
+    BSI_HIP_CHECK(hipDeviceSynchronize());
+    BSI_HIP_CHECK(hipMemcpyFromSymbol(cycles_host, HIP_SYMBOL(g_timeline_cycles), sizeof(unsigned long long) * 8 * workgroups));
     return BSI_OK;
 #else
     return fail(BSI_ERR_INVALID, "this library was built without the timeline stamps (make TIMELINE=1 builds one with)");

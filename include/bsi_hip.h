@@ -437,6 +437,11 @@ int bsi_hip_probe_stream_read(const void* buf_device, size_t bytes, double* byte
  * issued; a workgroup that has not run since the last read gives zeros (the read clears the stamps).  Synchronises the
  * device.  No counterpart in the reference: a measuring aid. */
 int bsi_hip_timeline_read(unsigned long long* stamps_host, int workgroups);
+/* The shader-clock counter (clock64: cycles of the clock the waves run on) read at the same points by the same launch,
+ * same layout; not cleared (bsi_hip_timeline_read clears the wall-clock stamps, which tell which workgroups ran).  The
+ * ratio of a cycle difference to a wall-clock difference is the clock the GPU held between two points.  Same builds,
+ * same error from the ordinary one. */
+int bsi_hip_timeline_read_cycles(unsigned long long* cycles_host, int workgroups);
 /* What the int8-image kernel's operand path delivers: every CU streams an L2-resident part of buf_device (at least
  * 2 MiB are read) into LDS with LDS-direct 16-byte buffer loads, 96 KiB in flight per CU, all CUs at once; the result
  * is the aggregate rate over all CUs in bytes per second.  loader_pattern = 0: eight issuing waves per CU, contiguous
