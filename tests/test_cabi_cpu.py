@@ -211,8 +211,31 @@ def test_set_option_validates_on_host():
     assert _lib.lib.bsi_hip_set_option(_lib.OPT_BUILD_ITEMS, 4) == 0
     assert _lib.lib.bsi_hip_set_option(_lib.OPT_BUILD_ITEMS, 3) == 1
     assert _lib.lib.bsi_hip_set_option(_lib.OPT_BUILD_ITEMS, 0) == 0
+    assert _lib.lib.bsi_hip_set_option(_lib.OPT_I8_SPLIT, 6) == 0
+    assert _lib.lib.bsi_hip_set_option(_lib.OPT_I8_SPLIT, 65) == 1
+    assert _lib.lib.bsi_hip_set_option(_lib.OPT_I8_SPLIT, 0) == 0
     assert _lib.lib.bsi_hip_set_option(999, 1) == 1
     assert b"unknown option" in _lib.lib.bsi_hip_last_error()
+
+
+def test_split_scratch_host_side():
+    """What the D-split's host side decides without touching a device: the scratch size that serves every choice, the
+    refusal of a misaligned or too small region, detaching, and the plan of a thread with no region attached (the
+    unsplit tile the launcher would take)."""
+    import ctypes
+
+    from bsipytorch_amd import _lib
+
+    L = _lib.lib
+    assert L.bsi_hip_dot_split_scratch_bytes() == 4096 + 256 * 128 * 128 * 4
+    assert L.bsi_hip_dot_attach_split_scratch(None, 0) == 0                       # detaching is always fine
+    assert L.bsi_hip_dot_attach_split_scratch(0x1008, 1 << 20) == 1 and b"aligned" in L.bsi_hip_last_error()
+    assert L.bsi_hip_dot_attach_split_scratch(0x1000, 4096) == 1 and b"counters" in L.bsi_hip_last_error()
+    tile, seg = ctypes.c_int(0), ctypes.c_int(0)
+    for (R, Q, W), want in (((2048, 512, 128), 64), ((8192, 512, 32), 128), ((4096, 512, 64), 12864), ((4096, 128, 256), 6432)):
+        assert L.bsi_hip_dot_split_plan(R, Q, W, ctypes.byref(tile), ctypes.byref(seg)) == 0
+        assert (tile.value, seg.value) == (want, 1)
+    assert L.bsi_hip_dot_split_plan(0, 512, 32, ctypes.byref(tile), ctypes.byref(seg)) == 1
 
 
 def test_load_keyset_refuses_foreign_files_before_touching_the_device(tmp_path):
