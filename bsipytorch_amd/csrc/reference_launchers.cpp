@@ -6,6 +6,10 @@
 // name and argument list (cudaStream_t is hipStream_t under ROCm's torch headers) and forwards to the C ABI of
 // include/bsi_hip.h.  Plain host code: no torch, no kernels.
 //
+// One stream per device at a time, as the reference uses them: the dot's int8 query operands go to the library's
+// per-device static scratch (or a per-device buffer of this module), and the query image remembered for registered
+// keysets is per device too, so launchers running on two streams of one device at the same time would race on them.
+//
 // The launchers return void, as in the reference, so a failure is kept for the caller to ask about:
 // bsi_launchers_last_status() / bsi_launchers_last_error() report the calling thread's last failing launcher
 // (BSI_OK / "" when none failed since the last bsi_launchers_clear_status()), and the first failure of a process
