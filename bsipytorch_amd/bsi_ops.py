@@ -669,7 +669,7 @@ def _dot_ewah_batch(qb: "PrebuiltBSIQueryBatchHybridCUDA", keys: "PrebuiltBSIKey
     ws_bytes = int(lib.bsi_hip_dot_ewah_batch_workspace_bytes(Q, W))
     ws = _get_workspace(ws_bytes, dev)
     if Q >= _SPLIT_MIN_Q and chunk_ints is None:
-        attach_split_scratch(dev)
+        _attach_split_scratch_for(dev, Q, R, W)
     prof = f["profile"]
     if prof:
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -962,6 +962,25 @@ def attach_split_scratch(dev=None) -> bool:
     return buf is not None
 
 
+_split_shapes: dict = {}  # (device index, Q, R, W) -> whether the launcher splits a dot of that shape
+
+
+def _attach_split_scratch_for(dev, Q: int, R: int, W: int) -> None:
+    """attach_split_scratch for the shapes the launcher would split, nothing for the others (a model's layers of a
+    few hundred rows against thousands of keys never split: asking once per shape keeps the stream and capture
+    look-ups out of every other forward).  The library's choice depends on the shape and the region's size only."""
+    key = (dev.index, Q, R, W)
+    use = _split_shapes.get(key)
+    if use is None:
+        if not attach_split_scratch(dev):
+            return  # no region yet (a capture before any eager call): ask again next time
+        tile, segments = ctypes.c_int(0), ctypes.c_int(0)
+        check(lib.bsi_hip_dot_split_plan(R, Q, W, ctypes.byref(tile), ctypes.byref(segments)), "bsi_hip_dot_split_plan")
+        _split_shapes[key] = segments.value > 1
+    elif use:
+        attach_split_scratch(dev)
+
+
 def _scale_inv(dec_q: int, dec_k: int) -> float:
     # bsi_cuda.cpp:709-711: (float)(1.0 / 10^(dq + dk)); the C ABI takes it as float
     total = dec_q + dec_k
@@ -1007,7 +1026,7 @@ def _dot(words, ints8, scales, scale_stride, Sa, W, keys: PrebuiltBSIKeysCUDA, Q
         e0.record()
     kptr, klayout = key_operand(keys, Q, Sa, core)
     if Q >= _SPLIT_MIN_Q and chunk_ints is None:
-        attach_split_scratch(dev)
+        _attach_split_scratch_for(dev, Q, R, W)
     if warm_keys is not None and chunk_ints is None:
         # the kernel also touches what the next layer's dot will read, so that it is cache-resident by then
         wptr, wbytes = _warm_region(warm_keys, Q, Sa, core)
@@ -1248,7 +1267,7 @@ def linear_cuda(x2d: torch.Tensor, keyset_cuda_cap, decimal_places: int, bias=No
     core = f["core"]
     kptr, klayout = key_operand(keys, Q, bits, core)
     if Q >= _SPLIT_MIN_Q:
-        attach_split_scratch(x2d.device)
+        _attach_split_scratch_for(x2d.device, Q, R, (d + 63) // 64)
     wptr, wbytes = _warm_region(_capsule(warm_keys, PrebuiltBSIKeysCUDA, "Invalid CUDA keys capsule") if warm_keys is not None
                                 else None, Q, bits, core)
     check(lib.bsi_hip_linear(x2d.data_ptr(), _dtype_code(x2d), Q, d, int(decimal_places), bits, rebuild, wsptr, ws["bytes"],
