@@ -57,33 +57,43 @@ bool mask_is_low_bits(unsigned long long value_mask, int slices) {
 struct Workspace {
     void* ptr = nullptr;
     size_t bytes = 0;
+    bool recorded = false;  // a launch recorded into a graph holds this address: the buffer is never freed
 };
 std::mutex g_ws_mutex;
 Workspace g_ws[64];
 
-// Growing the buffer synchronises the device and frees memory, which a stream that is being captured into a graph
-// must not see: while `stream` is capturing, a need beyond the present buffer is refused (run the call once eagerly
-// first, and the buffer is there).
+// A buffer of this module that has to grow: the old one is freed once the device is idle (launches in flight may
+// still read it) -- unless a graph has recorded a launch on it, which may be replayed at any later time: that buffer
+// is left allocated for the rest of the process.
+bool release_for_growth(void* ptr, bool recorded) {
+    if (ptr == nullptr || recorded) return true;
+    if (hipDeviceSynchronize() != hipSuccess) return false;
+    (void)hipFree(ptr);
+    return true;
+}
+
+// Growing the buffer synchronises the device and allocates memory, which a stream that is being captured into a
+// graph must not see: while `stream` is capturing, a need beyond the present buffer is refused (run the call once
+// eagerly first, and the buffer is there).
 int workspace_for(size_t need, hipStream_t stream, void** ptr, size_t* bytes) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return BSI_ERR_HIP;
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capturing) != hipSuccess) return BSI_ERR_HIP;
     std::lock_guard<std::mutex> lock(g_ws_mutex);
     Workspace& w = g_ws[dev];
     if (w.bytes < need) {
-        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-        if (hipStreamIsCapturing(stream, &capturing) != hipSuccess) return BSI_ERR_HIP;
         if (capturing != hipStreamCaptureStatusNone) return BSI_ERR_UNSUPPORTED;
-        // the old buffer may still be read by launches in flight: free it only once the device is idle
-        if (w.ptr != nullptr) {
-            if (hipDeviceSynchronize() != hipSuccess) return BSI_ERR_HIP;
-            (void)hipFree(w.ptr);
-            w.ptr = nullptr;
-            w.bytes = 0;
-        }
+        if (!release_for_growth(w.ptr, w.recorded)) return BSI_ERR_HIP;
+        w = Workspace{};
         const size_t size = (need + (size_t{1} << 20) - 1) & ~((size_t{1} << 20) - 1);
-        if (hipMalloc(&w.ptr, size) != hipSuccess) return BSI_ERR_HIP;
+        if (hipMalloc(&w.ptr, size) != hipSuccess) {
+            w = Workspace{};
+            return BSI_ERR_HIP;
+        }
         w.bytes = size;
     }
+    if (capturing != hipStreamCaptureStatusNone) w.recorded = true;
     *ptr = w.ptr;
     *bytes = w.bytes;
     return BSI_OK;
@@ -112,6 +122,7 @@ struct QueryImage {  // per device: the int8 image of the query planes packed la
     int Sa = 0, W = 0;
     int8_t* image = nullptr;
     size_t bytes = 0;
+    bool recorded = false;  // as for Workspace
 };
 QueryImage g_query_image[64];
 
@@ -164,7 +175,8 @@ int bsi_launchers_register_keys(const unsigned long long* B, int R, int Sb, int 
 }
 
 // Forgets the keyset registered for these planes (when the reference's keyset capsule is destroyed).  The image is
-// freed, which waits for work in flight on the device, so: not while a stream is being captured.
+// freed, which waits for work in flight on the device, so: not while a stream is being captured, and not while a
+// graph that has recorded a dot against this keyset may still be replayed (as for the keyset's own tensors).
 int bsi_launchers_forget_keys(const unsigned long long* B) {
     int8_t* image = nullptr;
     {
@@ -377,19 +389,23 @@ void launch_quantize_shift_pack_chunk_batch(const void* input, int input_dtype, 
     }
     if (!any_keys || Q <= 32) return;
     const size_t bytes = static_cast<size_t>(Q) * static_cast<size_t>((words_per_slice + 3) / 4) * 256;
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capturing) != hipSuccess) return;
     if (qi.bytes < bytes) {
-        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-        if (hipStreamIsCapturing(stream, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) return;
-        if (qi.image != nullptr) {
-            if (hipDeviceSynchronize() != hipSuccess) return;
-            (void)hipFree(qi.image);
-            qi.image = nullptr;
-            qi.bytes = 0;
-        }
+        if (capturing != hipStreamCaptureStatusNone) return;
+        const bool released = release_for_growth(qi.image, qi.recorded);
+        qi.image = nullptr;
+        qi.bytes = 0;
+        qi.recorded = false;
+        if (!released) return;
         const size_t size = (bytes + (size_t{1} << 20) - 1) & ~((size_t{1} << 20) - 1);
-        if (hipMalloc(reinterpret_cast<void**>(&qi.image), size) != hipSuccess) return;
+        if (hipMalloc(reinterpret_cast<void**>(&qi.image), size) != hipSuccess) {
+            qi.image = nullptr;
+            return;
+        }
         qi.bytes = size;
     }
+    if (capturing != hipStreamCaptureStatusNone) qi.recorded = true;
     if (bsi_hip_planes_to_int8(reinterpret_cast<const uint64_t*>(out), Q, slices, words_per_slice, qi.image, stream) != BSI_OK) return;
     qi.planes = out;
     qi.Q = Q;

@@ -223,3 +223,71 @@ def test_registered_keys_take_the_int8_image_route(launchers, oracle):
     assert L.bsi_launchers_forget_keys(B.data_ptr()) == 0
     np.testing.assert_array_equal(build_and_dot(xs[1]), want(xs[1])[0])
     assert L.bsi_launchers_forget_keys(B.data_ptr()) == 0   # forgetting twice is not an error
+
+
+def test_a_recorded_query_image_survives_a_larger_batch(launchers, oracle):
+    """The packer and the dot of a registered keyset recorded into a HIP graph hold the address of the module's query
+    image; a later, larger batch makes the module allocate a bigger image, and the recorded one must stay valid: the
+    graph, replayed on new inputs afterwards (with eager work of the larger batch in between), still gives the oracle's bits."""
+    L = launchers
+    L.bsi_launchers_register_keys.argtypes, L.bsi_launchers_register_keys.restype = [vp, i32, i32, i32, vp], i32
+    L.bsi_launchers_forget_keys.argtypes, L.bsi_launchers_forget_keys.restype = [vp], i32
+    L.bsi_launchers_clear_status()
+    R, d = 192, 1024
+    W, chunks = d // 64, d // 256
+    rng = np.random.default_rng(5150)
+    k = (rng.standard_normal((R, d)) * 0.02).astype(np.float32)
+    kb = oracle.build_keys(k)
+    B = torch.from_numpy(kb["words"].view(np.int64)).cuda()
+    Bw = torch.from_numpy(kb["slice_weights"]).cuda()
+    assert L.bsi_launchers_register_keys(B.data_ptr(), R, 6, W, _st()) == 0
+    scale_inv = float(np.float32(1.0 / 10.0 ** 4))
+
+    class Batch:
+        def __init__(self, Q):
+            self.Q = Q
+            self.x = torch.zeros((Q, d), dtype=torch.float32, device="cuda")
+            self.Aw = torch.tensor([1, 2, 4, 8, 16, 32, -64], dtype=torch.float32, device="cuda").repeat(Q, 1).contiguous()
+            self.A = torch.empty((Q, 7, W), dtype=torch.int64, device="cuda")
+            self.qshift = torch.empty((Q, chunks), dtype=torch.int32, device="cuda")
+            self.qscale = torch.empty((Q, chunks), dtype=torch.float32, device="cuda")
+            self.out = torch.zeros((Q, R), dtype=torch.float32, device="cuda")
+
+        def launch(self):
+            st, Q = _st(), self.Q
+            L.launch_compute_chunk_shift_scale_from_input(self.x.data_ptr(), 0, Q, d, chunks, 100.0, 7, 0.0,
+                                                          self.qshift.data_ptr(), self.qscale.data_ptr(), st)
+            L.launch_quantize_shift_pack_chunk_batch(self.x.data_ptr(), 0, Q, d, chunks, 7, W, 0x7F, 100.0, 7,
+                                                     self.qshift.data_ptr(), self.A.data_ptr(), st)
+            L.launch_popcount_weighted_keys_literal_fused_multiq(self.A.data_ptr(), self.Aw.data_ptr(), self.qscale.data_ptr(),
+                                                                 chunks, 7, W, B.data_ptr(), Bw.data_ptr(), 6, R, Q, 8, 4, None,
+                                                                 None, scale_inv, R, self.out.data_ptr(), st)
+
+    def want(x):
+        qb = oracle.build_queries(x)
+        return oracle.dot_fixed(qb["words"], qb["scales"], kb["words"], kb["scales"], oracle.scale_inv(2, 2), want_ints=False)[1]
+
+    small, large = Batch(96), Batch(384)
+    xs = [rng.standard_normal((small.Q, d)).astype(np.float32) for _ in range(3)]
+    small.x.copy_(torch.from_numpy(xs[0]))
+    small.launch()                      # eager first: the image buffer of 96 rows exists
+    torch.cuda.synchronize()
+    _ok(L)
+    np.testing.assert_array_equal(small.out.cpu().numpy(), want(xs[0]))
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        small.launch()
+    _ok(L)
+    xl = rng.standard_normal((large.Q, d)).astype(np.float32)
+    for x in xs[1:]:
+        large.x.copy_(torch.from_numpy(xl))
+        large.launch()                  # the first of these outgrows the recorded image
+        torch.cuda.synchronize()
+        _ok(L)
+        np.testing.assert_array_equal(large.out.cpu().numpy(), want(xl))
+        small.x.copy_(torch.from_numpy(x))
+        small.out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(small.out.cpu().numpy(), want(x))
+    assert L.bsi_launchers_forget_keys(B.data_ptr()) == 0
